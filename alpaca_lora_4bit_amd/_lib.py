@@ -1,0 +1,52 @@
+"""ctypes binding of libq4gptq.so (C ABI declared in include/q4_gptq.h)."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libq4gptq.so")
+ABI_VERSION = 1
+
+_lib = None
+
+# name -> (restype, argtypes); must list every symbol of include/q4_gptq.h
+_vp, _i, _sz = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+SIGNATURES = {
+    "q4_abi_version": (_i, []),
+    "q4_error_string": (ctypes.c_char_p, [_i]),
+    "q4_dequant_f16": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp]),
+    "q4_gemv_workspace_bytes": (_sz, [_i, _i, _i]),
+    "q4_gemv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "q4_gemm_fwd_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
+    "q4_gemm_bwd_dx_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _i, _i, _i, _i, _vp]),
+}
+
+
+class Q4Error(RuntimeError):
+    pass
+
+
+def lib() -> ctypes.CDLL:
+    """Load the HIP library; raise ImportError (never fall back) when it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} not found: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(hipcc --offload-arch=gfx950). There is no CPU fallback for the 4-bit kernels.")
+    L = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(L, name)
+        fn.restype = res
+        fn.argtypes = args
+    if L.q4_abi_version() != ABI_VERSION:
+        raise ImportError(f"{LIB_PATH}: ABI version {L.q4_abi_version()} != expected {ABI_VERSION}; rebuild")
+    _lib = L
+    return L
+
+
+def check(code: int, what: str) -> None:
+    if code != 0:
+        raise Q4Error(f"{what}: {lib().q4_error_string(code).decode()} (code {code})")

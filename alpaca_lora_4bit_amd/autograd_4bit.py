@@ -1,0 +1,267 @@
+"""Quant-linear module and autograd Functions with the interface of the reference's
+src/alpaca_lora_4bit/autograd_4bit.py:13-244, running on the gfx950 kernels.
+
+Kept exactly: class names (callers match on `str(type(m))`, finetune.py:101), the 7-argument
+`AutogradMatmul4bit.apply(x, qweight, scales, zeros, g_idx, bits, maxq)` with a 7-tuple
+backward, the rebindable module globals `AutogradMatmul4bit` / `backend`, buffer names, shapes
+and dtypes of `Autograd4bitQuantLinear` (they are the checkpoint format), `switch_backend_to`,
+`matmul4bit_with_backend`, `make_quant_for_4bit_autograd`, `model_to_half/float`, `find_layers`.
+
+There is ONE backend and it answers to the name 'cuda' (the torch device string on ROCm, and
+what finetune.py:37-40 asks for).  'triton' raises ValueError like an absent Triton does in
+the reference (autograd_4bit.py:144-145).
+"""
+import logging
+import math
+
+import torch
+import torch.nn as nn
+from torch.amp import custom_bwd, custom_fwd
+
+gptq_backend_loaded = False
+triton_backend_loaded = False
+
+
+class AutogradMatmul4bitNotImplemented(torch.autograd.Function):
+    """Placeholder bound when the HIP library is missing (autograd_4bit.py:17-26)."""
+
+    @staticmethod
+    @custom_fwd(device_type='cuda', cast_inputs=torch.float16)
+    def forward(ctx, x, qweight, scales, zeros, g_idx, bits, maxq):
+        raise NotImplementedError()
+
+    @staticmethod
+    @custom_bwd(device_type='cuda')
+    def backward(ctx, grad_output):
+        raise NotImplementedError()
+
+
+try:
+    from . import matmul_utils_4bit as mm4b
+    from . import quant_hip
+
+    class AutogradMatmul4bitCuda(torch.autograd.Function):
+        """y = x @ W with W packed; backward returns dy @ W^T and None for the frozen tensors
+        (autograd_4bit.py:32-54).  Only the packed tensors are saved, never a dense W."""
+
+        @staticmethod
+        @custom_fwd(device_type='cuda', cast_inputs=torch.float16)
+        def forward(ctx, x, qweight, scales, zeros, g_idx, bits, maxq):
+            if g_idx is None or zeros.dtype != torch.int32:
+                mm4b._v1_unsupported()
+            ctx.save_for_backward(qweight, scales, zeros, g_idx)
+            rows = x.numel() // x.shape[-1]
+            if 1 <= rows <= quant_hip.MAX_GEMV_ROWS:
+                return mm4b._matmul4bit_v2(x, qweight, scales, zeros, g_idx)
+            return mm4b._matmul4bit_v2_recons(x, qweight, scales, zeros, g_idx)
+
+        @staticmethod
+        @custom_bwd(device_type='cuda')
+        def backward(ctx, grad_output):
+            qweight, scales, zeros, g_idx = ctx.saved_tensors
+            grad = None
+            if ctx.needs_input_grad[0]:
+                grad = mm4b._matmul4bit_v2_recons(grad_output, qweight, scales, zeros, g_idx, transpose=True)
+            return grad, None, None, None, None, None, None
+
+    class AutogradMatmul2bitCuda(torch.autograd.Function):
+        """2-bit checkpoints are outside what is built for gfx950."""
+
+        @staticmethod
+        def forward(ctx, x, qweight, scales, zeros, g_idx, bits, maxq):
+            mm4b._v1_unsupported()
+
+        @staticmethod
+        def backward(ctx, grad_output):
+            mm4b._v1_unsupported()
+
+    gptq_backend_loaded = True
+except ImportError:
+    print('libq4gptq.so not found. Build it with __graft_entry__.build() (hipcc, gfx950).')
+
+
+def is_triton_backend_available():
+    return False
+
+
+def is_gptq_backend_available():
+    return 'AutogradMatmul4bitCuda' in globals()
+
+
+AutogradMatmul4bit = AutogradMatmul4bitNotImplemented
+AutogradMatmul2bit = AutogradMatmul4bitNotImplemented
+backend = None
+if is_gptq_backend_available():
+    AutogradMatmul4bit = AutogradMatmul4bitCuda
+    AutogradMatmul2bit = AutogradMatmul2bitCuda
+    backend = 'cuda'
+else:
+    logging.warning("The gfx950 4-bit backend is not available.")
+
+
+def switch_backend_to(to_backend):
+    global AutogradMatmul4bit
+    global backend
+    if to_backend == 'cuda':
+        if not is_gptq_backend_available():
+            raise ValueError('libq4gptq.so not found. Build it with __graft_entry__.build().')
+        AutogradMatmul4bit = AutogradMatmul4bitCuda
+        backend = 'cuda'
+        print('Using the gfx950 HIP implementation (backend name: cuda).')
+    elif to_backend == 'triton':
+        raise ValueError('Triton not found. This build has a single HIP backend; use "cuda".')
+    else:
+        raise ValueError('Backend not supported.')
+
+
+def matmul4bit_with_backend(x, qweight, scales, qzeros, g_idx, bits, maxq, groupsize=None):
+    if backend == 'cuda':
+        return mm4b.matmul4bit(x, qweight, scales, qzeros, g_idx, groupsize)
+    raise ValueError('Backend not supported.')
+
+
+class Autograd4bitQuantLinear(nn.Module):
+    """GPTQ 4-bit linear layer; buffers as registered at autograd_4bit.py:166-189."""
+
+    def __init__(self, in_features, out_features, groupsize=-1, is_v1_model=False, bits=4):
+        super().__init__()
+        self.in_features = in_features
+        self.out_features = out_features
+        self.bits = bits
+        self.maxq = 2 ** self.bits - 1
+        groupsize = groupsize if groupsize != -1 else in_features
+        self.groupsize = groupsize
+        self.is_v1_model = is_v1_model
+        self.disable_bias = False
+        n_groups = math.ceil(in_features / groupsize)
+        if is_v1_model:
+            self.register_buffer('zeros', torch.empty((out_features, 1)))
+            self.register_buffer('scales', torch.empty((out_features, 1)))
+            self.g_idx = None
+        else:
+            self.register_buffer('qzeros', torch.empty((n_groups, out_features * bits // 32), dtype=torch.int32))
+            self.register_buffer('scales', torch.empty((n_groups, out_features)))
+            self.register_buffer('g_idx', (torch.arange(in_features, dtype=torch.int64) // groupsize).to(torch.int32))
+        self.register_buffer('bias', torch.zeros(out_features))
+        self.register_buffer('qweight', torch.empty((in_features * bits // 32, out_features), dtype=torch.int32))
+
+    def forward(self, x):
+        zeros = self.zeros if self.is_v1_model else self.qzeros
+        if self.bits == 4:
+            if torch.is_grad_enabled():
+                out = AutogradMatmul4bit.apply(x, self.qweight, self.scales, zeros, self.g_idx, self.bits, self.maxq)
+            else:
+                out = matmul4bit_with_backend(x, self.qweight, self.scales, zeros, self.g_idx, self.bits, self.maxq,
+                                              self.groupsize)
+        elif self.bits == 2:
+            out = AutogradMatmul2bit.apply(x, self.qweight, self.scales, self.qzeros, self.g_idx, self.bits, self.maxq)
+        else:
+            raise ValueError('Unsupported bitwidth.')
+        if not self.disable_bias:
+            out += self.bias
+        return out
+
+
+def make_quant_for_4bit_autograd(module, names, name='', groupsize=-1, is_v1_model=False, bits=4):
+    """Replace every attribute of `module` (recursively) whose dotted path is in `names` by an
+    empty Autograd4bitQuantLinear of the same in/out features (autograd_4bit.py:211-222)."""
+    if isinstance(module, Autograd4bitQuantLinear):
+        return
+    for child_name, child in list(module.named_children()):
+        path = f'{name}.{child_name}' if name else child_name
+        if path in names:
+            setattr(module, child_name, Autograd4bitQuantLinear(child.in_features, child.out_features,
+                                                                groupsize=groupsize, is_v1_model=is_v1_model, bits=bits))
+        else:
+            make_quant_for_4bit_autograd(child, names, path, groupsize=groupsize, is_v1_model=is_v1_model, bits=bits)
+
+
+def _cast_quant_buffers(model, dtype):
+    for _, m in model.named_modules():
+        if isinstance(m, Autograd4bitQuantLinear):
+            if m.is_v1_model:
+                m.zeros = m.zeros.to(dtype)
+            m.scales = m.scales.to(dtype)
+            m.bias = m.bias.to(dtype)
+
+
+def model_to_half(model):
+    """autograd_4bit.py:225-233."""
+    model.half()
+    _cast_quant_buffers(model, torch.float16)
+    print('Converted as Half.')
+
+
+def model_to_float(model):
+    """autograd_4bit.py:236-244.  Note: the HIP kernels take fp16 scales; fp32 scales are
+    rounded to fp16 on every call, so prefer model_to_half."""
+    model.float()
+    _cast_quant_buffers(model, torch.float32)
+    print('Converted as Float.')
+
+
+def find_layers(module, layers=(nn.Conv2d, nn.Linear), name=''):
+    """{dotted name: module} of every leaf whose exact type is in `layers` (autograd_4bit.py:247-255)."""
+    if type(module) in layers:
+        return {name: module}
+    res = {}
+    for child_name, child in module.named_children():
+        res.update(find_layers(child, layers=layers, name=f'{name}.{child_name}' if name else child_name))
+    return res
+
+
+class AutogradMatmul4bitLora(torch.autograd.Function):
+    """Fused  y = x @ W (+ bias) + scaling * (x @ A^T) @ B^T  for one LoRA adapter.
+
+    No counterpart in the reference as a single op: it is Autograd4bitQuantLinear.forward
+    (autograd_4bit.py:192-208) followed by the adapter lines of Linear4bitLt.forward
+    (models.py:58-66) and, in backward, AutogradMatmul4bitCuda.backward (autograd_4bit.py:45-54)
+    plus torch autograd over the two adapter Linears.  Here the rank-r products ride in the
+    main GEMM as one extra reduction step, forward and backward:
+        fwd   xa  = scaling * x @ A^T   [M, r]   then  y  = [x | xa]  @ [W ; B^T]
+        bwd   dyb = scaling * dy @ B    [M, r]   then  dx = [dy | dyb] @ [W^T ; A]
+              dA  = dyb^T @ x   [r, K]            dB = dy^T @ xa   [N, r]
+    A: lora_A.weight [r, K], B: lora_B.weight [N, r] (any float dtype; products run in fp16
+    with fp32 accumulation, like the reference under autocast)."""
+
+    @staticmethod
+    @custom_fwd(device_type='cuda', cast_inputs=torch.float16)
+    def forward(ctx, x, qweight, scales, zeros, g_idx, bias, lora_a, lora_b, scaling, groupsize):
+        K, N = qweight.shape[0] * 8, qweight.shape[1]
+        x2 = x.reshape(-1, K)
+        if x2.dtype != torch.float16:
+            x2 = x2.half()
+        a16 = lora_a.to(torch.float16)
+        b16 = lora_b.to(torch.float16)
+        xa = torch.matmul(x2, a16.t())
+        if scaling != 1.0:
+            xa = xa * scaling
+        y = quant_hip.gemm_fwd(x2, qweight, zeros, scales, g_idx, groupsize, bias=bias,
+                               xa=xa, lora_bt=b16.t().contiguous())
+        ctx.save_for_backward(x2, xa, qweight, scales, zeros, g_idx, a16, b16)
+        ctx.scaling = scaling
+        ctx.groupsize = groupsize
+        ctx.ab_dtypes = (lora_a.dtype, lora_b.dtype)
+        return y.reshape(x.shape[:-1] + (N,))
+
+    @staticmethod
+    @custom_bwd(device_type='cuda')
+    def backward(ctx, grad_output):
+        x2, xa, qweight, scales, zeros, g_idx, a16, b16 = ctx.saved_tensors
+        N = qweight.shape[1]
+        dy = grad_output.reshape(-1, N)
+        if dy.dtype != torch.float16:
+            dy = dy.half()
+        dy = dy.contiguous()
+        dyb = torch.matmul(dy, b16)
+        if ctx.scaling != 1.0:
+            dyb = dyb * ctx.scaling
+        dx = da = db = None
+        if ctx.needs_input_grad[0]:
+            dx = quant_hip.gemm_bwd_dx(dy, qweight, zeros, scales, g_idx, ctx.groupsize, dyb=dyb, lora_a=a16)
+            dx = dx.reshape(grad_output.shape[:-1] + (dx.shape[-1],))
+        if ctx.needs_input_grad[6]:
+            da = torch.matmul(dyb.t(), x2).to(ctx.ab_dtypes[0])
+        if ctx.needs_input_grad[7]:
+            db = torch.matmul(dy.t(), xa).to(ctx.ab_dtypes[1])
+        return dx, None, None, None, None, None, da, db, None, None

@@ -1,0 +1,98 @@
+// C ABI of libq4gptq (declared in include/q4_gptq.h): argument validation + kernel launches.
+// No torch types, no allocation, no synchronisation.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "q4_gptq.h"
+
+extern "C" {
+int q4_launch_dequant(const int32_t*, const int32_t*, const void*, const int32_t*, int, void*, int, int, hipStream_t);
+int q4_launch_gemv(const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, void*, int,
+                   int, int, int, void*, hipStream_t);
+int q4_launch_gemm(int, const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, const void*,
+                   const void*, const void*, int, void*, int, int, int, hipStream_t);
+}
+
+namespace {
+inline bool misaligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+
+int check_layer(const void* qweight, const void* qzeros, const void* scales, const void* g_idx,
+                int groupsize, int K, int N, int G) {
+    if (!qweight || !qzeros || !scales) return Q4_ERR_NULL_POINTER;
+    if (K < 64 || N < 64 || G < 1 || (K % 32) != 0 || (N % 64) != 0) return Q4_ERR_BAD_SHAPE;
+    if (!g_idx) {
+        if (groupsize < 32 || (groupsize % 32) != 0) return Q4_ERR_BAD_SHAPE;
+        if ((long)G * groupsize < K) return Q4_ERR_BAD_SHAPE;
+    }
+    if (misaligned(qweight) || misaligned(qzeros) || misaligned(scales) || (g_idx && misaligned(g_idx)))
+        return Q4_ERR_MISALIGNED;
+    return Q4_OK;
+}
+}  // namespace
+
+extern "C" int q4_abi_version(void) { return 1; }
+
+extern "C" const char* q4_error_string(int code) {
+    switch (code) {
+        case Q4_OK: return "ok";
+        case Q4_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case Q4_ERR_BAD_SHAPE: return "shape outside the supported range (see q4_gptq.h)";
+        case Q4_ERR_WORKSPACE: return "workspace missing or too small";
+        case Q4_ERR_LAUNCH: return "kernel launch failed";
+        case Q4_ERR_MISALIGNED: return "pointer not 16-byte aligned";
+        default: return "unknown error";
+    }
+}
+
+extern "C" int q4_dequant_f16(const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                              const int32_t* g_idx, int groupsize, void* out, int K, int N, int G, void* stream) {
+    int rc = check_layer(qweight, qzeros, scales, g_idx, groupsize, K, N, G);
+    if (rc != Q4_OK) return rc;
+    if (!out) return Q4_ERR_NULL_POINTER;
+    if (misaligned(out)) return Q4_ERR_MISALIGNED;
+    if (!g_idx && groupsize % 8 != 0) return Q4_ERR_BAD_SHAPE;
+    return q4_launch_dequant(qweight, qzeros, scales, g_idx, groupsize, out, K, N, (hipStream_t)stream);
+}
+
+extern "C" int q4_gemv_f16(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                           const int32_t* g_idx, int groupsize, void* y, int accumulate,
+                           int M, int K, int N, int G, void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = check_layer(qweight, qzeros, scales, g_idx, groupsize, K, N, G);
+    if (rc != Q4_OK) return rc;
+    if (!x || !y) return Q4_ERR_NULL_POINTER;
+    if (M < 1 || M > 16 || N > 262144) return Q4_ERR_BAD_SHAPE;
+    if (misaligned(x) || misaligned(y)) return Q4_ERR_MISALIGNED;
+    if (!workspace || workspace_bytes < q4_gemv_workspace_bytes(M, K, N)) return Q4_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
+    return q4_launch_gemv(x, qweight, qzeros, scales, g_idx, groupsize, y, accumulate, M, K, N, workspace,
+                          (hipStream_t)stream);
+}
+
+static int gemm_common(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                       const int32_t* g_idx, int groupsize, const void* bias, const void* la, const void* lb, int R,
+                       void* out, int M, int K, int N, int G, void* stream) {
+    int rc = check_layer(qweight, qzeros, scales, g_idx, groupsize, K, N, G);
+    if (rc != Q4_OK) return rc;
+    if (!act || !out) return Q4_ERR_NULL_POINTER;
+    if (M < 1 || (K % 128) != 0 || (N % 128) != 0) return Q4_ERR_BAD_SHAPE;
+    if (!g_idx && (groupsize % 64) != 0) return Q4_ERR_BAD_SHAPE;
+    if ((la != nullptr) != (lb != nullptr)) return Q4_ERR_NULL_POINTER;
+    if (la && (R < 8 || R > 64 || (R % 8) != 0)) return Q4_ERR_BAD_SHAPE;
+    if (misaligned(act) || misaligned(out) || (la && misaligned(la)) || (lb && misaligned(lb)))
+        return Q4_ERR_MISALIGNED;
+    return q4_launch_gemm(fwd, act, qweight, qzeros, scales, g_idx, groupsize, bias, la, lb, R, out, M, K, N,
+                          (hipStream_t)stream);
+}
+
+extern "C" int q4_gemm_fwd_f16(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                               const int32_t* g_idx, int groupsize, const void* bias,
+                               const void* xa, const void* lora_bt, int R,
+                               void* y, int M, int K, int N, int G, void* stream) {
+    return gemm_common(1, x, qweight, qzeros, scales, g_idx, groupsize, bias, xa, lora_bt, R, y, M, K, N, G, stream);
+}
+
+extern "C" int q4_gemm_bwd_dx_f16(const void* dy, const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                                  const int32_t* g_idx, int groupsize,
+                                  const void* dyb, const void* lora_a, int R,
+                                  void* dx, int M, int K, int N, int G, void* stream) {
+    return gemm_common(0, dy, qweight, qzeros, scales, g_idx, groupsize, nullptr, dyb, lora_a, R, dx, M, K, N, G, stream);
+}

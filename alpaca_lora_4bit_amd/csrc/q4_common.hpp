@@ -1,0 +1,64 @@
+// Shared device helpers for the gfx950 4-bit GPTQ kernels.
+//
+// Layout being decoded (reference: src/alpaca_lora_4bit/quant_cuda/quant_cuda_kernel.cu:1138-1152):
+//   qweight[k/8, n] holds the code of row k in bits 4*(k%8)..4*(k%8)+3,
+//   qzeros[g, n/8] holds the zero code of column n in bits 4*(n%8)..,
+//   W[k,n] = rn16( rn16(s*q) - rn16(s*(z+1)) ) with s = scales[g,n].
+// All fp16 arithmetic that must reproduce those three roundings is written on _Float16
+// vectors and this code is compiled with -ffp-contract=off, so a multiply is never fused
+// with the subtraction that follows it.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace q4 {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+
+constexpr uint32_t kMagic = 0x64006400u;  // two fp16 1024.0: (0x6400 | q) == 1024 + q exactly
+
+__device__ __forceinline__ half2_t as_half2(uint32_t u) {
+    return __builtin_bit_cast(half2_t, u);
+}
+__device__ __forceinline__ uint32_t as_u32(half2_t h) {
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+// (lo | hi << 16) of two 4-bit codes -> two fp16 values equal to the codes (exact).
+__device__ __forceinline__ half2_t codes_to_half2(uint32_t packed_codes) {
+    const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+    return as_half2(packed_codes | kMagic) - k1024;
+}
+
+// Three-rounding dequant of a pair: rn16(rn16(s*q) - zero), zero = rn16(s*(z+1)) precomputed.
+__device__ __forceinline__ half2_t dequant_pair(half2_t q, half2_t s, half2_t zero) {
+    half2_t p = s * q;
+    return p - zero;
+}
+
+// zero term rn16(s * half(z+1)) for two columns.
+__device__ __forceinline__ half2_t zero_term(half2_t s, uint32_t z_lo, uint32_t z_hi) {
+    half2_t zp1 = {(half_t)(float)(z_lo + 1u), (half_t)(float)(z_hi + 1u)};
+    return s * zp1;
+}
+
+// Natural-order unpack of one packed word (eight codes e0..e7 of one column) into four
+// half2 registers (e0,e1) (e2,e3) (e4,e5) (e6,e7), each value exactly the code.
+__device__ __forceinline__ void unpack8_natural(uint32_t w, half2_t out[4]) {
+    const uint32_t lo = w & 0x0F0F0F0Fu;          // bytes e0 e2 e4 e6
+    const uint32_t hi = (w >> 4) & 0x0F0F0F0Fu;   // bytes e1 e3 e5 e7
+    // v_perm_b32 byte selectors: 0-3 pick from the 2nd operand, 4-7 from the 1st, 0x0c = 0x00.
+    out[0] = codes_to_half2(__builtin_amdgcn_perm(hi, lo, 0x0c040c00u));
+    out[1] = codes_to_half2(__builtin_amdgcn_perm(hi, lo, 0x0c050c01u));
+    out[2] = codes_to_half2(__builtin_amdgcn_perm(hi, lo, 0x0c060c02u));
+    out[3] = codes_to_half2(__builtin_amdgcn_perm(hi, lo, 0x0c070c03u));
+}
+
+}  // namespace q4

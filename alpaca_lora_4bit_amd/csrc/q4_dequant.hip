@@ -1,0 +1,70 @@
+// Dense dequantization  out fp16 [K, N] = W   (HBM-bound: reads K*N/2 B, writes 2*K*N B).
+//
+// One thread owns one packed word-row (8 rows of W) x 8 adjacent columns: it reads 32 B of
+// qweight with two 128-bit loads and writes eight 16-byte row segments, so a wavefront
+// writes 1 KiB contiguous per row.  Scale / zero are re-fetched only when the row's group
+// changes, which is never inside a word-row without act-order and up to 8 times with it.
+//
+// Values follow src/alpaca_lora_4bit/quant_cuda/quant_cuda_kernel.cu:1138-1152 bit for bit.
+#include "q4_common.hpp"
+
+namespace q4 {
+
+__global__ __launch_bounds__(256) void dequant_kernel(
+    const uint32_t* __restrict__ qweight, const uint32_t* __restrict__ qzeros,
+    const half_t* __restrict__ scales, const int32_t* __restrict__ g_idx, int groupsize,
+    half_t* __restrict__ out, int K, int N) {
+    const int ncol8 = N >> 3;
+    const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long total = (long)(K >> 3) * ncol8;
+    if (tid >= total) return;
+    const int kw = (int)(tid / ncol8);
+    const int nb = (int)(tid - (long)kw * ncol8);
+    const int n0 = nb << 3;
+
+    const uint4_t* wp = reinterpret_cast<const uint4_t*>(qweight + (size_t)kw * N + n0);
+    const uint4_t wa = wp[0], wb = wp[1];
+    const uint32_t w[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+
+    int gprev = -1;
+    half2_t s2[4], zero2[4];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int k = (kw << 3) + e;
+        const int g = g_idx ? g_idx[k] : k / groupsize;
+        if (g != gprev) {
+            gprev = g;
+            const uint4_t sv = *reinterpret_cast<const uint4_t*>(scales + (size_t)g * N + n0);
+            const uint32_t zw = qzeros[(size_t)g * ncol8 + nb];
+            const uint32_t sraw[4] = {sv.x, sv.y, sv.z, sv.w};
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                s2[p] = as_half2(sraw[p]);
+                zero2[p] = zero_term(s2[p], (zw >> (8 * p)) & 0xFu, (zw >> (8 * p + 4)) & 0xFu);
+            }
+        }
+        uint32_t o[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const uint32_t codes = ((w[2 * p] >> (4 * e)) & 0xFu) | (((w[2 * p + 1] >> (4 * e)) & 0xFu) << 16);
+            o[p] = as_u32(dequant_pair(codes_to_half2(codes), s2[p], zero2[p]));
+        }
+        uint4_t ov = {o[0], o[1], o[2], o[3]};
+        *reinterpret_cast<uint4_t*>(out + (size_t)k * N + n0) = ov;
+    }
+}
+
+}  // namespace q4
+
+extern "C" int q4_launch_dequant(const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                                 const int32_t* g_idx, int groupsize, void* out, int K, int N,
+                                 hipStream_t stream) {
+    const long total = (long)(K / 8) * (N / 8);
+    const int threads = 256;
+    const long blocks = (total + threads - 1) / threads;
+    hipLaunchKernelGGL(q4::dequant_kernel, dim3((unsigned)blocks), dim3(threads), 0, stream,
+                       reinterpret_cast<const uint32_t*>(qweight), reinterpret_cast<const uint32_t*>(qzeros),
+                       reinterpret_cast<const q4::half_t*>(scales), g_idx, groupsize,
+                       reinterpret_cast<q4::half_t*>(out), K, N);
+    return hipGetLastError() == hipSuccess ? 0 : -4;
+}

@@ -1,0 +1,115 @@
+"""Host dispatch for the 4-bit matmul: same functions and module-level knobs as the reference's
+src/alpaca_lora_4bit/matmul_utils_4bit.py, routed to the gfx950 kernels.
+
+What changed underneath (none of it visible in the signatures):
+
+* rows <= auto_switch_thd (default 16, the most the GEMV kernel takes) go to one GEMV launch
+  that reads the packed weights once for all rows; the reference launches one grid slice per row
+  and switches to recons + matmul above 8 rows (matmul_utils_4bit.py:15,164-167).
+* larger inputs go to the fused dequant + MFMA GEMM.  No dense [K, N] buffer exists, so
+  `get_buffer` / `cache_buffer` / `buffer_mat_dic` are kept only as inert names.
+* `act_order` and `faster_mode` no longer select kernels: whether `g_idx` is a real
+  permutation is detected per tensor (quant_hip.classify_g_idx).  The reference's default
+  kernel ignores g_idx unless the user sets `act_order = True` by hand (:75-87); here a
+  permuted g_idx is always honoured.
+"""
+import logging
+
+import numpy as np
+import torch
+
+try:
+    from . import quant_hip
+except (ImportError, ModuleNotFoundError) as e:   # same convention as matmul_utils_4bit.py:5-9
+    logging.exception("libq4gptq.so is not built: run __graft_entry__.build()")
+    raise e
+
+# Global knobs (names and defaults of matmul_utils_4bit.py:11-20; see the module docstring)
+buffer_mat_dic = {}
+use_new = True
+auto_switch = True
+auto_switch_thd = 16
+debug = False
+faster_mode = 'old_faster'
+valid_faster_mode = ('faster', 'old_faster')
+act_order = False
+cache_buffer = True
+
+
+def get_buffer(shape_of_qweight, dtype=torch.float16, device='cuda', bits=4):
+    """Dense [K, N] scratch of the reference (matmul_utils_4bit.py:22-33).  Nothing in this
+    package uses it; it is provided for callers that dequantize explicitly."""
+    target_shape = (shape_of_qweight[0] * (32 // bits), shape_of_qweight[1])
+    if not cache_buffer:
+        return torch.zeros(target_shape, dtype=dtype, device=device)
+    buf = buffer_mat_dic.get(target_shape)
+    if buf is None or buf.device != torch.device(device) or buf.dtype != dtype:
+        buf = torch.zeros(target_shape, dtype=dtype, device=device)
+        buffer_mat_dic[target_shape] = buf
+    return buf
+
+
+def _groupsize_of(qweight, scales, groupsize):
+    if groupsize is not None and groupsize > 0:
+        return int(groupsize)
+    K, G = qweight.shape[0] * 8, scales.shape[0]
+    return -(-K // G)
+
+
+def _half_scales(scales):
+    return scales if scales.dtype == torch.float16 else scales.half()
+
+
+def _matmul4bit_v2(x, qweight, scales, zeros, g_idx, groupsize=None):
+    """x @ W for a handful of rows (decode).  matmul_utils_4bit.py:59-95."""
+    if debug:
+        print('_matmul4bit_v2')
+    assert qweight.shape[0] * 8 == x.shape[-1]
+    if faster_mode not in valid_faster_mode and faster_mode != 'disable':
+        raise ValueError('faster_mode should be in {}'.format(valid_faster_mode))
+    outshape = x.shape[:-1] + (qweight.shape[1],)
+    dtype = x.dtype
+    y = quant_hip.gemv(x, qweight, zeros, _half_scales(scales), g_idx, _groupsize_of(qweight, scales, groupsize))
+    return y.to(dtype).reshape(outshape)
+
+
+def _matmul4bit_v2_recons(x, qweight, scales, zeros, g_idx, transpose=False, groupsize=None):
+    """x @ W (or x @ W.T with transpose=True) through the fused dequant-MFMA GEMM; the
+    reference dequantizes into a dense buffer and calls torch.matmul (matmul_utils_4bit.py:114-127)."""
+    if debug:
+        print('_matmul4bit_v2_recons')
+    if not transpose:
+        assert qweight.shape[0] * 8 == x.shape[-1]
+    else:
+        assert qweight.shape[1] == x.shape[-1]
+    gs = _groupsize_of(qweight, scales, groupsize)
+    lead = x.shape[:-1]
+    if not transpose:
+        out = quant_hip.gemm_fwd(x, qweight, zeros, _half_scales(scales), g_idx, gs)
+    else:
+        out = quant_hip.gemm_bwd_dx(x, qweight, zeros, _half_scales(scales), g_idx, gs)
+    return out.reshape(lead + (out.shape[-1],))
+
+
+def _v1_unsupported(*args, **kwargs):
+    raise NotImplementedError('the v1 (per-column fp zeros) and 2-bit layouts are not built for gfx950; '
+                              'only 4-bit v2 checkpoints (int32 qzeros) are supported')
+
+
+_matmul4bit_v1 = _v1_unsupported
+_matmul4bit_v1_recons = _v1_unsupported
+_matmul2bit_v2_recons = _v1_unsupported
+v2_to_v1 = _v1_unsupported
+
+
+def matmul4bit(x, qweight, scales, zeros, g_idx=None, groupsize=None):
+    """No-grad dispatcher, matmul_utils_4bit.py:146-170."""
+    if zeros.dtype != torch.int32:
+        return _v1_unsupported()
+    gs = _groupsize_of(qweight, scales, groupsize)
+    rows = int(np.prod(x.shape[:-1]))
+    thd = min(int(auto_switch_thd), quant_hip.MAX_GEMV_ROWS)
+    use_gemv = rows <= thd if (use_new and auto_switch) else rows <= quant_hip.MAX_GEMV_ROWS
+    if use_gemv and rows >= 1:
+        return _matmul4bit_v2(x, qweight, scales, zeros, g_idx, gs)
+    return _matmul4bit_v2_recons(x.half(), qweight, scales.half(), zeros, g_idx, groupsize=gs)

@@ -1,0 +1,287 @@
+"""LoRA on top of the 4-bit linear: `Linear4bitLt` and `GPTQLoraModel` with the interface of the
+reference's src/alpaca_lora_4bit/models.py:13-163 (written against peft 0.6).
+
+When peft is importable its `LoraLayer` / `LoraModel` are the base classes, exactly as in the
+reference.  When it is not, a small stand-in `LoraLayer` with the same attribute names
+(`r, lora_alpha, scaling, lora_dropout, lora_A, lora_B, active_adapters, disable_adapters,
+update_layer, set_adapter`) keeps `Linear4bitLt` usable on its own.  The stand-in follows
+peft 0.6's documented behaviour (A: Kaiming-uniform with a=sqrt(5), B: zeros, scaling =
+lora_alpha / r); peft itself could not be imported where this was written, so equality with
+peft's internals is not verified -- the adapter arithmetic (models.py:58-66) is.
+"""
+import math
+import warnings
+
+import torch
+import torch.nn as nn
+
+from . import autograd_4bit
+from .autograd_4bit import Autograd4bitQuantLinear
+
+try:  # pragma: no cover - depends on the environment
+    from peft.tuners import lora as _peft_lora
+    from peft.tuners.lora import LoraLayer
+    HAVE_PEFT = True
+except ImportError:
+    _peft_lora = None
+    HAVE_PEFT = False
+
+    class LoraLayer:
+        """Minimal stand-in for peft.tuners.lora.LoraLayer (see the module docstring)."""
+
+        adapter_layer_names = ("lora_A", "lora_B")
+
+        def __init__(self, in_features: int, out_features: int, **kwargs):
+            self.r = {}
+            self.lora_alpha = {}
+            self.scaling = {}
+            self.lora_dropout = nn.ModuleDict({})
+            self.lora_A = nn.ModuleDict({})
+            self.lora_B = nn.ModuleDict({})
+            self._disable_adapters = False
+            self._active_adapter = "default"
+            self.merged_adapters = []
+            self.in_features = in_features
+            self.out_features = out_features
+            self.kwargs = kwargs
+
+        @property
+        def disable_adapters(self):
+            return self._disable_adapters
+
+        @property
+        def active_adapters(self):
+            a = self._active_adapter
+            return [a] if isinstance(a, str) else list(a)
+
+        @property
+        def active_adapter(self):
+            return self._active_adapter
+
+        def enable_adapters(self, enabled: bool):
+            self._disable_adapters = not enabled
+
+        def set_adapter(self, adapter_names):
+            if isinstance(adapter_names, str):
+                adapter_names = [adapter_names]
+            for layer_name in self.adapter_layer_names:
+                for key, layer in getattr(self, layer_name).items():
+                    layer.requires_grad_(key in adapter_names)
+            self._active_adapter = adapter_names
+
+        def update_layer(self, adapter_name, r, lora_alpha, lora_dropout, init_lora_weights):
+            if r <= 0:
+                raise ValueError(f"`r` should be a positive integer value but the value passed is {r}")
+            self.r[adapter_name] = r
+            self.lora_alpha[adapter_name] = lora_alpha
+            self.lora_dropout[adapter_name] = nn.Dropout(p=lora_dropout) if lora_dropout > 0.0 else nn.Identity()
+            self.lora_A[adapter_name] = nn.Linear(self.in_features, r, bias=False)
+            self.lora_B[adapter_name] = nn.Linear(r, self.out_features, bias=False)
+            self.scaling[adapter_name] = lora_alpha / r
+            if init_lora_weights:
+                nn.init.kaiming_uniform_(self.lora_A[adapter_name].weight, a=math.sqrt(5))
+                nn.init.zeros_(self.lora_B[adapter_name].weight)
+            weight = getattr(self, "weight", None)
+            if weight is not None:
+                for name in self.adapter_layer_names:
+                    getattr(self, name)[adapter_name].to(weight.device)
+            self.set_adapter(self.active_adapters)
+
+
+# Use the fused GEMM (adapter folded into the main kernel) whenever the case allows it.
+fuse_lora = True
+
+
+class Linear4bitLt(Autograd4bitQuantLinear, LoraLayer):
+    """4-bit linear + LoRA adapters (models.py:13-76)."""
+
+    def __init__(self, adapter_name, in_features, out_features, groupsize: int = -1, is_v1_model: bool = False,
+                 r: int = 0, lora_alpha: int = 1, lora_dropout: float = 0.0, **kwargs):
+        Autograd4bitQuantLinear.__init__(self, in_features, out_features, groupsize, is_v1_model)
+        LoraLayer.__init__(self, in_features=in_features, out_features=out_features)
+
+        # the quantized base weights are frozen (models.py:37-45)
+        for name in ('qweight', 'scales', 'bias') + (('zeros',) if self.is_v1_model else ('qzeros', 'g_idx')):
+            getattr(self, name).requires_grad = False
+
+        init_lora_weights = kwargs.pop("init_lora_weights", True)
+        self.update_layer(adapter_name, r, lora_alpha, lora_dropout, init_lora_weights)
+        self.set_adapter(adapter_names=[adapter_name])
+
+    # ---- fused path --------------------------------------------------------------------
+    def _fusable_adapter(self, x):
+        """Name of the single adapter the fused kernel can take for this call, else None."""
+        if not fuse_lora or self.is_v1_model or self.bits != 4 or not x.is_cuda:
+            return None
+        if autograd_4bit.backend != 'cuda':
+            return None
+        active = [a for a in self.active_adapters if a in self.lora_A.keys()]
+        if len(active) != 1:
+            return None
+        name = active[0]
+        r = self.lora_A[name].weight.shape[0]
+        if r % 8 != 0 or not (8 <= r <= 64):
+            return None
+        drop = self.lora_dropout[name]
+        if isinstance(drop, nn.Dropout) and drop.p > 0.0 and self.training:
+            return None
+        rows = x.numel() // x.shape[-1]
+        if rows <= autograd_4bit.quant_hip.MAX_GEMV_ROWS:
+            return None
+        if self.in_features % 128 or self.out_features % 128:
+            return None
+        if not (torch.is_autocast_enabled('cuda') or x.dtype == torch.float16):
+            return None
+        return name
+
+    def forward(self, x: torch.Tensor):
+        if not self.disable_adapters:
+            name = self._fusable_adapter(x)
+            if name is not None:
+                bias = None
+                if not self.disable_bias:
+                    bias = self.bias if self.bias.dtype == torch.float16 else self.bias.half()
+                return autograd_4bit.AutogradMatmul4bitLora.apply(
+                    x, self.qweight, self.scales, self.qzeros, self.g_idx, bias,
+                    self.lora_A[name].weight, self.lora_B[name].weight, float(self.scaling[name]), self.groupsize)
+
+        # reference composition (models.py:51-69)
+        result = super().forward(x)
+        if self.disable_adapters:
+            return result
+        previous_dtype = result.dtype
+        for active_adapter in self.active_adapters:
+            if active_adapter not in self.lora_A.keys():
+                continue
+            lora_A = self.lora_A[active_adapter]
+            lora_B = self.lora_B[active_adapter]
+            dropout = self.lora_dropout[active_adapter]
+            scaling = self.scaling[active_adapter]
+            x = x.to(lora_A.weight.dtype)
+            result = result + (lora_B(lora_A(dropout(x))) * scaling).to(result.dtype)
+        return result.to(previous_dtype)
+
+    @property
+    def weight(self):
+        """Device/dtype carrier so that peft's update_layer moves the adapter weights to the
+        GPU without changing their dtype (models.py:71-76: dtype is the int32 of qweight)."""
+        qweight = self.qweight
+
+        class WeightDeviceClass:
+            device = qweight.device
+            dtype = qweight.dtype
+        return WeightDeviceClass()
+
+
+def _share_quant_tensors(new_module, child):
+    """models.py:119-127: the replacement shares the packed tensors with the layer it replaces."""
+    new_module.qweight = child.qweight
+    new_module.scales = child.scales
+    if child.is_v1_model:
+        new_module.zeros = child.zeros
+    else:
+        new_module.qzeros = child.qzeros
+        new_module.g_idx = child.g_idx
+    new_module.bias = child.bias
+
+
+def _move_adapters(new_module, device):
+    for name, module in new_module.named_modules():
+        if "lora_" in name or "ranknum" in name:
+            module.to(device)
+
+
+if HAVE_PEFT:  # pragma: no cover - peft is not available where the tests run
+    from peft.tuners.lora import Linear as _PeftLinear
+    from transformers.pytorch_utils import Conv1D
+
+    class GPTQLoraModel(_peft_lora.LoraModel):
+        """peft LoraModel that builds Linear4bitLt for 4-bit targets (models.py:79-163)."""
+
+        @staticmethod
+        def _create_new_module(lora_config, adapter_name, target, **kwargs):
+            bias = kwargs.pop("bias", False)
+            if isinstance(target, Autograd4bitQuantLinear):
+                return Linear4bitLt(adapter_name, target.in_features, target.out_features, target.groupsize,
+                                    target.is_v1_model, bias=bias, **kwargs)
+            if isinstance(target, torch.nn.Linear):
+                in_features, out_features = target.in_features, target.out_features
+                if kwargs["fan_in_fan_out"]:
+                    warnings.warn("fan_in_fan_out is set to True but the target module is `torch.nn.Linear`. "
+                                  "Setting fan_in_fan_out to False.")
+                    kwargs["fan_in_fan_out"] = lora_config.fan_in_fan_out = False
+            elif isinstance(target, Conv1D):
+                in_features, out_features = (target.weight.ds_shape if hasattr(target.weight, "ds_shape")
+                                             else target.weight.shape)
+                kwargs["is_target_conv_1d_layer"] = True
+                if not kwargs["fan_in_fan_out"]:
+                    warnings.warn("fan_in_fan_out is set to False but the target module is `Conv1D`. "
+                                  "Setting fan_in_fan_out to True.")
+                    kwargs["fan_in_fan_out"] = lora_config.fan_in_fan_out = True
+            else:
+                raise ValueError(f"Target module {target} is not supported. "
+                                 f"Currently, only `torch.nn.Linear` and `Conv1D` are supported.")
+            return _PeftLinear(adapter_name, in_features, out_features, bias=bias, **kwargs)
+
+        @staticmethod
+        def _replace_module(parent, child_name, new_module, child):
+            setattr(parent, child_name, new_module)
+            if isinstance(child, Autograd4bitQuantLinear) and isinstance(new_module, Linear4bitLt):
+                _share_quant_tensors(new_module, child)
+                if getattr(child, "state", None) is not None:
+                    new_module.state = child.state
+                    new_module.to(child.qweight.device)
+                _move_adapters(new_module, child.qweight.device)
+                return
+            if hasattr(child, "base_layer"):
+                child = child.base_layer
+            elif hasattr(child, "quant_linear_module"):
+                child = child.quant_linear_module
+            if not hasattr(new_module, "base_layer"):
+                new_module.weight = child.weight
+                if hasattr(child, "bias"):
+                    new_module.bias = child.bias
+            if getattr(child, "state", None) is not None:
+                if hasattr(new_module, "base_layer"):
+                    new_module.base_layer.state = child.state
+                else:
+                    new_module.state = child.state
+                new_module.to(child.weight.device)
+            _move_adapters(new_module, child.weight.device)
+else:
+    class GPTQLoraModel:
+        """Without peft there is no LoraModel to derive from; the two hooks the monkeypatch
+        installs are still provided (same signatures as models.py:80-81,116-117) for 4-bit targets."""
+
+        @staticmethod
+        def _create_new_module(lora_config, adapter_name, target, **kwargs):
+            kwargs.pop("bias", False)
+            if not isinstance(target, Autograd4bitQuantLinear):
+                raise ValueError(f"Target module {target} is not supported without peft installed.")
+            return Linear4bitLt(adapter_name, target.in_features, target.out_features, target.groupsize,
+                                target.is_v1_model, **kwargs)
+
+        @staticmethod
+        def _replace_module(parent, child_name, new_module, child):
+            setattr(parent, child_name, new_module)
+            _share_quant_tensors(new_module, child)
+            _move_adapters(new_module, child.qweight.device)
+
+
+def inject_lora_layers(model, target_modules=("q_proj", "v_proj"), r=8, lora_alpha=16, lora_dropout=0.0,
+                       adapter_name="default", init_lora_weights=True):
+    """peft-free injection: swap every Autograd4bitQuantLinear whose attribute name is in
+    `target_modules` for a Linear4bitLt sharing its packed tensors (what get_peft_model does
+    through GPTQLoraModel, finetune.py:75-84), freeze everything else, return the new layers."""
+    for p in model.parameters():
+        p.requires_grad_(False)
+    replaced = {}
+    for parent_name, parent in list(model.named_modules()):
+        for child_name, child in list(parent.named_children()):
+            if child_name in target_modules and type(child) is Autograd4bitQuantLinear:
+                new = Linear4bitLt(adapter_name, child.in_features, child.out_features, child.groupsize,
+                                   child.is_v1_model, r=r, lora_alpha=lora_alpha, lora_dropout=lora_dropout,
+                                   init_lora_weights=init_lora_weights)
+                GPTQLoraModel._replace_module(parent, child_name, new, child)
+                replaced[f"{parent_name}.{child_name}" if parent_name else child_name] = new
+    return replaced

@@ -1,0 +1,257 @@
+"""Tensor-level host side of libq4gptq: the stand-in for the reference's `quant_cuda` module.
+
+Two layers:
+
+* `dequant`, `gemv`, `gemm_fwd`, `gemm_bwd_dx` -- the operators the rest of this package uses.
+  They do the checks the reference's C++ binding leaves out (dtype, device, contiguity, shape,
+  g_idx range), pick torch's CURRENT stream for the tensor's device, and call the C ABI.
+* `vecquant4recons_v2`, `vecquant4matmul`, `vecquant4matmul_faster`, `vecquant4matmul_old_faster`
+  -- same names, argument order and "write into the caller's buffer, return None" convention as
+  the pybind functions of src/alpaca_lora_4bit/quant_cuda/quant_cuda.cpp:204-227, so code
+  written against `quant_cuda` keeps working.
+
+Nothing here computes on the CPU: without the built library the import fails.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from ._lib import Q4Error  # noqa: F401  (re-exported)
+
+_lib.lib()  # fail at import time, loudly, if the HIP library is missing
+
+MAX_GEMV_ROWS = 16
+_workspaces = {}
+
+
+def _ptr(t):
+    return 0 if t is None else t.data_ptr()
+
+
+def _stream(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require(cond, msg):
+    if not cond:
+        raise ValueError(msg)
+
+
+def _check_layer(qweight, qzeros, scales, g_idx, groupsize):
+    _require(qweight.is_cuda, "qweight must be on the GPU")
+    dev = qweight.device
+    _require(qweight.dtype == torch.int32 and qweight.dim() == 2, "qweight must be int32 [K/8, N]")
+    _require(qzeros.dtype == torch.int32 and qzeros.dim() == 2, "qzeros must be int32 [G, N/8]")
+    _require(scales.dtype == torch.float16 and scales.dim() == 2, "scales must be float16 [G, N]")
+    K, N = qweight.shape[0] * 8, qweight.shape[1]
+    G = scales.shape[0]
+    _require(scales.shape[1] == N and tuple(qzeros.shape) == (G, N // 8),
+             f"scales {tuple(scales.shape)} / qzeros {tuple(qzeros.shape)} do not match qweight {tuple(qweight.shape)}")
+    for t in (qweight, qzeros, scales):
+        _require(t.is_contiguous() and t.device == dev, "quantized tensors must be contiguous and on one device")
+    if g_idx is not None:
+        _require(g_idx.dtype == torch.int32 and g_idx.shape == (K,) and g_idx.is_contiguous() and g_idx.device == dev,
+                 "g_idx must be a contiguous int32 [K] tensor on the same device")
+    else:
+        _require(groupsize is not None and groupsize > 0, "groupsize is required when g_idx is None")
+    return dev, K, N, G
+
+
+def classify_g_idx(g_idx, groupsize, G):
+    """'seq' when g_idx[k] == k // groupsize for every k (the kernels then skip the gather),
+    else 'gidx'.  Also validates 0 <= g_idx < G.  The verdict is cached on the tensor object
+    together with its in-place version counter; the first call per tensor synchronises."""
+    if g_idx is None:
+        return "seq"
+    key = (g_idx._version, int(groupsize or 0), G)
+    cached = getattr(g_idx, "_q4_kind", None)
+    if cached is not None and cached[0] == key:
+        return cached[1]
+    lo, hi = int(g_idx.min()), int(g_idx.max())
+    if lo < 0 or hi >= G:
+        raise ValueError(f"g_idx values must lie in [0, {G}); found [{lo}, {hi}]")
+    kind = "gidx"
+    if groupsize and groupsize > 0 and groupsize % 32 == 0:
+        ref = torch.arange(g_idx.numel(), device=g_idx.device, dtype=torch.int32) // groupsize
+        if bool(torch.equal(g_idx, ref)):
+            kind = "seq"
+    g_idx._q4_kind = (key, kind)
+    return kind
+
+
+def _gidx_arg(g_idx, groupsize, G, need_multiple=32):
+    """Returns (pointer-or-0, groupsize) to hand to the C ABI."""
+    if g_idx is None:
+        _require(groupsize % need_multiple == 0, f"groupsize must be a multiple of {need_multiple} without g_idx")
+        return 0, int(groupsize)
+    kind = classify_g_idx(g_idx, groupsize, G)
+    if kind == "seq" and groupsize % need_multiple == 0:
+        return 0, int(groupsize)
+    return g_idx.data_ptr(), int(groupsize or 0)
+
+
+def _workspace(device, nbytes):
+    key = (device.index, _stream(device))
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(max(nbytes, 1 << 22), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def _flat_half(x, K, dev, what):
+    _require(x.is_cuda and x.device == dev, f"{what} must be on {dev}")
+    _require(x.shape[-1] == K, f"{what} last dimension {x.shape[-1]} != {K}")
+    x2 = x.reshape(-1, K)
+    if x2.dtype != torch.float16:
+        x2 = x2.half()
+    return x2.contiguous()
+
+
+# ------------------------------------------------------------------------------- operators
+def dequant(qweight, qzeros, scales, g_idx=None, groupsize=None, out=None):
+    """W fp16 [K, N], bit-exact with vecquant4recons_v2 (quant_cuda_kernel.cu:1127-1153)."""
+    dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
+    if out is None:
+        out = torch.empty((K, N), dtype=torch.float16, device=dev)
+    _require(out.dtype == torch.float16 and tuple(out.shape) == (K, N) and out.is_contiguous() and out.device == dev,
+             "out must be a contiguous float16 [K, N] tensor on the same device")
+    gp, gs = _gidx_arg(g_idx, groupsize, G, need_multiple=8)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().q4_dequant_f16(qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), gp, gs,
+                                       out.data_ptr(), K, N, G, _stream(dev))
+    _lib.check(rc, "q4_dequant_f16")
+    return out
+
+
+def gemv(x, qweight, qzeros, scales, g_idx=None, groupsize=None, out=None, accumulate=False):
+    """y fp16 [M, N] = x [M, K] @ W for M <= 16 (decode)."""
+    dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
+    x2 = _flat_half(x, K, dev, "x")
+    M = x2.shape[0]
+    _require(1 <= M <= MAX_GEMV_ROWS, f"gemv handles 1..{MAX_GEMV_ROWS} rows, got {M}")
+    if out is None:
+        _require(not accumulate, "accumulate needs an output tensor")
+        out = torch.empty((M, N), dtype=torch.float16, device=dev)
+    _require(out.dtype == torch.float16 and tuple(out.shape) == (M, N) and out.is_contiguous() and out.device == dev,
+             "out must be a contiguous float16 [M, N] tensor on the same device")
+    gp, gs = _gidx_arg(g_idx, groupsize, G)
+    L = _lib.lib()
+    nbytes = L.q4_gemv_workspace_bytes(M, K, N)
+    with torch.cuda.device(dev):
+        ws = _workspace(dev, nbytes)
+        rc = L.q4_gemv_f16(x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), gp, gs,
+                           out.data_ptr(), int(bool(accumulate)), M, K, N, G, ws.data_ptr(), ws.numel(), _stream(dev))
+    _lib.check(rc, "q4_gemv_f16")
+    return out
+
+
+def _lora_pair(la, lb, rows, cols, dev):
+    if la is None and lb is None:
+        return None, None, 0
+    _require(la is not None and lb is not None, "both LoRA operands are required")
+    R = la.shape[-1]
+    _require(la.dtype == torch.float16 and lb.dtype == torch.float16, "LoRA operands must be float16")
+    _require(tuple(la.shape) == (rows, R) and tuple(lb.shape) == (R, cols), "LoRA operand shapes do not match")
+    _require(R % 8 == 0 and 8 <= R <= 64, "LoRA rank must be a multiple of 8 in [8, 64] for the fused path")
+    _require(la.is_contiguous() and lb.is_contiguous() and la.device == dev and lb.device == dev,
+             "LoRA operands must be contiguous and on the same device")
+    return la, lb, R
+
+
+def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, xa=None, lora_bt=None):
+    """y fp16 [M, N] = x @ W (+ bias) (+ xa @ lora_bt), W dequantized tile by tile in LDS."""
+    dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
+    x2 = _flat_half(x, K, dev, "x")
+    M = x2.shape[0]
+    if bias is not None:
+        _require(bias.dtype == torch.float16 and tuple(bias.shape) == (N,) and bias.is_contiguous()
+                 and bias.device == dev, "bias must be a contiguous float16 [N] tensor on the same device")
+    xa, lora_bt, R = _lora_pair(xa, lora_bt, M, N, dev)
+    gp, gs = _gidx_arg(g_idx, groupsize, G, need_multiple=64)
+    out = torch.empty((M, N), dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().q4_gemm_fwd_f16(x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
+                                        gp, gs, _ptr(bias), _ptr(xa), _ptr(lora_bt), R,
+                                        out.data_ptr(), M, K, N, G, _stream(dev))
+    _lib.check(rc, "q4_gemm_fwd_f16")
+    return out
+
+
+def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=None, lora_a=None):
+    """dx fp16 [M, K] = dy [M, N] @ W^T (+ dyb @ lora_a)."""
+    dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
+    dy2 = _flat_half(dy, N, dev, "grad_output")
+    M = dy2.shape[0]
+    dyb, lora_a, R = _lora_pair(dyb, lora_a, M, K, dev)
+    gp, gs = _gidx_arg(g_idx, groupsize, G, need_multiple=64)
+    out = torch.empty((M, K), dtype=torch.float16, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().q4_gemm_bwd_dx_f16(dy2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
+                                           gp, gs, _ptr(dyb), _ptr(lora_a), R,
+                                           out.data_ptr(), M, K, N, G, _stream(dev))
+    _lib.check(rc, "q4_gemm_bwd_dx_f16")
+    return out
+
+
+# ------------------------------------------------- quant_cuda-compatible entry points
+def _infer_groupsize(K, G):
+    return -(-K // G)
+
+
+def _scales_half(scales):
+    # the reference hands fp32 copies of fp16 scales to some kernels (matmul_utils_4bit.py:78,87)
+    return scales if scales.dtype == torch.float16 else scales.half()
+
+
+def vecquant4recons_v2(mat, res, scales, zeros, g_idx):
+    """quant_cuda.vecquant4recons_v2(mat, res, scales, zeros, g_idx) -> None; res[K,N] = W.
+    (quant_cuda.cpp:143-148).  fp16 `res` is written in place; other dtypes via one cast."""
+    K = mat.shape[0] * 8
+    gs = _infer_groupsize(K, scales.shape[0])
+    if res.dtype == torch.float16 and res.is_contiguous():
+        dequant(mat, zeros, _scales_half(scales), g_idx, gs, out=res)
+    else:
+        res.copy_(dequant(mat, zeros, _scales_half(scales), g_idx, gs))
+
+
+def _matmul_into(vec, mat, mul, scales, zeros, g_idx, groupsize):
+    y = gemv(vec, mat, zeros, _scales_half(scales), g_idx, groupsize)
+    mul.add_(y.to(mul.dtype))          # the reference kernels accumulate into a pre-zeroed `mul`
+
+
+def vecquant4matmul(vec, mat, mul, scales, zeros, g_idx):
+    """quant_cuda.vecquant4matmul (quant_cuda.cpp:55-61): mul += vec @ W, rows grouped by g_idx."""
+    K = mat.shape[0] * 8
+    _matmul_into(vec, mat, mul, scales, zeros, g_idx, _infer_groupsize(K, scales.shape[0]))
+
+
+def vecquant4matmul_faster(vec, mat, mul, scales, zeros, g_idx, vec_height):
+    """quant_cuda.vecquant4matmul_faster (quant_cuda.cpp:93-101)."""
+    K = mat.shape[0] * 8
+    assert vec_height * 2 == K
+    _matmul_into(vec, mat, mul, scales, zeros, g_idx, _infer_groupsize(K, scales.shape[0]))
+
+
+def vecquant4matmul_old_faster(vec, mat, mul, scales, zeros, groupsize, vec_height):
+    """quant_cuda.vecquant4matmul_old_faster (quant_cuda.cpp:105-113): sequential groups of
+    `groupsize` rows, g_idx not consulted (quant_cuda_kernel.cu:1024)."""
+    K = mat.shape[0] * 8
+    assert vec_height * 2 == K
+    if groupsize is None or groupsize <= 0:
+        groupsize = _infer_groupsize(K, scales.shape[0])
+    _matmul_into(vec, mat, mul, scales, zeros, None, groupsize)
+
+
+def _unsupported(name):
+    def fn(*args, **kwargs):
+        raise NotImplementedError(f"{name}: only the 4-bit v2 (grouped, int32 qzeros) layout is built for gfx950")
+    fn.__name__ = name
+    return fn
+
+
+for _n in ("vecquant2matmul", "vecquant3matmul", "vecquant8matmul", "vecquant2matmul_faster", "vecquant3matmul_faster",
+           "vecquant4matmul_v1_faster", "vecquant4recons_v1", "vecquant2recons_v2", "vecquant4matmul_seq_v2",
+           "vecquant4matmul_g"):
+    globals()[_n] = _unsupported(_n)

@@ -1,0 +1,93 @@
+/* C ABI of libq4gptq: 4-bit GPTQ dequantize / multiply kernels for AMD MI355X (gfx950).
+ *
+ * Plain pointers and sizes only.  Every pointer is DEVICE memory on the current HIP device
+ * unless said otherwise; `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ * All calls are asynchronous on `stream`, keep no reference to any argument after the
+ * kernels they enqueue have run, and return Q4_OK or a negative Q4_ERR_* code (never throw,
+ * never abort).  Tensors are dense row-major in the GPTQ "v2" layout:
+ *
+ *   qweight int32  [K/8, N]   eight 4-bit codes per word along K (code of row k in bits 4*(k%8)..)
+ *   qzeros  int32  [G, N/8]   eight 4-bit zero codes per word along N; the zero point is code+1
+ *   scales  fp16   [G, N]
+ *   g_idx   int32  [K]        group of row k (act-order); NULL means k / groupsize
+ *   W[k,n] = rn16( rn16(s*q) - rn16(s*(z+1)) ),  s = scales[g,n], g = g_idx[k]
+ *
+ * Shape limits common to all entry points: K % 32 == 0, N % 64 == 0, K,N >= 64, G >= 1,
+ * 0 <= g_idx[k] < G (not checked on the device side of the hot loops: validate on the host).
+ *
+ * The reference is johnsmith0031/alpaca_lora_4bit; paths below are relative to its
+ * src/alpaca_lora_4bit/.
+ */
+#ifndef Q4_GPTQ_H
+#define Q4_GPTQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define Q4_OK 0
+#define Q4_ERR_NULL_POINTER (-1)   /* a required pointer is NULL */
+#define Q4_ERR_BAD_SHAPE (-2)      /* a size violates the limits above / of the entry point */
+#define Q4_ERR_WORKSPACE (-3)      /* workspace missing or smaller than *_workspace_bytes() */
+#define Q4_ERR_LAUNCH (-4)         /* hipLaunch reported an error (see hipGetLastError) */
+#define Q4_ERR_MISALIGNED (-5)     /* a pointer is not 16-byte aligned */
+
+/* Library ABI version (bumped when a signature changes). */
+int q4_abi_version(void);
+
+/* Static string for a return code. */
+const char *q4_error_string(int code);
+
+/* Dense dequantization: out fp16 [K, N] = W.
+ * Replaces quant_cuda.vecquant4recons_v2(mat, res, scales, zeros, g_idx)
+ * (quant_cuda/quant_cuda.cpp:137-148, kernel quant_cuda/quant_cuda_kernel.cu:1127-1183).
+ * Bit-exact with that kernel's fp16 instantiation. */
+int q4_dequant_f16(const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                   const int32_t *g_idx, int groupsize, void *out,
+                   int K, int N, int G, void *stream);
+
+/* Decode GEMV / skinny GEMM, 1 <= M <= 16:  y fp16 [M, N] = x fp16 [M, K] @ W  (fp32 accumulate).
+ * If accumulate != 0 the product is added to the existing contents of y.
+ * Replaces quant_cuda.vecquant4matmul / vecquant4matmul_faster / vecquant4matmul_old_faster
+ * (quant_cuda/quant_cuda.cpp:55-61, 93-113; kernels quant_cuda_kernel.cu:443-536, 874-1073)
+ * as dispatched by matmul_utils_4bit.py:59-95.  g_idx == NULL selects sequential groups of
+ * `groupsize` rows (the old_faster convention, quant_cuda_kernel.cu:1024); otherwise rows are
+ * gathered through g_idx (the vecquant4matmul convention, :513-520).
+ * `workspace` must hold q4_gemv_workspace_bytes(M, K, N) bytes, 256-byte aligned, and must be
+ * ZERO before its first use; every call leaves it zeroed again.  Calls sharing one workspace
+ * must be ordered on one stream. */
+size_t q4_gemv_workspace_bytes(int M, int K, int N);
+int q4_gemv_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                const int32_t *g_idx, int groupsize, void *y, int accumulate,
+                int M, int K, int N, int G,
+                void *workspace, size_t workspace_bytes, void *stream);
+
+/* Forward GEMM, any M >= 1:
+ *   y fp16 [M, N] = x fp16 [M, K] @ W  (+ bias fp16 [N])  (+ xa fp16 [M, R] @ lora_bt fp16 [R, N])
+ * with fp32 accumulation on MFMA; W tiles are dequantized in LDS and never written to HBM.
+ * Replaces vecquant4recons_v2 + torch.matmul(x, buffer) (matmul_utils_4bit.py:114-124),
+ * the bias add (autograd_4bit.py:206-207) and, when xa/lora_bt are given, the adapter term
+ * result += lora_B(lora_A(x)) * scaling (models.py:58-66) where xa = scaling * x @ A^T and
+ * lora_bt = B^T.  bias, xa, lora_bt may be NULL; R is 0 or a multiple of 8, at most 64. */
+int q4_gemm_fwd_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                    const int32_t *g_idx, int groupsize, const void *bias,
+                    const void *xa, const void *lora_bt, int R,
+                    void *y, int M, int K, int N, int G, void *stream);
+
+/* Backward GEMM (grad of the input):
+ *   dx fp16 [M, K] = dy fp16 [M, N] @ W^T  (+ dyb fp16 [M, R] @ lora_a fp16 [R, K])
+ * Replaces vecquant4recons_v2 + torch.matmul(grad_output, buffer.T)
+ * (matmul_utils_4bit.py:114-126 with transpose=True, called from autograd_4bit.py:53) and the
+ * adapter's contribution to grad_input, with dyb = scaling * dy @ B and lora_a = A. */
+int q4_gemm_bwd_dx_f16(const void *dy, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                       const int32_t *g_idx, int groupsize,
+                       const void *dyb, const void *lora_a, int R,
+                       void *dx, int M, int K, int N, int G, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* Q4_GPTQ_H */

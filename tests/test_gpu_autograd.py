@@ -1,0 +1,165 @@
+"""Module-level parity: Autograd4bitQuantLinear / AutogradMatmul4bit / Linear4bitLt against
+(i) the CPU oracle and (ii) torch autograd through a dense nn.Linear holding the oracle's W."""
+import numpy as np
+import pytest
+
+from conftest import rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def _fill(module, layer):
+    import torch
+    module.qweight = torch.from_numpy(layer["qweight"]).cuda()
+    module.qzeros = torch.from_numpy(layer["qzeros"]).cuda()
+    module.scales = torch.from_numpy(layer["scales"]).cuda()
+    module.g_idx = torch.from_numpy(layer["g_idx"]).cuda()
+    module.bias = torch.zeros(layer["N"], dtype=torch.float16, device="cuda")
+    return module
+
+
+@pytest.mark.parametrize("act", [False, True])
+@pytest.mark.parametrize("shape", [(1, 1), (2, 4), (1, 16), (3, 40), (8, 256)])
+def test_quant_linear_forward_both_modes(oracle, shape, act):
+    """[batch, seq, K] inputs; no-grad (dispatcher) and grad mode (autograd Function) agree with
+    the oracle; leading dimensions are preserved (autograd_4bit.py:192-208)."""
+    import torch
+    from alpaca_lora_4bit_amd.autograd_4bit import Autograd4bitQuantLinear
+    K, N = 512, 384
+    layer = oracle.make_layer(K, N, 128, act_order=act, seed=13)
+    m = _fill(Autograd4bitQuantLinear(K, N, groupsize=128), layer)
+    rng = np.random.default_rng(5)
+    bias = (rng.standard_normal(N) * 0.1).astype(np.float16)
+    m.bias = torch.from_numpy(bias).cuda()
+    x = oracle.make_activations(shape[0] * shape[1], K, seed=3).reshape(shape[0], shape[1], K)
+    ref = oracle.matmul_recons(x.reshape(-1, K), layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
+    ref = (ref + bias.astype(np.float32)).reshape(shape[0], shape[1], N)
+    xt = torch.from_numpy(x).cuda()
+    with torch.no_grad():
+        y0 = m(xt)
+    y1 = m(xt.clone().requires_grad_(True))
+    assert y0.shape == (shape[0], shape[1], N) and y0.dtype == torch.float16
+    assert rel_err(y0.cpu().numpy(), ref) <= TOL
+    assert rel_err(y1.detach().cpu().numpy(), ref) <= TOL
+    m.disable_bias = True
+    with torch.no_grad():
+        y2 = m(xt)
+    assert rel_err(y2.cpu().numpy(), ref - bias.astype(np.float32)) <= TOL
+
+
+@pytest.mark.parametrize("rows", [4, 64])
+def test_autograd_matches_dense_linear(oracle, rows):
+    """dx from AutogradMatmul4bit.backward == dx of a dense fp32 nn.Linear built from W_ref;
+    the six non-input gradients are None (autograd_4bit.py:54)."""
+    import torch
+    from alpaca_lora_4bit_amd import autograd_4bit
+    K, N = 256, 384
+    layer = oracle.make_layer(K, N, 128, seed=17)
+    W = oracle.dequant_v2(layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
+    dense = torch.nn.Linear(K, N, bias=False).cuda()
+    dense.weight.data = torch.from_numpy(W.astype(np.float32)).cuda().t().contiguous()
+    x = torch.from_numpy(oracle.make_activations(rows, K, seed=1)).cuda()
+    dy = torch.from_numpy(oracle.make_activations(rows, N, seed=2)).cuda()
+
+    xq = x.clone().requires_grad_(True)
+    t = {k: torch.from_numpy(layer[k]).cuda() for k in ("qweight", "qzeros", "scales", "g_idx")}
+    y = autograd_4bit.AutogradMatmul4bit.apply(xq, t["qweight"], t["scales"], t["qzeros"], t["g_idx"], 4, 15)
+    y.backward(dy)
+    xd = x.float().clone().requires_grad_(True)
+    yd = dense(xd)
+    yd.backward(dy.float())
+    assert rel_err(y.detach().cpu().numpy(), yd.detach().cpu().numpy()) <= TOL
+    assert rel_err(xq.grad.cpu().numpy(), xd.grad.cpu().numpy()) <= TOL
+    assert xq.grad.dtype == torch.float16
+
+
+def test_autocast_casts_fp32_inputs(oracle):
+    """Under autocast custom_fwd(cast_inputs=fp16) casts x and scales (autograd_4bit.py:35)."""
+    import torch
+    from alpaca_lora_4bit_amd.autograd_4bit import Autograd4bitQuantLinear
+    K, N = 256, 128
+    layer = oracle.make_layer(K, N, 128, seed=19)
+    m = _fill(Autograd4bitQuantLinear(K, N, groupsize=128), layer)
+    x = oracle.make_activations(32, K, seed=4)
+    ref = oracle.matmul_recons(x, layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
+    xt = torch.from_numpy(x).cuda().float().requires_grad_(True)
+    with torch.amp.autocast(device_type="cuda"):
+        y = m(xt)
+    assert y.dtype == torch.float16
+    assert rel_err(y.detach().cpu().numpy(), ref) <= TOL
+    y.float().sum().backward()
+    assert xt.grad is not None and xt.grad.dtype == torch.float32
+
+
+@pytest.mark.parametrize("act", [False, True])
+@pytest.mark.parametrize("rows,K,N,r", [(2048, 4096, 4096, 8), (96, 256, 384, 16), (4, 256, 128, 8)])
+def test_linear4bitlt_forward_backward(oracle, rows, K, N, r, act):
+    """Linear4bitLt (fused path for rows > 16, reference composition otherwise) vs the closed-form
+    oracle: y, dx, dA, dB.  Config 2 is the first parameter set."""
+    import torch
+    from alpaca_lora_4bit_amd import models
+    layer = oracle.make_layer(K, N, 128, act_order=act, seed=23)
+    A, B = oracle.make_lora(K, N, r, seed=23)
+    m = models.Linear4bitLt("default", K, N, 128, False, r=r, lora_alpha=2 * r, lora_dropout=0.0).cuda()
+    _fill(m, layer)
+    m.lora_A["default"].weight.data = torch.from_numpy(A).cuda()
+    m.lora_B["default"].weight.data = torch.from_numpy(B).cuda()
+    assert m.scaling["default"] == 2.0
+    x = oracle.make_activations(rows, K, seed=51)
+    dy = oracle.make_activations(rows, N, seed=52)
+    W = oracle.dequant_v2(layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"]).astype(np.float64)
+    yref = oracle.lora_forward(x, W, A, B, 2.0)
+    dxref, dAref, dBref = oracle.lora_backward(x, dy, W, A, B, 2.0)
+
+    xt = torch.from_numpy(x).cuda().requires_grad_(True)
+    with torch.amp.autocast(device_type="cuda"):
+        y = m(xt)
+    y.backward(torch.from_numpy(dy).cuda())
+    assert y.dtype == torch.float16 and y.shape == (rows, N)
+    assert rel_err(y.detach().cpu().numpy(), yref) <= TOL
+    assert rel_err(xt.grad.cpu().numpy(), dxref) <= TOL
+    gA, gB = m.lora_A["default"].weight.grad, m.lora_B["default"].weight.grad
+    assert gA.dtype == torch.float32 and gB.dtype == torch.float32
+    assert rel_err(gA.cpu().numpy(), dAref) <= TOL
+    assert rel_err(gB.cpu().numpy(), dBref) <= TOL
+    assert m.qweight.grad is None and m.scales.grad is None
+
+
+def test_fused_and_unfused_lora_agree(oracle):
+    import torch
+    from alpaca_lora_4bit_amd import models
+    K, N, r, rows = 512, 256, 8, 160
+    layer = oracle.make_layer(K, N, 128, seed=29)
+    A, B = oracle.make_lora(K, N, r, seed=29)
+    m = models.Linear4bitLt("default", K, N, 128, False, r=r, lora_alpha=16).cuda()
+    _fill(m, layer)
+    m.lora_A["default"].weight.data = torch.from_numpy(A).cuda()
+    m.lora_B["default"].weight.data = torch.from_numpy(B).cuda()
+    x = torch.from_numpy(oracle.make_activations(rows, K, seed=6)).cuda()
+    outs = []
+    for fuse in (True, False):
+        models.fuse_lora = fuse
+        try:
+            xt = x.clone().requires_grad_(True)
+            with torch.amp.autocast(device_type="cuda"):
+                y = m(xt)
+            y.float().square().sum().backward()
+            outs.append((y.detach().float().cpu().numpy(), xt.grad.float().cpu().numpy(),
+                         m.lora_A["default"].weight.grad.clone().cpu().numpy(),
+                         m.lora_B["default"].weight.grad.clone().cpu().numpy()))
+            m.zero_grad()
+        finally:
+            models.fuse_lora = True
+    for a, b in zip(*outs):
+        assert rel_err(a, b) <= TOL
+
+
+def test_backend_switch_and_errors():
+    from alpaca_lora_4bit_amd import autograd_4bit
+    autograd_4bit.switch_backend_to("cuda")
+    assert autograd_4bit.backend == "cuda"
+    with pytest.raises(ValueError):
+        autograd_4bit.switch_backend_to("triton")
+    with pytest.raises(ValueError):
+        autograd_4bit.switch_backend_to("metal")
