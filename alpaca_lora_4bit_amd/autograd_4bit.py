@@ -237,12 +237,12 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
         if scaling != 1.0:
             xa = xa * scaling
         y = quant_hip.gemm_fwd(x2, qweight, zeros, scales, g_idx, groupsize, bias=bias,
-                               xa=xa, lora_bt=b16.t().contiguous())
+                               xa=xa, lora_bt=b16.t().contiguous(), out_shape=tuple(x.shape[:-1]) + (N,))
         ctx.save_for_backward(x2, xa, qweight, scales, zeros, g_idx, a16, b16)
         ctx.scaling = scaling
         ctx.groupsize = groupsize
         ctx.ab_dtypes = (lora_a.dtype, lora_b.dtype)
-        return y.reshape(x.shape[:-1] + (N,))
+        return y
 
     @staticmethod
     @custom_bwd(device_type='cuda')
@@ -258,8 +258,8 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
             dyb = dyb * ctx.scaling
         dx = da = db = None
         if ctx.needs_input_grad[0]:
-            dx = quant_hip.gemm_bwd_dx(dy, qweight, zeros, scales, g_idx, ctx.groupsize, dyb=dyb, lora_a=a16)
-            dx = dx.reshape(grad_output.shape[:-1] + (dx.shape[-1],))
+            dx = quant_hip.gemm_bwd_dx(dy, qweight, zeros, scales, g_idx, ctx.groupsize, dyb=dyb, lora_a=a16,
+                                       out_shape=tuple(grad_output.shape[:-1]) + (qweight.shape[0] * 8,))
         if ctx.needs_input_grad[6]:
             da = torch.matmul(dyb.t(), x2).to(ctx.ab_dtypes[0])
         if ctx.needs_input_grad[7]:

@@ -7,7 +7,7 @@
 extern "C" {
 int q4_launch_dequant(const int32_t*, const int32_t*, const void*, const int32_t*, int, void*, int, int, hipStream_t);
 int q4_launch_gemv(const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, void*, int,
-                   int, int, int, void*, hipStream_t);
+                   int, int, int, int, void*, hipStream_t);
 int q4_launch_gemm(int, const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, const void*,
                    const void*, const void*, int, void*, int, int, int, hipStream_t);
 }
@@ -59,11 +59,11 @@ extern "C" int q4_gemv_f16(const void* x, const int32_t* qweight, const int32_t*
     int rc = check_layer(qweight, qzeros, scales, g_idx, groupsize, K, N, G);
     if (rc != Q4_OK) return rc;
     if (!x || !y) return Q4_ERR_NULL_POINTER;
-    if (M < 1 || M > 16 || N > 262144) return Q4_ERR_BAD_SHAPE;
+    if (M < 1 || M > 16 || K > 32 * 255 * 8 * 16) return Q4_ERR_BAD_SHAPE;
     if (misaligned(x) || misaligned(y)) return Q4_ERR_MISALIGNED;
     if (!workspace || workspace_bytes < q4_gemv_workspace_bytes(M, K, N)) return Q4_ERR_WORKSPACE;
     if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
-    return q4_launch_gemv(x, qweight, qzeros, scales, g_idx, groupsize, y, accumulate, M, K, N, workspace,
+    return q4_launch_gemv(x, qweight, qzeros, scales, g_idx, groupsize, y, accumulate, M, K, N, G, workspace,
                           (hipStream_t)stream);
 }
 

@@ -69,8 +69,9 @@ def _matmul4bit_v2(x, qweight, scales, zeros, g_idx, groupsize=None):
         raise ValueError('faster_mode should be in {}'.format(valid_faster_mode))
     outshape = x.shape[:-1] + (qweight.shape[1],)
     dtype = x.dtype
-    y = quant_hip.gemv(x, qweight, zeros, _half_scales(scales), g_idx, _groupsize_of(qweight, scales, groupsize))
-    return y.to(dtype).reshape(outshape)
+    y = quant_hip.gemv(x, qweight, zeros, _half_scales(scales), g_idx, _groupsize_of(qweight, scales, groupsize),
+                       out_shape=outshape)
+    return y.to(dtype)
 
 
 def _matmul4bit_v2_recons(x, qweight, scales, zeros, g_idx, transpose=False, groupsize=None):
@@ -83,12 +84,12 @@ def _matmul4bit_v2_recons(x, qweight, scales, zeros, g_idx, transpose=False, gro
     else:
         assert qweight.shape[1] == x.shape[-1]
     gs = _groupsize_of(qweight, scales, groupsize)
-    lead = x.shape[:-1]
+    lead = tuple(x.shape[:-1])
     if not transpose:
-        out = quant_hip.gemm_fwd(x, qweight, zeros, _half_scales(scales), g_idx, gs)
-    else:
-        out = quant_hip.gemm_bwd_dx(x, qweight, zeros, _half_scales(scales), g_idx, gs)
-    return out.reshape(lead + (out.shape[-1],))
+        return quant_hip.gemm_fwd(x, qweight, zeros, _half_scales(scales), g_idx, gs,
+                                  out_shape=lead + (qweight.shape[1],))
+    return quant_hip.gemm_bwd_dx(x, qweight, zeros, _half_scales(scales), g_idx, gs,
+                                 out_shape=lead + (qweight.shape[0] * 8,))
 
 
 def _v1_unsupported(*args, **kwargs):

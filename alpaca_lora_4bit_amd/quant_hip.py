@@ -100,6 +100,18 @@ def _workspace(device, nbytes):
     return ws
 
 
+def _out_shape(out_shape, rows, cols):
+    if out_shape is None:
+        return (rows, cols)
+    out_shape = tuple(out_shape)
+    n = 1
+    for d in out_shape:
+        n *= d
+    _require(len(out_shape) >= 1 and out_shape[-1] == cols and n == rows * cols,
+             f"out_shape {out_shape} does not hold {rows} rows of {cols}")
+    return out_shape
+
+
 def _flat_half(x, K, dev, what):
     _require(x.is_cuda and x.device == dev, f"{what} must be on {dev}")
     _require(x.shape[-1] == K, f"{what} last dimension {x.shape[-1]} != {K}")
@@ -125,17 +137,18 @@ def dequant(qweight, qzeros, scales, g_idx=None, groupsize=None, out=None):
     return out
 
 
-def gemv(x, qweight, qzeros, scales, g_idx=None, groupsize=None, out=None, accumulate=False):
-    """y fp16 [M, N] = x [M, K] @ W for M <= 16 (decode)."""
+def gemv(x, qweight, qzeros, scales, g_idx=None, groupsize=None, out=None, accumulate=False, out_shape=None):
+    """y fp16 [M, N] = x [M, K] @ W for M <= 16 (decode).  `out_shape` (same number of elements)
+    lets the result be allocated with the caller's leading dimensions instead of being a view."""
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     x2 = _flat_half(x, K, dev, "x")
     M = x2.shape[0]
     _require(1 <= M <= MAX_GEMV_ROWS, f"gemv handles 1..{MAX_GEMV_ROWS} rows, got {M}")
     if out is None:
         _require(not accumulate, "accumulate needs an output tensor")
-        out = torch.empty((M, N), dtype=torch.float16, device=dev)
-    _require(out.dtype == torch.float16 and tuple(out.shape) == (M, N) and out.is_contiguous() and out.device == dev,
-             "out must be a contiguous float16 [M, N] tensor on the same device")
+        out = torch.empty(_out_shape(out_shape, M, N), dtype=torch.float16, device=dev)
+    _require(out.dtype == torch.float16 and out.numel() == M * N and out.shape[-1] == N and out.is_contiguous()
+             and out.device == dev, "out must be a contiguous float16 [..., N] tensor with M rows on the same device")
     gp, gs = _gidx_arg(g_idx, groupsize, G)
     L = _lib.lib()
     nbytes = L.q4_gemv_workspace_bytes(M, K, N)
@@ -160,7 +173,8 @@ def _lora_pair(la, lb, rows, cols, dev):
     return la, lb, R
 
 
-def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, xa=None, lora_bt=None):
+def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, xa=None, lora_bt=None,
+             out_shape=None):
     """y fp16 [M, N] = x @ W (+ bias) (+ xa @ lora_bt), W dequantized tile by tile in LDS."""
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     x2 = _flat_half(x, K, dev, "x")
@@ -170,7 +184,7 @@ def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, 
                  and bias.device == dev, "bias must be a contiguous float16 [N] tensor on the same device")
     xa, lora_bt, R = _lora_pair(xa, lora_bt, M, N, dev)
     gp, gs = _gidx_arg(g_idx, groupsize, G, need_multiple=64)
-    out = torch.empty((M, N), dtype=torch.float16, device=dev)
+    out = torch.empty(_out_shape(out_shape, M, N), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().q4_gemm_fwd_f16(x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
                                         gp, gs, _ptr(bias), _ptr(xa), _ptr(lora_bt), R,
@@ -179,14 +193,14 @@ def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, 
     return out
 
 
-def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=None, lora_a=None):
+def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=None, lora_a=None, out_shape=None):
     """dx fp16 [M, K] = dy [M, N] @ W^T (+ dyb @ lora_a)."""
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     dy2 = _flat_half(dy, N, dev, "grad_output")
     M = dy2.shape[0]
     dyb, lora_a, R = _lora_pair(dyb, lora_a, M, K, dev)
     gp, gs = _gidx_arg(g_idx, groupsize, G, need_multiple=64)
-    out = torch.empty((M, K), dtype=torch.float16, device=dev)
+    out = torch.empty(_out_shape(out_shape, M, K), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().q4_gemm_bwd_dx_f16(dy2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
                                            gp, gs, _ptr(dyb), _ptr(lora_a), R,
