@@ -9,7 +9,7 @@ int q4_launch_dequant(const int32_t*, const int32_t*, const void*, const int32_t
 int q4_launch_gemv(const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, void*, int,
                    int, int, int, int, void*, hipStream_t);
 int q4_launch_gemm(int, const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, const void*,
-                   const void*, const void*, int, void*, int, int, int, hipStream_t);
+                   const void*, const void*, int, void*, int, int, int, int, hipStream_t);
 }
 
 namespace {
@@ -75,11 +75,14 @@ static int gemm_common(int fwd, const void* act, const int32_t* qweight, const i
     if (!act || !out) return Q4_ERR_NULL_POINTER;
     if (M < 1 || (K % 128) != 0 || (N % 128) != 0) return Q4_ERR_BAD_SHAPE;
     if (!g_idx && (groupsize % 64) != 0) return Q4_ERR_BAD_SHAPE;
+    // the kernels address the packed weights through 32-bit buffer offsets
+    if ((unsigned long long)(K / 8) * (unsigned long long)N * 4ull >= (1ull << 32)) return Q4_ERR_BAD_SHAPE;
+    if ((unsigned long long)(K > N ? K : N) * 512ull >= (1ull << 32)) return Q4_ERR_BAD_SHAPE;
     if ((la != nullptr) != (lb != nullptr)) return Q4_ERR_NULL_POINTER;
     if (la && (R < 8 || R > 64 || (R % 8) != 0)) return Q4_ERR_BAD_SHAPE;
     if (misaligned(act) || misaligned(out) || (la && misaligned(la)) || (lb && misaligned(lb)))
         return Q4_ERR_MISALIGNED;
-    return q4_launch_gemm(fwd, act, qweight, qzeros, scales, g_idx, groupsize, bias, la, lb, R, out, M, K, N,
+    return q4_launch_gemm(fwd, act, qweight, qzeros, scales, g_idx, groupsize, bias, la, lb, R, out, M, K, N, G,
                           (hipStream_t)stream);
 }
 

@@ -6,22 +6,40 @@
 // (src/alpaca_lora_4bit/quant_cuda/quant_cuda_kernel.cu:1146-1151), so the product equals
 // torch.matmul(x, recons(W)) of matmul_utils_4bit.py:122-126 up to fp32 summation order.
 //
-// Tiling.  Workgroup = 256 threads = 4 wavefronts in a 2 x 2 arrangement over a 128 x 128
-// output tile; each wavefront holds 2 x 2 accumulators of v_mfma_f32_32x32x16_f16 (64 fp32
-// registers per lane).  The reduction runs in steps of 64.  Both LDS tiles are stored
-// "row = output index, minor = reduction index" with 8 halves of padding per row (stride
-// 144 B), which makes the 128-bit operand fetches of 16 consecutive lanes hit 64 distinct banks.
-// Global loads of step t+1 are issued before the MFMAs of step t and land in registers.
+// Tiling.  A workgroup computes a BM x 128 output tile with 2*WGM wavefronts (WGM along M, 2
+// along N), each owning (BM/WGM) x 64 outputs as (BM/WGM/32) x 2 accumulators of
+// v_mfma_f32_32x32x16_f16.  Large problems use BM = 256 with 8 wavefronts of 64 x 64 (two per SIMD:
+// while one waits or dequantizes the other multiplies, and one dequantized slab of W serves 256
+// activation rows); problems with fewer than ~200 such tiles use BM = 128 with 4 wavefronts so that
+// every CU still gets a workgroup.  The reduction runs in steps of 64.  Both LDS tiles are stored "row = output index, minor = reduction index" with 8 halves of
+// padding per row (stride 144 B): the 128-bit operand fetches of 16 consecutive lanes then hit
+// 64 distinct banks.  LDS is double buffered in four distinct arrays (110 KB at BM = 256).
+//
+// Pipeline (hand-scheduled; with one or two wavefronts per SIMD little else hides a stall):
+//   * global loads of stage s+2 go to a second register set through buffer instructions whose
+//     per-thread offsets are computed once (zero address arithmetic in the loop; rows beyond M
+//     fall outside the buffer descriptor and read as zero);
+//   * the registers of stage s+1 are dequantized into the other LDS buffer in 16 small slices;
+//   * each of the 16 MFMAs of stage s is followed by one such slice / load batch / LDS
+//     store and a scheduling barrier that pins the interleaving, since an MFMA keeps the matrix
+//     pipe busy for 8 passes during which the wavefront may issue other instructions;
+//   * the workgroup barrier sits a few MFMAs before the end of the step and the first operand
+//     fragments of stage s+1 are fetched right after it, under the remaining MFMAs.
 //
 // The LoRA term is one more reduction step whose A operand is the precomputed [M,R] rank-R
 // activation and whose B operand is the fp16 adapter matrix: no second pass over the output.
+// The epilogue transposes the accumulators through LDS so that y is written in 16-byte pieces.
 #include "q4_common.hpp"
+#include <stdlib.h>
 #include <type_traits>
 
 namespace q4 {
 
-constexpr int BM = 128, BN = 128, BK = 64;
+constexpr int BN = 128, BK = 64;
 constexpr int LDS_STRIDE = BK + 8;   // halves
+constexpr int kRsrcFlags = 0x00020000;
+
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
 
 struct GemmArgs {
     const half_t* a;          // fwd: x [M,K]      bwd: dy [M,N]
@@ -35,58 +53,126 @@ struct GemmArgs {
     const half_t* lb;         // fwd: lora_bt [R,N] bwd: lora_a [R,K]
     int R;
     half_t* out;              // fwd: y [M,N]      bwd: dx [M,K]
-    int M, K, N;
+    int M, K, N, G;
+};
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, kRsrcFlags);
+}
+__device__ __forceinline__ uint4_t buf_load128(rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
+__device__ __forceinline__ uint2_t buf_load64(rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
+}
+__device__ __forceinline__ uint32_t buf_load32(rsrc_t r, int voff, int soff) {
+    return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+}
+__device__ __forceinline__ uint32_t buf_load16(rsrc_t r, int voff, int soff) {
+    return (uint32_t)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0);
+}
+
+// rn16(rn16(s*q) - zero) for a pair of codes given as (0x6400 | q): one fused multiply-add
+// computes s*(1024+q) - 1024*s = s*q with a single rounding (1024*s is exact), i.e. exactly
+// rn16(s*q); the subtraction of the zero term is the third rounding.  Needs |s| < 64 so that
+// 1024*s does not overflow (checked on the host; larger scales take the unfused path).
+__device__ __forceinline__ half2_t dequant_pair_magic(uint32_t codes_or_magic, half2_t s, half2_t s1024, half2_t zero) {
+    const half2_t p = __builtin_elementwise_fma(as_half2(codes_or_magic), s, -s1024);
+    return p - zero;
+}
+
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+struct SlabRsrc {
+    rsrc_t w, s, z;
 };
 
 // ---- weight slab loaders: global -> registers -> (dequant) -> LDS ----------------------
+// The dequantization of a slab is cut into kSlices = 16 pieces so that the main loop can hand
+// the vector ALU one piece between two MFMAs.  With GIDX (act-order, or scales too large for
+// the fused form) rows gather (scale, zero) through g_idx and everything happens in piece 0.
+//
 // Forward: slab = 64 rows (k) x 128 columns (n); LDS row = column n, minor = k.
-// A thread owns ONE column for the whole kernel and 4 packed words (32 rows) per step.
-template <bool GIDX>
+// A thread owns ONE column for the whole kernel and 4 packed words (32 rows) per step;
+// piece I handles pair I%4 of word I/4 and the word goes to LDS with its last piece.
+template <bool GIDX, int NT>
 struct FwdSlab {
-    uint32_t w[4];
-    int col;        // 0..127 within the tile
-    int wr0;        // first word-row within the slab (0 or 1), then +2 per word
-    __device__ __forceinline__ void init(int t) { col = t & 127; wr0 = t >> 7; }
-    __device__ __forceinline__ void load(const GemmArgs& a, int n0, int kred0) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            w[i] = a.qweight[(size_t)((kred0 >> 3) + wr0 + 2 * i) * a.N + n0 + col];
+    static constexpr int NW = 1024 / NT;          // packed words per thread per step (4 or 2)
+    static constexpr int WSTEP = NT / 128;        // word-row distance between a thread's words
+    static constexpr int kSlices = 4 * NW;
+    uint32_t w[NW];
+    uint32_t s_raw;  // fp16 bits of the scale of (current group, own column); decoded in the slices
+    uint32_t z_raw;  // packed zero word holding the own column's code
+    uint32_t o[4];
+    int col, wr0;    // column 0..127 of the tile; first word-row within the slab, then +WSTEP per word
+    int voff_w, voff_s, voff_z, wstride;
+    __device__ __forceinline__ void init(int t, const GemmArgs& a, int n0) {
+        col = t & 127; wr0 = t >> 7;
+        wstride = WSTEP * a.N * 4;
+        voff_w = (wr0 * a.N + n0 + col) * 4;
+        voff_s = (n0 + col) * 2;
+        voff_z = ((n0 + col) >> 3) * 4;
     }
-    __device__ __forceinline__ void store(const GemmArgs& a, int n0, int kred0, half_t* sB) const {
-        const int n = n0 + col;
-        const int ncol8 = a.N >> 3;
-        const int zsh = (n & 7) * 4;
-        half2_t s2, zero2;
+    // raw loads only: any arithmetic on the loaded values here would wait for them before the MFMAs
+    __device__ __forceinline__ void load(const GemmArgs& a, const SlabRsrc& r, int, int kred0) {
+        const int soff = (kred0 >> 3) * a.N * 4;
+#pragma unroll
+        for (int i = 0; i < NW; ++i) w[i] = buf_load32(r.w, voff_w + i * wstride, soff);
         if (!GIDX) {
             const int g = kred0 / a.groupsize;
-            const half_t s = a.scales[(size_t)g * a.N + n];
-            const uint32_t z = (a.qzeros[(size_t)g * ncol8 + (n >> 3)] >> zsh) & 0xFu;
-            s2 = half2_t{s, s};
-            zero2 = zero_term(s2, z, z);
+            s_raw = buf_load16(r.s, voff_s, g * a.N * 2);
+            z_raw = buf_load32(r.z, voff_z, g * (a.N >> 3) * 4);
         }
+    }
+    template <int I>
+    __device__ __forceinline__ void store_slice(const GemmArgs& a, int n0, int kred0, half_t* sB) {
+        const int n = n0 + col;
+        if constexpr (GIDX) {
+            if constexpr (I == 0) {
+                const int ncol8 = a.N >> 3;
+                const int zsh = (n & 7) * 4;
+                const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int wr = wr0 + 2 * i;
-            half2_t q2[4];
-            unpack8_natural(w[i], q2);
-            uint32_t o[4];
+                for (int i = 0; i < NW; ++i) {
+                    const int wr = wr0 + WSTEP * i;
+                    const uint32_t lo = w[i] & 0x0F0F0F0Fu, hi = (w[i] >> 4) & 0x0F0F0F0Fu;
+                    uint32_t oo[4];
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                if (GIDX) {
-                    const int k = kred0 + 8 * wr + 2 * p;
-                    const int g0 = a.g_idx[k], g1 = a.g_idx[k + 1];
-                    s2 = half2_t{a.scales[(size_t)g0 * a.N + n], a.scales[(size_t)g1 * a.N + n]};
-                    zero2 = zero_term(s2, (a.qzeros[(size_t)g0 * ncol8 + (n >> 3)] >> zsh) & 0xFu,
-                                      (a.qzeros[(size_t)g1 * ncol8 + (n >> 3)] >> zsh) & 0xFu);
+                    for (int p = 0; p < 4; ++p) {
+                        const uint32_t codes = __builtin_amdgcn_perm(hi, lo, 0x0c040c00u + 0x00010001u * p) | kMagic;
+                        const int k = kred0 + 8 * wr + 2 * p;
+                        const int g0 = a.g_idx[k], g1 = a.g_idx[k + 1];
+                        const half2_t s2 = {a.scales[(size_t)g0 * a.N + n], a.scales[(size_t)g1 * a.N + n]};
+                        const half2_t zero2 = zero_term(s2, (a.qzeros[(size_t)g0 * ncol8 + (n >> 3)] >> zsh) & 0xFu,
+                                                        (a.qzeros[(size_t)g1 * ncol8 + (n >> 3)] >> zsh) & 0xFu);
+                        oo[p] = as_u32(dequant_pair(as_half2(codes) - k1024, s2, zero2));
+                    }
+                    *reinterpret_cast<uint4_t*>(sB + col * LDS_STRIDE + 8 * wr) = uint4_t{oo[0], oo[1], oo[2], oo[3]};
                 }
-                o[p] = as_u32(dequant_pair(q2[p], s2, zero2));
             }
-            *reinterpret_cast<uint4_t*>(sB + col * LDS_STRIDE + 8 * wr) = uint4_t{o[0], o[1], o[2], o[3]};
+        } else {
+            constexpr int i = I / 4, p = I % 4;
+            const half2_t s2 = as_half2(s_raw | (s_raw << 16));
+            const uint32_t z_cur = (z_raw >> ((n & 7) * 4)) & 0xFu;
+            const half2_t zero2 = zero_term(s2, z_cur, z_cur);
+            const half2_t s1024 = s2 * half2_t{(half_t)1024.f, (half_t)1024.f};
+            const uint32_t lo = w[i] & 0x0F0F0F0Fu;          // bytes e0 e2 e4 e6
+            const uint32_t hi = (w[i] >> 4) & 0x0F0F0F0Fu;   // bytes e1 e3 e5 e7
+            const uint32_t codes = __builtin_amdgcn_perm(hi, lo, 0x0c040c00u + 0x00010001u * p) | kMagic;
+            o[p] = as_u32(dequant_pair_magic(codes, s2, s1024, zero2));
+            if constexpr (p == 3)
+                *reinterpret_cast<uint4_t*>(sB + col * LDS_STRIDE + 8 * (wr0 + WSTEP * i)) = uint4_t{o[0], o[1], o[2], o[3]};
         }
     }
     // LoRA step: B operand = lora_bt [R, N]; LDS row = column n, minor = r (zero padded to 64).
     __device__ __forceinline__ void store_lora(const GemmArgs& a, int n0, half_t* sB, int t) const {
-        for (int idx = t; idx < BN * BK; idx += 256) {
+        for (int idx = t; idx < BN * BK; idx += NT) {
             const int r = idx >> 7, c = idx & 127;
             sB[c * LDS_STRIDE + r] = (r < a.R) ? a.lb[(size_t)r * a.N + n0 + c] : (half_t)0.f;
         }
@@ -96,48 +182,84 @@ struct FwdSlab {
 // Backward: output columns are rows k of W, the reduction runs over n.
 // Slab = 128 rows (k) x 64 columns (n); LDS row = k, minor = n.
 // A thread owns one word-row (8 output rows) and 4 adjacent columns per step (one 128-bit load).
-template <bool GIDX>
+// With 512 threads two threads share a load and split the word-row's 8 rows 4 + 4.
+// Piece I dequantizes columns (0,1) [I even] or (2,3) [I odd] of the thread's row I/2; the
+// 8-byte row segment goes to LDS with the odd piece.
+template <bool GIDX, int NT>
 struct BwdSlab {
+    static constexpr int RPT = 8 * 256 / NT;      // rows of the word-row handled by one thread (8 or 4)
+    static constexpr int kSlices = 2 * RPT;
     uint4_t w;
-    int wr, n4;
-    __device__ __forceinline__ void init(int t) { wr = t >> 4; n4 = t & 15; }
-    __device__ __forceinline__ void load(const GemmArgs& a, int kout0, int nred0) {
-        w = *reinterpret_cast<const uint4_t*>(a.qweight + (size_t)((kout0 >> 3) + wr) * a.N + nred0 + 4 * n4);
+    uint2_t sv;
+    uint32_t zw, o01;
+    int wr, n4, e0;
+    int voff_w, voff_s, voff_z;
+    __device__ __forceinline__ void init(int t, const GemmArgs& a, int kout0) {
+        wr = (t & 255) >> 4; n4 = t & 15; e0 = (t >> 8) * RPT;
+        const int g = GIDX ? 0 : (kout0 + 8 * wr) / a.groupsize;      // fixed for the whole kernel
+        voff_w = (((kout0 >> 3) + wr) * a.N + 4 * n4) * 4;
+        voff_s = (g * a.N + 4 * n4) * 2;
+        voff_z = (g * (a.N >> 3) + (n4 >> 1)) * 4;
     }
-    __device__ __forceinline__ void store(const GemmArgs& a, int kout0, int nred0, half_t* sB) const {
+    __device__ __forceinline__ void load(const GemmArgs&, const SlabRsrc& r, int, int nred0) {
+        w = buf_load128(r.w, voff_w, nred0 * 4);
+        if (!GIDX) {
+            sv = buf_load64(r.s, voff_s, nred0 * 2);
+            zw = buf_load32(r.z, voff_z, (nred0 >> 3) * 4);       // shifted in the slices: no ALU on loaded data here
+        }
+    }
+    template <int I>
+    __device__ __forceinline__ void store_slice(const GemmArgs& a, int kout0, int nred0, half_t* sB) {
         const int n = nred0 + 4 * n4;
-        const int ncol8 = a.N >> 3;
-        const int zsh = (n & 7) * 4;    // 0 or 16
-        const int kbase = kout0 + 8 * wr;
-        const uint32_t wj[4] = {w.x, w.y, w.z, w.w};
-        uint32_t lo[4], hi[4];
+        const int zsh = (n4 & 1) * 16;
+        const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+        if constexpr (GIDX) {
+            if constexpr (I == 0) {
+                const int ncol8 = a.N >> 3;
+                const int kbase = kout0 + 8 * wr;
+                const uint32_t wj[4] = {w.x, w.y, w.z, w.w};
+                uint32_t lo[4], hi[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) { lo[j] = wj[j] & 0x0F0F0F0Fu; hi[j] = (wj[j] >> 4) & 0x0F0F0F0Fu; }
-        half2_t s01, s23, z01, z23;
-        auto fetch = [&](int g) {
-            const uint2_t sv = *reinterpret_cast<const uint2_t*>(a.scales + (size_t)g * a.N + n);
-            const uint32_t zw = a.qzeros[(size_t)g * ncol8 + (n >> 3)] >> zsh;
-            s01 = as_half2(sv.x); s23 = as_half2(sv.y);
-            z01 = zero_term(s01, zw & 0xFu, (zw >> 4) & 0xFu);
-            z23 = zero_term(s23, (zw >> 8) & 0xFu, (zw >> 12) & 0xFu);
-        };
-        if (!GIDX) fetch(kbase / a.groupsize);
+                for (int j = 0; j < 4; ++j) { lo[j] = wj[j] & 0x0F0F0F0Fu; hi[j] = (wj[j] >> 4) & 0x0F0F0F0Fu; }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            if (GIDX) fetch(a.g_idx[kbase + e]);
-            const int b = e >> 1;
-            const uint32_t sel = 0x0c000c00u | ((4u + b) << 16) | (uint32_t)b;
-            // (code of column j, code of column j+1) of row e
-            const uint32_t c01 = (e & 1) ? __builtin_amdgcn_perm(hi[1], hi[0], sel) : __builtin_amdgcn_perm(lo[1], lo[0], sel);
-            const uint32_t c23 = (e & 1) ? __builtin_amdgcn_perm(hi[3], hi[2], sel) : __builtin_amdgcn_perm(lo[3], lo[2], sel);
-            const uint2_t o = {as_u32(dequant_pair(codes_to_half2(c01), s01, z01)),
-                               as_u32(dequant_pair(codes_to_half2(c23), s23, z23))};
-            *reinterpret_cast<uint2_t*>(sB + (8 * wr + e) * LDS_STRIDE + 4 * n4) = o;
+                for (int ee = 0; ee < RPT; ++ee) {
+                    const int e = e0 + ee;
+                    const int g = a.g_idx[kbase + e];
+                    const uint2_t s4 = *reinterpret_cast<const uint2_t*>(a.scales + (size_t)g * a.N + n);
+                    const uint32_t z4 = a.qzeros[(size_t)g * ncol8 + (n >> 3)] >> zsh;
+                    const half2_t s01 = as_half2(s4.x), s23 = as_half2(s4.y);
+                    const half2_t z01 = zero_term(s01, z4 & 0xFu, (z4 >> 4) & 0xFu);
+                    const half2_t z23 = zero_term(s23, (z4 >> 8) & 0xFu, (z4 >> 12) & 0xFu);
+                    const int b = e >> 1;
+                    const uint32_t sel = 0x0c000c00u | ((4u + b) << 16) | (uint32_t)b;
+                    const uint32_t c01 = ((e & 1) ? __builtin_amdgcn_perm(hi[1], hi[0], sel) : __builtin_amdgcn_perm(lo[1], lo[0], sel)) | kMagic;
+                    const uint32_t c23 = ((e & 1) ? __builtin_amdgcn_perm(hi[3], hi[2], sel) : __builtin_amdgcn_perm(lo[3], lo[2], sel)) | kMagic;
+                    const uint2_t oo = {as_u32(dequant_pair(as_half2(c01) - k1024, s01, z01)),
+                                        as_u32(dequant_pair(as_half2(c23) - k1024, s23, z23))};
+                    *reinterpret_cast<uint2_t*>(sB + (8 * wr + e) * LDS_STRIDE + 4 * n4) = oo;
+                }
+            }
+        } else {
+            // row e = e0 + I/2 with e0 in {0, 4}: odd/even nibble and byte-in-half are compile-time,
+            // the half of the word (e0) is a per-thread shift by 0 or 16 bits
+            constexpr int el = I / 2, h = I % 2, b = el >> 1;
+            constexpr uint32_t sel = 0x0c000c00u | ((4u + b) << 16) | (uint32_t)b;
+            const int e = e0 + el;
+            const uint32_t z4 = zw >> zsh;
+            const uint32_t wa = (h ? w.z : w.x) >> (4 * e0), wb = (h ? w.w : w.y) >> (4 * e0);   // the two columns of this piece
+            const uint32_t na = (el & 1) ? ((wa >> 4) & 0x0F0F0F0Fu) : (wa & 0x0F0F0F0Fu);
+            const uint32_t nb = (el & 1) ? ((wb >> 4) & 0x0F0F0F0Fu) : (wb & 0x0F0F0F0Fu);
+            const uint32_t codes = __builtin_amdgcn_perm(nb, na, sel) | kMagic;  // (code of column a, of column b) of row e
+            const half2_t s2 = as_half2(h ? sv.y : sv.x);
+            const half2_t zero2 = zero_term(s2, (z4 >> (8 * h)) & 0xFu, (z4 >> (8 * h + 4)) & 0xFu);
+            const uint32_t r = as_u32(dequant_pair_magic(codes, s2, s2 * k1024, zero2));
+            if constexpr (h == 0) o01 = r;
+            else *reinterpret_cast<uint2_t*>(sB + (8 * wr + e) * LDS_STRIDE + 4 * n4) = uint2_t{o01, r};
         }
     }
     // LoRA step: B operand = lora_a [R, K]; LDS row = k, minor = r.
     __device__ __forceinline__ void store_lora(const GemmArgs& a, int kout0, half_t* sB, int t) const {
-        for (int idx = t; idx < BN * BK; idx += 256) {
+        for (int idx = t; idx < BN * BK; idx += NT) {
             const int r = idx >> 7, c = idx & 127;
             sB[c * LDS_STRIDE + r] = (r < a.R) ? a.lb[(size_t)r * a.K + kout0 + c] : (half_t)0.f;
         }
@@ -145,10 +267,21 @@ struct BwdSlab {
 };
 
 // FWD: out[M, NOUT=N], reduction length RED=K.   BWD: out[M, NOUT=K], reduction length RED=N.
-template <bool FWD, bool GIDX>
-__global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a) {
-    __shared__ __attribute__((aligned(16))) half_t sA[BM * LDS_STRIDE];
-    __shared__ __attribute__((aligned(16))) half_t sB[BN * LDS_STRIDE];
+// WGM = wavefronts along M (2 or 4); the workgroup has 2*WGM wavefronts = NT threads.
+template <int BM, int WGM, bool FWD, bool GIDX>
+__global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
+    // four distinct LDS objects (not one carved-up array): the compiler can then prove that the
+    // writes into one buffer do not alias the reads of the other and is free to interleave them
+    __shared__ __attribute__((aligned(16))) half_t sA0[BM * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) half_t sA1[BM * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) half_t sB0[BN * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) half_t sB1[BN * LDS_STRIDE];
+    constexpr int NT = 128 * WGM;                     // threads per workgroup
+    constexpr int WROWS = BM / WGM;                   // output rows per wavefront
+    constexpr int TM = WROWS / 32;                    // 32-row accumulator tiles per wavefront
+    constexpr int NA = BM * 8 / NT;                   // 16-byte activation loads per thread per step
+    constexpr int APASS = NT / 8;                     // activation rows covered by one pass of the workgroup
+    constexpr int KS = BK / 16;                       // MFMA reduction sub-steps per step
 
     const int t = threadIdx.x;
     const int lane = t & 63, wave = t >> 6;
@@ -157,89 +290,189 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a) {
     const int RED = FWD ? a.K : a.N;
     const int m0 = blockIdx.y * BM;
     const int c0 = blockIdx.x * BN;          // first output column of the tile
+    const int rows_valid = min(BM, a.M - m0);
 
-    // activation tile: 128 rows x 64 reduction entries, 16 B per thread per pass, 4 passes
+    // buffer descriptors: activations of this workgroup's rows (rows beyond M read as zero), weights
+    const rsrc_t rs_a = make_rsrc(a.a + (size_t)m0 * RED, (unsigned)rows_valid * (unsigned)RED * 2u);
+    SlabRsrc rs;
+    rs.w = make_rsrc(a.qweight, (unsigned)(a.K >> 3) * (unsigned)a.N * 4u);
+    rs.s = make_rsrc(a.scales, (unsigned)a.G * (unsigned)a.N * 2u);
+    rs.z = make_rsrc(a.qzeros, (unsigned)a.G * (unsigned)(a.N >> 3) * 4u);
+
+    // activation tile: BM rows x 64 reduction entries, 16 B per thread per pass.
+    // Two register sets (areg / slab): while stage s is multiplied out of LDS, stage s+1 sits in
+    // registers waiting to be dequantized into the other LDS buffer and stage s+2 is in flight.
     const int arow = t >> 3, acol = (t & 7) * 8;
-    uint4_t areg[4];
-    auto load_a = [&](const half_t* base, int ld, int red0, int redlen) {
+    const int voff_a = (arow * RED + acol) * 2;
+    const int astride = APASS * RED * 2;
+    uint4_t areg[2][NA];
+    auto load_a = [&](uint4_t* dst, int red0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int m = m0 + arow + 32 * i;
-            areg[i] = uint4_t{0u, 0u, 0u, 0u};
-            if (m < a.M && red0 + acol < redlen)
-                areg[i] = *reinterpret_cast<const uint4_t*>(base + (size_t)m * ld + red0 + acol);
-        }
+        for (int i = 0; i < NA; ++i) dst[i] = buf_load128(rs_a, voff_a + i * astride, red0 * 2);
     };
-    auto store_a = [&]() {
+    auto store_a = [&](const uint4_t* src, half_t* dst) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            *reinterpret_cast<uint4_t*>(sA + (arow + 32 * i) * LDS_STRIDE + acol) = areg[i];
+        for (int i = 0; i < NA; ++i)
+            *reinterpret_cast<uint4_t*>(dst + (arow + APASS * i) * LDS_STRIDE + acol) = src[i];
     };
 
-    typename std::conditional<FWD, FwdSlab<GIDX>, BwdSlab<GIDX>>::type slab;
-    slab.init(t);
+    using Slab = typename std::conditional<FWD, FwdSlab<GIDX, NT>, BwdSlab<GIDX, NT>>::type;
+    constexpr int NSL = Slab::kSlices;
+    Slab slab[2];
+    slab[0].init(t, a, c0);
+    slab[1].init(t, a, c0);
 
-    float16_t acc[2][2];
+    float16_t acc[TM][2];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TM; ++i)
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    auto mma_tile = [&](int ksteps) {
-        const int lr = lane & 31, lk = (lane >> 5) * 8;
-        for (int ks = 0; ks < ksteps; ++ks) {
-            half8_t af[2], bf[2];
+    const int lr = lane & 31, lk = (lane >> 5) * 8;
+    const int a_off = (wm * WROWS + lr) * LDS_STRIDE + lk;
+    const int b_off = (wn * 64 + lr) * LDS_STRIDE + lk;
+    auto read_frags = [&](half8_t* af, half8_t* bf, const half_t* pa, const half_t* pb, int ks) {
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
-                af[i] = *reinterpret_cast<const half8_t*>(sA + (wm * 64 + 32 * i + lr) * LDS_STRIDE + 16 * ks + lk);
+        for (int i = 0; i < TM; ++i)
+            af[i] = *reinterpret_cast<const half8_t*>(pa + a_off + 32 * i * LDS_STRIDE + 16 * ks);
 #pragma unroll
-            for (int j = 0; j < 2; ++j)
-                bf[j] = *reinterpret_cast<const half8_t*>(sB + (wn * 64 + 32 * j + lr) * LDS_STRIDE + 16 * ks + lk);
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
-        }
+        for (int j = 0; j < 2; ++j)
+            bf[j] = *reinterpret_cast<const half8_t*>(pb + b_off + 32 * j * LDS_STRIDE + 16 * ks);
     };
 
-    const int nsteps = RED / BK;
-    load_a(a.a, RED, 0, RED);
-    slab.load(a, c0, 0);
-    for (int s = 0; s < nsteps; ++s) {
-        store_a();
-        slab.store(a, c0, s * BK, sB);
-        __syncthreads();
-        if (s + 1 < nsteps) {
-            load_a(a.a, RED, (s + 1) * BK, RED);
-            slab.load(a, c0, (s + 1) * BK);
-        }
-        mma_tile(BK / 16);
-        __syncthreads();
+    const int nsteps = RED / BK;              // even: RED is a multiple of 128
+    const int last = (nsteps - 1) * BK;
+    half8_t af[2][TM], bf[2][2];              // operand fragments, double buffered over the sub-steps
+
+    // One pipeline step, branch-free.  CUR = LDS buffer / register set of the stage being multiplied:
+    //   registers[CUR]   <- global loads of stage s+2 (clamped to the last stage: a harmless reload)
+    //   LDS[CUR^1]       <- dequantized stage s+1 from registers[CUR^1]
+    //   acc              += LDS[CUR] (stage s); on entry af[0]/bf[0] already hold sub-step 0
+    auto step = [&](int s, auto cur_tag) {
+        constexpr int CUR = decltype(cur_tag)::value;
+        constexpr int NM = TM * 2 * KS;                        // MFMAs per step
+        constexpr int NITEM = 2 + NSL + NA;                    // side-work items per step
+        constexpr int BAR = NM - 4;                            // MFMA index after which the barrier sits
+        // fragment set 0 is reloaded right after the barrier: every MFMA of sub-step KS-2 (its last
+        // user in this step) must have been issued by then
+        static_assert(BAR >= (KS - 1) * TM * 2 - 1, "barrier placed before the last use of fragment set 0");
+        const int red_next2 = min((s + 2) * BK, last);
+        const int red_next1 = min((s + 1) * BK, last);
+        const half_t* const a_cur = CUR ? sA1 : sA0;
+        const half_t* const b_cur = CUR ? sB1 : sB0;
+        half_t* const a_nxt = CUR ? sA0 : sA1;
+        half_t* const b_nxt = CUR ? sB0 : sB1;
+        static_for<0, NM>([&](auto ic) {
+            constexpr int i = decltype(ic)::value;
+            constexpr int ks = i / (TM * 2), r = i % (TM * 2), ti = r / 2, tj = r % 2;
+            if constexpr (r == 0 && ks + 1 < KS)
+                read_frags(af[(ks + 1) & 1], bf[(ks + 1) & 1], a_cur, b_cur, ks + 1);
+            acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[ks & 1][ti], bf[ks & 1][tj], acc[ti][tj], 0, 0, 0);
+            // side work is spread over MFMAs 0..BAR so that it is complete when the barrier comes
+            constexpr int j_lo = i <= BAR ? (i * NITEM) / (BAR + 1) : NITEM;
+            constexpr int j_hi = i <= BAR ? ((i + 1) * NITEM) / (BAR + 1) : NITEM;
+            static_for<j_lo, j_hi>([&](auto jc) {
+                constexpr int j = decltype(jc)::value;
+                if constexpr (j == 0) slab[CUR].load(a, rs, c0, red_next2);
+                else if constexpr (j == 1) load_a(areg[CUR], red_next2);
+                else if constexpr (j < 2 + NSL) slab[CUR ^ 1].template store_slice<j - 2>(a, c0, red_next1, b_nxt);
+                else
+                    *reinterpret_cast<uint4_t*>(a_nxt + (arow + APASS * (j - 2 - NSL)) * LDS_STRIDE + acol) =
+                        areg[CUR ^ 1][j - 2 - NSL];
+            });
+            if constexpr (i == BAR) {
+                // every wavefront has finished reading LDS[CUR] (the last fragments were fetched at
+                // sub-step KS-2) and has written its share of LDS[CUR^1]
+                __syncthreads();
+                read_frags(af[0], bf[0], a_nxt, b_nxt, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+
+    load_a(areg[0], 0);
+    slab[0].load(a, rs, c0, 0);
+    load_a(areg[1], min(BK, last));
+    slab[1].load(a, rs, c0, min(BK, last));
+    store_a(areg[0], sA0);
+    static_for<0, NSL>([&](auto jc) { slab[0].template store_slice<decltype(jc)::value>(a, c0, 0, sB0); });
+    __syncthreads();
+    read_frags(af[0], bf[0], sA0, sB0, 0);
+    for (int s = 0; s < nsteps; s += 2) {
+        step(s, std::integral_constant<int, 0>{});
+        step(s + 1, std::integral_constant<int, 1>{});
     }
     if (a.R > 0) {
-        load_a(a.la, a.R, 0, a.R);
-        store_a();
-        slab.store_lora(a, c0, sB, t);
+        // rank-R adapter step: activations [M, R] (columns beyond R are zero), adapter matrix from lb
         __syncthreads();
-        mma_tile((a.R + 15) / 16);
+        const rsrc_t rs_l = make_rsrc(a.la + (size_t)m0 * a.R, (unsigned)rows_valid * (unsigned)a.R * 2u);
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+            uint4_t v = {0u, 0u, 0u, 0u};
+            if (acol < a.R) v = buf_load128(rs_l, ((arow + APASS * i) * a.R + acol) * 2, 0);
+            *reinterpret_cast<uint4_t*>(sA0 + (arow + APASS * i) * LDS_STRIDE + acol) = v;
+        }
+        slab[0].store_lora(a, c0, sB0, t);
+        __syncthreads();
+        for (int ks = 0; ks < (a.R + 15) / 16; ++ks) {
+            read_frags(af[0], bf[0], sA0, sB0, ks);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][i], bf[0][j], acc[i][j], 0, 0, 0);
+        }
     }
 
-    // epilogue: acc[i][j][r] is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of its 32x32 tile
+    // epilogue: acc[i][j][r] is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of its 32x32 tile.
+    // Each wavefront transposes one 32 x 64 block at a time through its own 4.5 KB of LDS
+    // (row stride 72 halves) and writes it as 16-byte pieces: 8 lanes cover one 128-byte row segment.
+    __syncthreads();
+    half_t* stage = sA0 + wave * (32 * LDS_STRIDE);
     const int lc = lane & 31, lrow = (lane >> 5) * 4;
+    const int orow = lane >> 3, ocol = (lane & 7) * 8;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const int col = c0 + wn * 64 + 32 * j + lc;
-        const float bv = (FWD && a.bias) ? (float)a.bias[col] : 0.f;
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int j = 0; j < 2; ++j) {
+            const float bv = (FWD && a.bias) ? (float)a.bias[c0 + wn * 64 + 32 * j + lc] : 0.f;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int m = m0 + wm * 64 + 32 * i + 8 * (r >> 2) + lrow + (r & 3);
-                if (m < a.M) a.out[(size_t)m * NOUT + col] = (half_t)(acc[i][j][r] + bv);
-            }
+            for (int r = 0; r < 16; ++r)
+                stage[(8 * (r >> 2) + lrow + (r & 3)) * LDS_STRIDE + 32 * j + lc] = (half_t)(acc[i][j][r] + bv);
+        }
+        // wavefront-private staging area: a workgroup barrier is not needed, only completion of
+        // this wavefront's own LDS writes (the compiler inserts the lgkmcnt wait for the reads)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int rr = orow + 8 * p;
+            const int m = m0 + wm * WROWS + 32 * i + rr;
+            const uint4_t v = *reinterpret_cast<const uint4_t*>(stage + rr * LDS_STRIDE + ocol);
+            if (m < a.M) *reinterpret_cast<uint4_t*>(a.out + (size_t)m * NOUT + c0 + wn * 64 + ocol) = v;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
+template <int BM, int WGM, bool FWD, bool GIDX>
+static hipError_t launch_gemm(const GemmArgs& a, int nout, hipStream_t stream) {
+    const dim3 grid(nout / BN, (a.M + BM - 1) / BM);
+    hipLaunchKernelGGL((gemm_kernel<BM, WGM, FWD, GIDX>), grid, dim3(128 * WGM), 0, stream, a);
+    return hipGetLastError();
+}
+
+template <bool FWD, bool GIDX>
+static hipError_t launch_gemm_cfg(int cfg, const GemmArgs& a, int nout, hipStream_t stream) {
+    switch (cfg) {
+        case 0: return launch_gemm<128, 2, FWD, GIDX>(a, nout, stream);    // 128 x 128, 4 wavefronts of 64 x 64
+        case 1: return launch_gemm<256, 2, FWD, GIDX>(a, nout, stream);    // 256 x 128, 4 wavefronts of 128 x 64
+        default: return launch_gemm<256, 4, FWD, GIDX>(a, nout, stream);   // 256 x 128, 8 wavefronts of 64 x 64
     }
 }
 
@@ -247,7 +480,7 @@ __global__ __launch_bounds__(256) void gemm_kernel(GemmArgs a) {
 
 extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros,
                               const void* scales, const int32_t* g_idx, int groupsize, const void* bias,
-                              const void* la, const void* lb, int R, void* out, int M, int K, int N,
+                              const void* la, const void* lb, int R, void* out, int M, int K, int N, int G,
                               hipStream_t stream) {
     using namespace q4;
     GemmArgs a;
@@ -262,17 +495,15 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     a.lb = reinterpret_cast<const half_t*>(lb);
     a.R = (la && lb) ? R : 0;
     a.out = reinterpret_cast<half_t*>(out);
-    a.M = M; a.K = K; a.N = N;
+    a.M = M; a.K = K; a.N = N; a.G = G;
     const int nout = fwd ? N : K;
-    const dim3 grid(nout / BN, (M + BM - 1) / BM);
-    const dim3 block(256);
     const bool gidx = g_idx != nullptr;
-    if (fwd) {
-        if (gidx) hipLaunchKernelGGL((gemm_kernel<true, true>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((gemm_kernel<true, false>), grid, block, 0, stream, a);
-    } else {
-        if (gidx) hipLaunchKernelGGL((gemm_kernel<false, true>), grid, block, 0, stream, a);
-        else hipLaunchKernelGGL((gemm_kernel<false, false>), grid, block, 0, stream, a);
-    }
-    return hipGetLastError() == hipSuccess ? 0 : -4;
+    // tile configuration: 256-row tiles once they still give every CU a workgroup
+    static const int env_cfg = getenv("Q4_GEMM_CFG") ? atoi(getenv("Q4_GEMM_CFG")) : -1;
+    const bool tall = (long)(nout / BN) * ((M + 255) / 256) >= 200;
+    const int cfg = env_cfg >= 0 ? env_cfg : (tall ? 2 : 0);
+    hipError_t e;
+    if (fwd) e = gidx ? launch_gemm_cfg<true, true>(cfg, a, nout, stream) : launch_gemm_cfg<true, false>(cfg, a, nout, stream);
+    else e = gidx ? launch_gemm_cfg<false, true>(cfg, a, nout, stream) : launch_gemm_cfg<false, false>(cfg, a, nout, stream);
+    return e == hipSuccess ? 0 : -4;
 }

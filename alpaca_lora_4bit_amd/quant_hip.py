@@ -80,6 +80,29 @@ def classify_g_idx(g_idx, groupsize, G):
     return kind
 
 
+def scales_fit_fused_dequant(scales):
+    """True when every |scale| < 64: the GEMM kernels then form rn16(s*q) with one fused
+    multiply-add on (1024 + q), which needs 1024*s to be finite.  Cached on the tensor like
+    the g_idx verdict (first call per tensor synchronises).  Real GPTQ scales are ~1e-2."""
+    key = scales._version
+    cached = getattr(scales, "_q4_small", None)
+    if cached is not None and cached[0] == key:
+        return cached[1]
+    ok = bool(torch.isfinite(scales).all()) and float(scales.abs().max()) < 64.0
+    scales._q4_small = (key, ok)
+    return ok
+
+
+def _gemm_gidx_arg(g_idx, groupsize, G, K, scales):
+    """Like _gidx_arg for the GEMM kernels; layers with huge scales are routed to the
+    per-row-group path, whose dequant has no range restriction."""
+    if scales_fit_fused_dequant(scales):
+        return _gidx_arg(g_idx, groupsize, G, need_multiple=64) + (g_idx,)
+    if g_idx is None:
+        g_idx = (torch.arange(K, device=scales.device, dtype=torch.int32) // int(groupsize)).contiguous()
+    return g_idx.data_ptr(), int(groupsize or 0), g_idx
+
+
 def _gidx_arg(g_idx, groupsize, G, need_multiple=32):
     """Returns (pointer-or-0, groupsize) to hand to the C ABI."""
     if g_idx is None:
@@ -183,7 +206,7 @@ def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, 
         _require(bias.dtype == torch.float16 and tuple(bias.shape) == (N,) and bias.is_contiguous()
                  and bias.device == dev, "bias must be a contiguous float16 [N] tensor on the same device")
     xa, lora_bt, R = _lora_pair(xa, lora_bt, M, N, dev)
-    gp, gs = _gidx_arg(g_idx, groupsize, G, need_multiple=64)
+    gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
     out = torch.empty(_out_shape(out_shape, M, N), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().q4_gemm_fwd_f16(x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
@@ -199,7 +222,7 @@ def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=Non
     dy2 = _flat_half(dy, N, dev, "grad_output")
     M = dy2.shape[0]
     dyb, lora_a, R = _lora_pair(dyb, lora_a, M, K, dev)
-    gp, gs = _gidx_arg(g_idx, groupsize, G, need_multiple=64)
+    gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
     out = torch.empty(_out_shape(out_shape, M, K), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().q4_gemm_bwd_dx_f16(dy2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),

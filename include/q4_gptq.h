@@ -56,9 +56,9 @@ int q4_dequant_f16(const int32_t *qweight, const int32_t *qzeros, const void *sc
  * as dispatched by matmul_utils_4bit.py:59-95.  g_idx == NULL selects sequential groups of
  * `groupsize` rows (the old_faster convention, quant_cuda_kernel.cu:1024); otherwise rows are
  * gathered through g_idx (the vecquant4matmul convention, :513-520).
- * `workspace` must hold q4_gemv_workspace_bytes(M, K, N) bytes, 256-byte aligned, and must be
- * ZERO before its first use; every call leaves it zeroed again.  Calls sharing one workspace
- * must be ordered on one stream. */
+ * `workspace` must hold q4_gemv_workspace_bytes(M, K, N) = 8*M*N bytes, 256-byte aligned, and must be
+ * ZERO before its first use; every call leaves it zeroed again (it carries the fixed-point split-K
+ * sums).  Calls sharing one workspace must be ordered on one stream.  K <= 1 044 480. */
 size_t q4_gemv_workspace_bytes(int M, int K, int N);
 int q4_gemv_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                 const int32_t *g_idx, int groupsize, void *y, int accumulate,
@@ -71,7 +71,10 @@ int q4_gemv_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, co
  * Replaces vecquant4recons_v2 + torch.matmul(x, buffer) (matmul_utils_4bit.py:114-124),
  * the bias add (autograd_4bit.py:206-207) and, when xa/lora_bt are given, the adapter term
  * result += lora_B(lora_A(x)) * scaling (models.py:58-66) where xa = scaling * x @ A^T and
- * lora_bt = B^T.  bias, xa, lora_bt may be NULL; R is 0 or a multiple of 8, at most 64. */
+ * lora_bt = B^T.  bias, xa, lora_bt may be NULL; R is 0 or a multiple of 8, at most 64.
+ * Both GEMM entry points need K % 128 == 0 and N % 128 == 0, and with g_idx == NULL also
+ * groupsize % 64 == 0 and every |scale| < 64 (the sequential-group dequant forms s*q with a fused
+ * multiply-add on 1024+q; pass g_idx to lift the restriction on the scales). */
 int q4_gemm_fwd_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                     const int32_t *g_idx, int groupsize, const void *bias,
                     const void *xa, const void *lora_bt, int R,
