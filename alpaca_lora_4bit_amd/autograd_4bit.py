@@ -218,11 +218,12 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
     (models.py:58-66) and, in backward, AutogradMatmul4bitCuda.backward (autograd_4bit.py:45-54)
     plus torch autograd over the two adapter Linears.  Here the rank-r products ride in the
     main GEMM as one extra reduction step, forward and backward:
-        fwd   xa  = scaling * x @ A^T   [M, r]   then  y  = [x | xa]  @ [W ; B^T]
-        bwd   dyb = scaling * dy @ B    [M, r]   then  dx = [dy | dyb] @ [W^T ; A]
-              dA  = dyb^T @ x   [r, K]            dB = dy^T @ xa   [N, r]
+        fwd   xa  = x @ A^T    [M, r]   then  y  = [x | xa]  @ [W ; scaling * B^T]
+        bwd   dyb = dy @ B     [M, r]   then  dx = [dy | dyb] @ [W^T ; scaling * A]
+              dA  = scaling * dyb^T @ x   [r, K]        dB = scaling * dy^T @ xa   [N, r]
     A: lora_A.weight [r, K], B: lora_B.weight [N, r] (any float dtype; products run in fp16
-    with fp32 accumulation, like the reference under autocast)."""
+    with fp32 accumulation, like the reference under autocast).  The adapter matrices go to the
+    kernels as strided views: no transposed or pre-scaled copies are made."""
 
     @staticmethod
     @custom_fwd(device_type='cuda', cast_inputs=torch.float16)
@@ -233,11 +234,9 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
             x2 = x2.half()
         a16 = lora_a.to(torch.float16)
         b16 = lora_b.to(torch.float16)
-        xa = torch.matmul(x2, a16.t())
-        if scaling != 1.0:
-            xa = xa * scaling
+        xa = torch.mm(x2, a16.t())
         y = quant_hip.gemm_fwd(x2, qweight, zeros, scales, g_idx, groupsize, bias=bias,
-                               xa=xa, lora_bt=b16.t().contiguous(), out_shape=tuple(x.shape[:-1]) + (N,))
+                               xa=xa, lora_bt=b16.t(), lora_scale=scaling, out_shape=tuple(x.shape[:-1]) + (N,))
         ctx.save_for_backward(x2, xa, qweight, scales, zeros, g_idx, a16, b16)
         ctx.scaling = scaling
         ctx.groupsize = groupsize
@@ -253,15 +252,14 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
         if dy.dtype != torch.float16:
             dy = dy.half()
         dy = dy.contiguous()
-        dyb = torch.matmul(dy, b16)
-        if ctx.scaling != 1.0:
-            dyb = dyb * ctx.scaling
+        dyb = torch.mm(dy, b16)
         dx = da = db = None
         if ctx.needs_input_grad[0]:
             dx = quant_hip.gemm_bwd_dx(dy, qweight, zeros, scales, g_idx, ctx.groupsize, dyb=dyb, lora_a=a16,
+                                       lora_scale=ctx.scaling,
                                        out_shape=tuple(grad_output.shape[:-1]) + (qweight.shape[0] * 8,))
         if ctx.needs_input_grad[6]:
-            da = torch.matmul(dyb.t(), x2).to(ctx.ab_dtypes[0])
+            da = torch.addmm(a16, dyb.t(), x2, beta=0.0, alpha=ctx.scaling).to(ctx.ab_dtypes[0])
         if ctx.needs_input_grad[7]:
-            db = torch.matmul(dy.t(), xa).to(ctx.ab_dtypes[1])
+            db = torch.addmm(b16, dy.t(), xa, beta=0.0, alpha=ctx.scaling).to(ctx.ab_dtypes[1])
         return dx, None, None, None, None, None, da, db, None, None

@@ -9,7 +9,7 @@ int q4_launch_dequant(const int32_t*, const int32_t*, const void*, const int32_t
 int q4_launch_gemv(const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, void*, int,
                    int, int, int, int, void*, hipStream_t);
 int q4_launch_gemm(int, const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, const void*,
-                   const void*, const void*, int, void*, int, int, int, int, hipStream_t);
+                   const void*, const void*, int, int, float, int, void*, int, int, int, int, hipStream_t);
 }
 
 namespace {
@@ -29,7 +29,7 @@ int check_layer(const void* qweight, const void* qzeros, const void* scales, con
 }
 }  // namespace
 
-extern "C" int q4_abi_version(void) { return 1; }
+extern "C" int q4_abi_version(void) { return 2; }
 
 extern "C" const char* q4_error_string(int code) {
     switch (code) {
@@ -68,7 +68,8 @@ extern "C" int q4_gemv_f16(const void* x, const int32_t* qweight, const int32_t*
 }
 
 static int gemm_common(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros, const void* scales,
-                       const int32_t* g_idx, int groupsize, const void* bias, const void* la, const void* lb, int R,
+                       const int32_t* g_idx, int groupsize, const void* bias, const void* la, const void* lb,
+                       int lb_sr, int lb_sc, float lb_scale, int R,
                        void* out, int M, int K, int N, int G, void* stream) {
     int rc = check_layer(qweight, qzeros, scales, g_idx, groupsize, K, N, G);
     if (rc != Q4_OK) return rc;
@@ -80,22 +81,25 @@ static int gemm_common(int fwd, const void* act, const int32_t* qweight, const i
     if ((unsigned long long)(K > N ? K : N) * 512ull >= (1ull << 32)) return Q4_ERR_BAD_SHAPE;
     if ((la != nullptr) != (lb != nullptr)) return Q4_ERR_NULL_POINTER;
     if (la && (R < 8 || R > 64 || (R % 8) != 0)) return Q4_ERR_BAD_SHAPE;
-    if (misaligned(act) || misaligned(out) || (la && misaligned(la)) || (lb && misaligned(lb)))
-        return Q4_ERR_MISALIGNED;
-    return q4_launch_gemm(fwd, act, qweight, qzeros, scales, g_idx, groupsize, bias, la, lb, R, out, M, K, N, G,
-                          (hipStream_t)stream);
+    if (misaligned(act) || misaligned(out) || (la && misaligned(la))) return Q4_ERR_MISALIGNED;
+    if (lb && (reinterpret_cast<uintptr_t>(lb) & 1u)) return Q4_ERR_MISALIGNED;
+    if (lb && (lb_sr < 1 || lb_sc < 1)) return Q4_ERR_BAD_SHAPE;
+    return q4_launch_gemm(fwd, act, qweight, qzeros, scales, g_idx, groupsize, bias, la, lb, lb_sr, lb_sc, lb_scale, R,
+                          out, M, K, N, G, (hipStream_t)stream);
 }
 
 extern "C" int q4_gemm_fwd_f16(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
                                const int32_t* g_idx, int groupsize, const void* bias,
-                               const void* xa, const void* lora_bt, int R,
+                               const void* xa, const void* lora_b, int ldb_r, int ldb_n, float lora_scale, int R,
                                void* y, int M, int K, int N, int G, void* stream) {
-    return gemm_common(1, x, qweight, qzeros, scales, g_idx, groupsize, bias, xa, lora_bt, R, y, M, K, N, G, stream);
+    return gemm_common(1, x, qweight, qzeros, scales, g_idx, groupsize, bias, xa, lora_b, ldb_r, ldb_n, lora_scale, R,
+                       y, M, K, N, G, stream);
 }
 
 extern "C" int q4_gemm_bwd_dx_f16(const void* dy, const int32_t* qweight, const int32_t* qzeros, const void* scales,
                                   const int32_t* g_idx, int groupsize,
-                                  const void* dyb, const void* lora_a, int R,
+                                  const void* dyb, const void* lora_a, int lda_r, int lda_k, float lora_scale, int R,
                                   void* dx, int M, int K, int N, int G, void* stream) {
-    return gemm_common(0, dy, qweight, qzeros, scales, g_idx, groupsize, nullptr, dyb, lora_a, R, dx, M, K, N, G, stream);
+    return gemm_common(0, dy, qweight, qzeros, scales, g_idx, groupsize, nullptr, dyb, lora_a, lda_r, lda_k, lora_scale, R,
+                       dx, M, K, N, G, stream);
 }

@@ -50,7 +50,9 @@ struct GemmArgs {
     int groupsize;
     const half_t* bias;       // fwd only, [N] or null
     const half_t* la;         // fwd: xa [M,R]     bwd: dyb [M,R]   (or null)
-    const half_t* lb;         // fwd: lora_bt [R,N] bwd: lora_a [R,K]
+    const half_t* lb;         // adapter matrix, element (r, c) at lb[r*lb_sr + c*lb_sc]; fwd: c = n, bwd: c = k
+    int lb_sr, lb_sc;
+    float lb_scale;           // multiplied into the adapter matrix when it is staged in LDS
     int R;
     half_t* out;              // fwd: y [M,N]      bwd: dx [M,K]
     int M, K, N, G;
@@ -170,11 +172,12 @@ struct FwdSlab {
                 *reinterpret_cast<uint4_t*>(sB + col * LDS_STRIDE + 8 * (wr0 + WSTEP * i)) = uint4_t{o[0], o[1], o[2], o[3]};
         }
     }
-    // LoRA step: B operand = lora_bt [R, N]; LDS row = column n, minor = r (zero padded to 64).
+    // LoRA step: B operand = adapter matrix [R, N]; LDS row = column n, minor = r (zero padded to 64).
     __device__ __forceinline__ void store_lora(const GemmArgs& a, int n0, half_t* sB, int t) const {
         for (int idx = t; idx < BN * BK; idx += NT) {
             const int r = idx >> 7, c = idx & 127;
-            sB[c * LDS_STRIDE + r] = (r < a.R) ? a.lb[(size_t)r * a.N + n0 + c] : (half_t)0.f;
+            sB[c * LDS_STRIDE + r] = (r < a.R) ? (half_t)(a.lb_scale * (float)a.lb[(size_t)r * a.lb_sr + (size_t)(n0 + c) * a.lb_sc])
+                                               : (half_t)0.f;
         }
     }
 };
@@ -257,11 +260,12 @@ struct BwdSlab {
             else *reinterpret_cast<uint2_t*>(sB + (8 * wr + e) * LDS_STRIDE + 4 * n4) = uint2_t{o01, r};
         }
     }
-    // LoRA step: B operand = lora_a [R, K]; LDS row = k, minor = r.
+    // LoRA step: B operand = adapter matrix [R, K]; LDS row = k, minor = r.
     __device__ __forceinline__ void store_lora(const GemmArgs& a, int kout0, half_t* sB, int t) const {
         for (int idx = t; idx < BN * BK; idx += NT) {
             const int r = idx >> 7, c = idx & 127;
-            sB[c * LDS_STRIDE + r] = (r < a.R) ? a.lb[(size_t)r * a.K + kout0 + c] : (half_t)0.f;
+            sB[c * LDS_STRIDE + r] = (r < a.R) ? (half_t)(a.lb_scale * (float)a.lb[(size_t)r * a.lb_sr + (size_t)(kout0 + c) * a.lb_sc])
+                                               : (half_t)0.f;
         }
     }
 };
@@ -480,8 +484,8 @@ static hipError_t launch_gemm_cfg(int cfg, const GemmArgs& a, int nout, hipStrea
 
 extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros,
                               const void* scales, const int32_t* g_idx, int groupsize, const void* bias,
-                              const void* la, const void* lb, int R, void* out, int M, int K, int N, int G,
-                              hipStream_t stream) {
+                              const void* la, const void* lb, int lb_sr, int lb_sc, float lb_scale, int R,
+                              void* out, int M, int K, int N, int G, hipStream_t stream) {
     using namespace q4;
     GemmArgs a;
     a.a = reinterpret_cast<const half_t*>(act);
@@ -493,6 +497,7 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     a.bias = reinterpret_cast<const half_t*>(bias);
     a.la = reinterpret_cast<const half_t*>(la);
     a.lb = reinterpret_cast<const half_t*>(lb);
+    a.lb_sr = lb_sr; a.lb_sc = lb_sc; a.lb_scale = lb_scale;
     a.R = (la && lb) ? R : 0;
     a.out = reinterpret_cast<half_t*>(out);
     a.M = M; a.K = K; a.N = N; a.G = G;

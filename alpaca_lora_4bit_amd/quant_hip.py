@@ -184,49 +184,53 @@ def gemv(x, qweight, qzeros, scales, g_idx=None, groupsize=None, out=None, accum
 
 
 def _lora_pair(la, lb, rows, cols, dev):
+    """la: [rows, R] fp16 contiguous; lb: [R, cols] fp16 with any (positive) strides."""
     if la is None and lb is None:
-        return None, None, 0
+        return None, None, 0, 0, 0
     _require(la is not None and lb is not None, "both LoRA operands are required")
     R = la.shape[-1]
     _require(la.dtype == torch.float16 and lb.dtype == torch.float16, "LoRA operands must be float16")
     _require(tuple(la.shape) == (rows, R) and tuple(lb.shape) == (R, cols), "LoRA operand shapes do not match")
     _require(R % 8 == 0 and 8 <= R <= 64, "LoRA rank must be a multiple of 8 in [8, 64] for the fused path")
-    _require(la.is_contiguous() and lb.is_contiguous() and la.device == dev and lb.device == dev,
-             "LoRA operands must be contiguous and on the same device")
-    return la, lb, R
+    _require(la.is_contiguous() and la.device == dev and lb.device == dev, "LoRA operands must be on the same device")
+    sr, sc = lb.stride()
+    _require(sr >= 1 and sc >= 1, "the adapter matrix must have positive strides")
+    return la, lb, R, int(sr), int(sc)
 
 
 def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, xa=None, lora_bt=None,
-             out_shape=None):
-    """y fp16 [M, N] = x @ W (+ bias) (+ xa @ lora_bt), W dequantized tile by tile in LDS."""
+             lora_scale=1.0, out_shape=None):
+    """y fp16 [M, N] = x @ W (+ bias) (+ lora_scale * xa @ lora_bt), W dequantized tile by tile in LDS.
+    `lora_bt` is the adapter matrix as an [R, N] view with any strides (e.g. `lora_B.weight.half().t()`)."""
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     x2 = _flat_half(x, K, dev, "x")
     M = x2.shape[0]
     if bias is not None:
         _require(bias.dtype == torch.float16 and tuple(bias.shape) == (N,) and bias.is_contiguous()
                  and bias.device == dev, "bias must be a contiguous float16 [N] tensor on the same device")
-    xa, lora_bt, R = _lora_pair(xa, lora_bt, M, N, dev)
+    xa, lora_bt, R, sr, sc = _lora_pair(xa, lora_bt, M, N, dev)
     gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
     out = torch.empty(_out_shape(out_shape, M, N), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().q4_gemm_fwd_f16(x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
-                                        gp, gs, _ptr(bias), _ptr(xa), _ptr(lora_bt), R,
+                                        gp, gs, _ptr(bias), _ptr(xa), _ptr(lora_bt), sr, sc, float(lora_scale), R,
                                         out.data_ptr(), M, K, N, G, _stream(dev))
     _lib.check(rc, "q4_gemm_fwd_f16")
     return out
 
 
-def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=None, lora_a=None, out_shape=None):
-    """dx fp16 [M, K] = dy [M, N] @ W^T (+ dyb @ lora_a)."""
+def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=None, lora_a=None, lora_scale=1.0,
+                out_shape=None):
+    """dx fp16 [M, K] = dy [M, N] @ W^T (+ lora_scale * dyb @ lora_a); lora_a is an [R, K] view."""
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     dy2 = _flat_half(dy, N, dev, "grad_output")
     M = dy2.shape[0]
-    dyb, lora_a, R = _lora_pair(dyb, lora_a, M, K, dev)
+    dyb, lora_a, R, sr, sc = _lora_pair(dyb, lora_a, M, K, dev)
     gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
     out = torch.empty(_out_shape(out_shape, M, K), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().q4_gemm_bwd_dx_f16(dy2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
-                                           gp, gs, _ptr(dyb), _ptr(lora_a), R,
+                                           gp, gs, _ptr(dyb), _ptr(lora_a), sr, sc, float(lora_scale), R,
                                            out.data_ptr(), M, K, N, G, _stream(dev))
     _lib.check(rc, "q4_gemm_bwd_dx_f16")
     return out

@@ -157,23 +157,51 @@ def bench_lora_step(reps, seed=5):
         with torch.amp.autocast(device_type="cuda"):
             y = m(x)
         y.backward(dy)
+
+    def clear():
         x.grad = None
         m.lora_A["default"].weight.grad = None
         m.lora_B["default"].weight.grad = None
 
+    # eager: Python launches every kernel
     for _ in range(3):
         step()
+        clear()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(reps):
         step()
+        clear()
     e1.record()
     torch.cuda.synchronize()
+    eager = e0.elapsed_time(e1) * 1e-3 / reps
+
+    # the same forward + backward captured once as a HIP graph and replayed (no Python between kernels)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        for _ in range(2):
+            step()
+            clear()
+    s.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        step()
+    with torch.cuda.stream(s):
+        g.replay()
+        s.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(s)
+        for _ in range(reps):
+            g.replay()
+        e1.record(s)
+        torch.cuda.synchronize()
     per = e0.elapsed_time(e1) * 1e-3 / reps
     flop = 2 * 2 * M * K * N + (2 * M * K * r + 2 * M * r * N) + 2 * (2 * M * K * r + 2 * M * r * N)
     return dict(ms=per * 1e3, tokens_per_s=M / per, tflops=flop / per / 1e12,
-                frac_mfma=flop / per / 1e12 / MFMA_FP16_PEAK_TFLOPS, gflop_per_step=flop / 1e9)
+                frac_mfma=flop / per / 1e12 / MFMA_FP16_PEAK_TFLOPS, gflop_per_step=flop / 1e9,
+                eager_ms=eager * 1e3, eager_tokens_per_s=M / eager)
 
 
 def bench_gemm_only(M, K, N, act_order, reps, seed=7):

@@ -66,28 +66,31 @@ int q4_gemv_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, co
                 void *workspace, size_t workspace_bytes, void *stream);
 
 /* Forward GEMM, any M >= 1:
- *   y fp16 [M, N] = x fp16 [M, K] @ W  (+ bias fp16 [N])  (+ xa fp16 [M, R] @ lora_bt fp16 [R, N])
+ *   y fp16 [M, N] = x fp16 [M, K] @ W  (+ bias fp16 [N])  (+ lora_scale * xa fp16 [M, R] @ Bm [R, N])
  * with fp32 accumulation on MFMA; W tiles are dequantized in LDS and never written to HBM.
  * Replaces vecquant4recons_v2 + torch.matmul(x, buffer) (matmul_utils_4bit.py:114-124),
- * the bias add (autograd_4bit.py:206-207) and, when xa/lora_bt are given, the adapter term
- * result += lora_B(lora_A(x)) * scaling (models.py:58-66) where xa = scaling * x @ A^T and
- * lora_bt = B^T.  bias, xa, lora_bt may be NULL; R is 0 or a multiple of 8, at most 64.
- * Both GEMM entry points need K % 128 == 0 and N % 128 == 0, and with g_idx == NULL also
+ * the bias add (autograd_4bit.py:206-207) and, when xa/lora_b are given, the adapter term
+ * result += lora_B(lora_A(x)) * scaling (models.py:58-66) where xa = x @ A^T.
+ * The adapter matrix is addressed as Bm[r, n] = lora_b[r*ldb_r + n*ldb_n] (fp16), so both
+ * lora_B.weight [N, R] (ldb_r = 1, ldb_n = R) and its transpose can be passed without a copy.
+ * bias, xa, lora_b may be NULL; R is 0 or a multiple of 8, at most 64.
+ * Both GEMM entry points need K % 128 == 0, N % 128 == 0, K*N < 2^33, and with g_idx == NULL also
  * groupsize % 64 == 0 and every |scale| < 64 (the sequential-group dequant forms s*q with a fused
  * multiply-add on 1024+q; pass g_idx to lift the restriction on the scales). */
 int q4_gemm_fwd_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                     const int32_t *g_idx, int groupsize, const void *bias,
-                    const void *xa, const void *lora_bt, int R,
+                    const void *xa, const void *lora_b, int ldb_r, int ldb_n, float lora_scale, int R,
                     void *y, int M, int K, int N, int G, void *stream);
 
 /* Backward GEMM (grad of the input):
- *   dx fp16 [M, K] = dy fp16 [M, N] @ W^T  (+ dyb fp16 [M, R] @ lora_a fp16 [R, K])
+ *   dx fp16 [M, K] = dy fp16 [M, N] @ W^T  (+ lora_scale * dyb fp16 [M, R] @ Am [R, K])
  * Replaces vecquant4recons_v2 + torch.matmul(grad_output, buffer.T)
  * (matmul_utils_4bit.py:114-126 with transpose=True, called from autograd_4bit.py:53) and the
- * adapter's contribution to grad_input, with dyb = scaling * dy @ B and lora_a = A. */
+ * adapter's contribution to grad_input, with dyb = dy @ B and Am[r, k] = lora_a[r*lda_r + k*lda_k]
+ * (lora_A.weight [R, K]: lda_r = K, lda_k = 1). */
 int q4_gemm_bwd_dx_f16(const void *dy, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                        const int32_t *g_idx, int groupsize,
-                       const void *dyb, const void *lora_a, int R,
+                       const void *dyb, const void *lora_a, int lda_r, int lda_k, float lora_scale, int R,
                        void *dx, int M, int K, int N, int G, void *stream);
 
 #ifdef __cplusplus

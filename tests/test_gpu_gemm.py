@@ -84,11 +84,16 @@ def test_gemm_lora_steps(oracle, M, K, N, r, act):
 
     xt, dyt = _t(x), _t(dy)
     a16, b16 = _t(A16), _t(B16)
-    xa = (xt @ a16.t()) * scaling
+    xa = xt @ a16.t()
     y = quant_hip.gemm_fwd(xt, t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 128, bias=_t(bias),
-                           xa=xa, lora_bt=b16.t().contiguous())
-    dyb = (dyt @ b16) * scaling
-    dx = quant_hip.gemm_bwd_dx(dyt, t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 128, dyb=dyb, lora_a=a16)
+                           xa=xa, lora_bt=b16.t(), lora_scale=scaling)          # strided view of B [N, r]
+    dyb = dyt @ b16
+    dx = quant_hip.gemm_bwd_dx(dyt, t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 128, dyb=dyb, lora_a=a16,
+                               lora_scale=scaling)
+    # a contiguous [r, N] copy of the adapter matrix must give the same bits as the strided view
+    y_c = quant_hip.gemm_fwd(xt, t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 128, bias=_t(bias),
+                             xa=xa, lora_bt=b16.t().contiguous(), lora_scale=scaling)
+    assert torch.equal(y, y_c)
     torch.cuda.synchronize()
     assert rel_err(y.cpu().numpy(), yref) <= TOL
     assert rel_err(dx.cpu().numpy(), dxref) <= TOL
