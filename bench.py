@@ -24,6 +24,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, GB/s
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
+# HBM bytes per launch of the headline GEMV kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# scaled by a 256 MiB copy (profiles/gemv_seq_mlp_decode_M1_hbm_traffic.md): 23 571 KiB read + 432 KiB written.
+GEMV_TRAFFIC_BYTES = 24578000
 
 
 def gemv_bytes(M, K, N, G, act_order=False):
@@ -270,6 +273,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="headline workload only (for profiling runs)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy: a kernel of known traffic for scaling rocprofv3 "
+                         "FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's share of the path only; --gpus must be 1 "
@@ -281,6 +287,13 @@ def main():
     torch.cuda.set_device(0)
     from alpaca_lora_4bit_amd import quant_hip  # noqa: F401  (fails loudly if the HIP library is missing)
 
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     head = bench_mlp_decode(1, args.steps, args.warmup)
     out = {
         "metric": "4-bit GEMV HBM GB/s (%peak) at M=1; LoRA fwd+bwd tokens/sec, LLaMA-7B shapes",
@@ -297,7 +310,7 @@ def main():
                    "bytes_per_step": head["bytes_per_step"]},
         "pct_of_hbm_peak": round(100 * head["gbs_wall"] / HBM_PEAK_GBS, 2),
         "roofline": {"bound": "hbm", "achieved": round(head["gbs_kernel"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(head["gbs_kernel"] / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(head["gbs_kernel"] / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES,
                      "kernel": "q4::gemv_seq_kernel<4, 0>", "bytes_per_launch": head["bytes_per_launch"],
                      "avg_launch_us": round(head["avg_launch_us"], 3)},
     }
