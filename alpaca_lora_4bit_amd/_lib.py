@@ -16,6 +16,7 @@ SIGNATURES = {
     "q4_abi_version": (_i, []),
     "q4_error_string": (ctypes.c_char_p, [_i]),
     "q4_dequant_f16": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp]),
+    "q4_permute_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "q4_gemv_workspace_bytes": (_sz, [_i, _i, _i]),
     "q4_gemv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "q4_gemm_fwd_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _f, _i, _vp, _i, _i, _i, _i, _vp]),

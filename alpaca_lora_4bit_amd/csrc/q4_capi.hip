@@ -6,6 +6,7 @@
 
 extern "C" {
 int q4_launch_dequant(const int32_t*, const int32_t*, const void*, const int32_t*, int, void*, int, int, hipStream_t);
+int q4_launch_permute_rows(const int32_t*, const int32_t*, int32_t*, int, int, hipStream_t);
 int q4_launch_gemv(const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, void*, int,
                    int, int, int, int, void*, hipStream_t);
 int q4_launch_gemm(int, const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, const void*,
@@ -51,6 +52,15 @@ extern "C" int q4_dequant_f16(const int32_t* qweight, const int32_t* qzeros, con
     if (misaligned(out)) return Q4_ERR_MISALIGNED;
     if (!g_idx && groupsize % 8 != 0) return Q4_ERR_BAD_SHAPE;
     return q4_launch_dequant(qweight, qzeros, scales, g_idx, groupsize, out, K, N, (hipStream_t)stream);
+}
+
+extern "C" int q4_permute_rows(const int32_t* qweight, const int32_t* perm, int32_t* out, int K, int N, void* stream) {
+    if (!qweight || !perm || !out) return Q4_ERR_NULL_POINTER;
+    if (K < 8 || N < 1 || (K % 8) != 0) return Q4_ERR_BAD_SHAPE;
+    if (qweight == out) return Q4_ERR_BAD_SHAPE;                      // not in place
+    if ((reinterpret_cast<uintptr_t>(qweight) | reinterpret_cast<uintptr_t>(perm) | reinterpret_cast<uintptr_t>(out)) & 3u)
+        return Q4_ERR_MISALIGNED;
+    return q4_launch_permute_rows(qweight, perm, out, K, N, (hipStream_t)stream);
 }
 
 extern "C" int q4_gemv_f16(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,

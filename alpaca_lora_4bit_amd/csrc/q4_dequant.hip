@@ -54,7 +54,37 @@ __global__ __launch_bounds__(256) void dequant_kernel(
     }
 }
 
+// Row permutation of the packed weights: out row p holds the codes of input row perm[p].
+// Used once per act-order layer to sort the rows by quantization group, after which the layer
+// runs through the sequential-group kernels with x gathered through the same permutation.
+// One thread per output word: eight nibbles gathered from eight source words (coalesced along N).
+__global__ __launch_bounds__(256) void permute_rows_kernel(const uint32_t* __restrict__ qweight,
+                                                           const int32_t* __restrict__ perm,
+                                                           uint32_t* __restrict__ out, int K, int N) {
+    const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long total = (long)(K >> 3) * N;
+    if (tid >= total) return;
+    const int kw = (int)(tid / N);
+    const int n = (int)(tid - (long)kw * N);
+    uint32_t word = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int k = perm[(kw << 3) + e];
+        const uint32_t src = qweight[(size_t)(k >> 3) * N + n];
+        word |= ((src >> ((k & 7) * 4)) & 0xFu) << (4 * e);
+    }
+    out[tid] = word;
+}
+
 }  // namespace q4
+
+extern "C" int q4_launch_permute_rows(const int32_t* qweight, const int32_t* perm, int32_t* out, int K, int N,
+                                      hipStream_t stream) {
+    const long total = (long)(K / 8) * N;
+    hipLaunchKernelGGL(q4::permute_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                       reinterpret_cast<const uint32_t*>(qweight), perm, reinterpret_cast<uint32_t*>(out), K, N);
+    return hipGetLastError() == hipSuccess ? 0 : -4;
+}
 
 extern "C" int q4_launch_dequant(const int32_t* qweight, const int32_t* qzeros, const void* scales,
                                  const int32_t* g_idx, int groupsize, void* out, int K, int N,

@@ -24,6 +24,12 @@ _lib.lib()  # fail at import time, loudly, if the HIP library is missing
 MAX_GEMV_ROWS = 16
 _workspaces = {}
 
+# Act-order layers (g_idx a real permutation): sort the packed rows by group once per layer and
+# run the sequential-group kernels on the sorted copy, gathering x through the permutation.
+# Costs a second copy of qweight (K*N/2 bytes) per act-order layer; set to False to use the
+# kernels that gather (scale, zero) through g_idx row by row instead.
+actorder_repack = True
+
 
 def _ptr(t):
     return 0 if t is None else t.data_ptr()
@@ -103,6 +109,41 @@ def _gemm_gidx_arg(g_idx, groupsize, G, K, scales):
     return g_idx.data_ptr(), int(groupsize or 0), g_idx
 
 
+def sorted_layer(qweight, g_idx, G):
+    """(perm, inv_perm, qweight_sorted, groupsize) for an act-order layer whose groups all own
+    exactly K/G rows (what GPTQ's act-order produces), else None.  perm[p] is the original index of
+    sorted row p.  Built once per (g_idx, qweight) pair and cached on the g_idx tensor object."""
+    K, N = qweight.shape[0] * 8, qweight.shape[1]
+    key = (g_idx._version, qweight._version, qweight.data_ptr())
+    cached = getattr(g_idx, "_q4_sorted", None)
+    if cached is not None and cached[0] == key:
+        return cached[1]
+    plan = None
+    if K % G == 0 and (K // G) % 64 == 0:
+        counts = torch.bincount(g_idx.long(), minlength=G)
+        if bool((counts == K // G).all()):
+            perm = torch.argsort(g_idx.long(), stable=True).to(torch.int32).contiguous()
+            inv = torch.empty_like(perm)
+            inv[perm.long()] = torch.arange(K, device=perm.device, dtype=torch.int32)
+            qs = torch.empty_like(qweight)
+            with torch.cuda.device(qweight.device):
+                rc = _lib.lib().q4_permute_rows(qweight.data_ptr(), perm.data_ptr(), qs.data_ptr(), K, N,
+                                                _stream(qweight.device))
+            _lib.check(rc, "q4_permute_rows")
+            plan = (perm, inv, qs, K // G)
+    g_idx._q4_sorted = (key, plan)
+    return plan
+
+
+def _actorder_plan(qweight, scales, g_idx, groupsize, G):
+    """The sorted-copy plan when this call should use it, else None."""
+    if g_idx is None or not actorder_repack:
+        return None
+    if classify_g_idx(g_idx, groupsize, G) != "gidx" or not scales_fit_fused_dequant(scales):
+        return None
+    return sorted_layer(qweight, g_idx, G)
+
+
 def _gidx_arg(g_idx, groupsize, G, need_multiple=32):
     """Returns (pointer-or-0, groupsize) to hand to the C ABI."""
     if g_idx is None:
@@ -172,7 +213,13 @@ def gemv(x, qweight, qzeros, scales, g_idx=None, groupsize=None, out=None, accum
         out = torch.empty(_out_shape(out_shape, M, N), dtype=torch.float16, device=dev)
     _require(out.dtype == torch.float16 and out.numel() == M * N and out.shape[-1] == N and out.is_contiguous()
              and out.device == dev, "out must be a contiguous float16 [..., N] tensor with M rows on the same device")
-    gp, gs = _gidx_arg(g_idx, groupsize, G)
+    plan = _actorder_plan(qweight, scales, g_idx, groupsize, G)
+    if plan is not None:
+        perm, _, qweight, gs_sorted = plan
+        x2 = x2.index_select(1, perm)
+        gp, gs = 0, gs_sorted
+    else:
+        gp, gs = _gidx_arg(g_idx, groupsize, G)
     L = _lib.lib()
     nbytes = L.q4_gemv_workspace_bytes(M, K, N)
     with torch.cuda.device(dev):
@@ -209,7 +256,13 @@ def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, 
         _require(bias.dtype == torch.float16 and tuple(bias.shape) == (N,) and bias.is_contiguous()
                  and bias.device == dev, "bias must be a contiguous float16 [N] tensor on the same device")
     xa, lora_bt, R, sr, sc = _lora_pair(xa, lora_bt, M, N, dev)
-    gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
+    plan = _actorder_plan(qweight, scales, g_idx, groupsize, G)
+    if plan is not None:
+        perm, _, qweight, gs_sorted = plan
+        x2 = x2.index_select(1, perm)
+        gp, gs = 0, gs_sorted
+    else:
+        gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
     out = torch.empty(_out_shape(out_shape, M, N), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().q4_gemm_fwd_f16(x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
@@ -225,6 +278,13 @@ def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=Non
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     dy2 = _flat_half(dy, N, dev, "grad_output")
     M = dy2.shape[0]
+    plan = _actorder_plan(qweight, scales, g_idx, groupsize, G)
+    if plan is not None:
+        # dx comes out in sorted row order and is scattered back; the adapter matrix [R, K] is gathered too
+        perm, inv, qs, gs_sorted = plan
+        la_sorted = None if lora_a is None else lora_a.index_select(1, perm)
+        dx_sorted = gemm_bwd_dx(dy2, qs, qzeros, scales, None, gs_sorted, dyb=dyb, lora_a=la_sorted, lora_scale=lora_scale)
+        return dx_sorted.index_select(1, inv).reshape(_out_shape(out_shape, M, K))
     dyb, lora_a, R, sr, sc = _lora_pair(dyb, lora_a, M, K, dev)
     gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
     out = torch.empty(_out_shape(out_shape, M, K), dtype=torch.float16, device=dev)

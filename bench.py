@@ -325,8 +325,12 @@ def main():
         c0h = bench_single_gemv(4096, 4096, 1, False, 20, 1)
         extra["config0_K4096_N4096_M1_hot_cache"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in c0h.items()}
         for M in (1, 16):
-            c3 = bench_single_gemv(5120, 13824, M, True, 10, 12)
+            c3 = bench_single_gemv(5120, 13824, M, True, 10, 12)     # includes the gather of x through the row sort
             extra[f"config3_actorder_K5120_N13824_M{M}"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in c3.items()}
+        quant_hip.actorder_repack = False
+        c3g = bench_single_gemv(5120, 13824, 1, True, 10, 12)
+        extra["config3_actorder_K5120_N13824_M1_gather_kernel"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in c3g.items()}
+        quant_hip.actorder_repack = True
         lo = bench_lora_step(20)
         extra["config2_lora_fwd_bwd_M2048"] = {k: round(v, 4) for k, v in lo.items()}
         gm = bench_gemm_only(2048, 4096, 4096, False, 20)

@@ -49,6 +49,13 @@ int q4_dequant_f16(const int32_t *qweight, const int32_t *qzeros, const void *sc
                    const int32_t *g_idx, int groupsize, void *out,
                    int K, int N, int G, void *stream);
 
+/* Row permutation of packed weights: out int32 [K/8, N] holds in row p the 4-bit codes of row perm[p]
+ * of qweight (perm int32 [K], a permutation of 0..K-1, not checked).  No counterpart in the reference:
+ * it is the one-time repack that lets an act-order layer (rows assigned to groups through g_idx,
+ * autograd_4bit.py:185, quant_cuda_kernel.cu:1143) run through the sequential-group kernels -- sort
+ * the rows by group, gather x through the same permutation.  Not in place. */
+int q4_permute_rows(const int32_t *qweight, const int32_t *perm, int32_t *out, int K, int N, void *stream);
+
 /* Decode GEMV / skinny GEMM, 1 <= M <= 16:  y fp16 [M, N] = x fp16 [M, K] @ W  (fp32 accumulate).
  * If accumulate != 0 the product is added to the existing contents of y.
  * Replaces quant_cuda.vecquant4matmul / vecquant4matmul_faster / vecquant4matmul_old_faster

@@ -1,0 +1,91 @@
+"""Act-order layers: the one-time row sort (q4_permute_rows + gathered x) and the direct
+gather kernels must both agree with the CPU oracle; the repack itself is bit-exact."""
+import numpy as np
+import pytest
+
+from conftest import rel_err, to_cuda_layer
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+@pytest.fixture(params=[True, False], ids=["repack", "gather"])
+def repack(request):
+    from alpaca_lora_4bit_amd import quant_hip
+    old = quant_hip.actorder_repack
+    quant_hip.actorder_repack = request.param
+    yield request.param
+    quant_hip.actorder_repack = old
+
+
+def test_permute_rows_bit_exact(oracle):
+    import torch
+    from alpaca_lora_4bit_amd import _lib, quant_hip
+    rng = np.random.default_rng(3)
+    K, N = 512, 192
+    codes = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    perm = rng.permutation(K).astype(np.int32)
+    qw = torch.from_numpy(oracle.pack_qweight(codes)).cuda()
+    out = torch.empty_like(qw)
+    rc = _lib.lib().q4_permute_rows(qw.data_ptr(), torch.from_numpy(perm).cuda().data_ptr(), out.data_ptr(), K, N,
+                                    torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    assert np.array_equal(out.cpu().numpy(), oracle.pack_qweight(codes[perm]))
+    assert _lib.lib().q4_permute_rows(qw.data_ptr(), qw.data_ptr(), qw.data_ptr(), K, N, None) == -2   # in place refused
+
+
+def test_sorted_layer_plan(oracle):
+    """Sorted copy dequantizes (with sequential groups) to the row-permuted dense weight."""
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    layer = oracle.make_layer(1024, 256, 128, act_order=True, seed=12)
+    t = to_cuda_layer(layer)
+    plan = quant_hip.sorted_layer(t["qweight"], t["g_idx"], 8)
+    assert plan is not None
+    perm, inv, qs, gs = plan
+    assert gs == 128 and torch.equal(perm.long()[inv.long()], torch.arange(1024, device="cuda"))
+    assert torch.equal(t["g_idx"].long()[perm.long()], torch.arange(1024, device="cuda") // 128)
+    W = oracle.dequant_v2(layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
+    Ws = quant_hip.dequant(qs, t["qzeros"], t["scales"], None, 128).cpu().numpy()
+    assert np.array_equal(Ws.view(np.uint16), W[perm.cpu().numpy()].view(np.uint16))
+    assert quant_hip.sorted_layer(t["qweight"], t["g_idx"], 8) is plan                # cached
+    # groups of unequal size cannot be sorted into the sequential layout
+    g2 = t["g_idx"].clone()
+    g2[0] = (g2[0] + 1) % 8
+    assert quant_hip.sorted_layer(t["qweight"], g2, 8) is None
+
+
+@pytest.mark.parametrize("K,N,M", [(5120, 13824, 1), (5120, 13824, 16), (512, 256, 5)])
+def test_actorder_gemv(oracle, repack, K, N, M):
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    layer = oracle.make_layer(K, N, 128, act_order=True, seed=K + N)
+    t = to_cuda_layer(layer)
+    x = oracle.make_activations(M, K, seed=M)
+    ref = oracle.matmul_recons(x, layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
+    y = quant_hip.gemv(torch.from_numpy(x).cuda(), t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 128)
+    assert rel_err(y.cpu().numpy(), ref) <= TOL
+
+
+@pytest.mark.parametrize("K,N,M", [(5120, 13824, 512), (512, 384, 40)])
+def test_actorder_gemm_forward_backward_lora(oracle, repack, K, N, M):
+    """Config 3 (M=512) forward, plus backward-dx with the adapter term through the permutation."""
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    layer = oracle.make_layer(K, N, 128, act_order=True, seed=K + N + 7)
+    t = to_cuda_layer(layer)
+    A, B = oracle.make_lora(K, N, 8, seed=5)
+    A16, B16 = A.astype(np.float16), B.astype(np.float16)
+    x = oracle.make_activations(M, K, seed=1)
+    dy = oracle.make_activations(M, N, seed=2)
+    W = oracle.dequant_v2(layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"]).astype(np.float64)
+    yref = oracle.lora_forward(x, W, A16, B16, 2.0)
+    dxref, _, _ = oracle.lora_backward(x, dy, W, A16, B16, 2.0)
+    xt, dyt = torch.from_numpy(x).cuda(), torch.from_numpy(dy).cuda()
+    a16, b16 = torch.from_numpy(A16).cuda(), torch.from_numpy(B16).cuda()
+    y = quant_hip.gemm_fwd(xt, t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 128, xa=xt @ a16.t(),
+                           lora_bt=b16.t(), lora_scale=2.0)
+    dx = quant_hip.gemm_bwd_dx(dyt, t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 128, dyb=dyt @ b16,
+                               lora_a=a16, lora_scale=2.0)
+    assert rel_err(y.cpu().numpy(), yref) <= TOL
+    assert rel_err(dx.cpu().numpy(), dxref) <= TOL
