@@ -176,6 +176,29 @@ def make_quant_for_4bit_autograd(module, names, name='', groupsize=-1, is_v1_mod
             make_quant_for_4bit_autograd(child, names, path, groupsize=groupsize, is_v1_model=is_v1_model, bits=bits)
 
 
+def fuse_quant_linears(layers):
+    """One Autograd4bitQuantLinear computing the concatenation of the outputs of `layers`
+    (same in_features, groupsize and g_idx): q/k/v or gate/up as a single, wider launch.
+    Every packed tensor is N-minor, so the fusion is a plain concatenation along N; it is what the
+    reference's make_quant_attn / make_fused_mlp do (model_attn_mlp_patch.py:88-100, 180-190)."""
+    first = layers[0]
+    for l in layers[1:]:
+        if (l.in_features, l.groupsize, l.bits, l.is_v1_model) != (first.in_features, first.groupsize, first.bits,
+                                                                   first.is_v1_model):
+            raise ValueError('layers to fuse must share in_features, groupsize, bits and layout')
+        if first.is_v1_model or not torch.equal(l.g_idx, first.g_idx):
+            raise ValueError('layers to fuse must be v2 layers with identical g_idx')
+    fused = Autograd4bitQuantLinear(first.in_features, sum(l.out_features for l in layers), groupsize=first.groupsize,
+                                    is_v1_model=False, bits=first.bits)
+    fused.qweight = torch.cat([l.qweight for l in layers], dim=1).contiguous()
+    fused.qzeros = torch.cat([l.qzeros for l in layers], dim=1).contiguous()
+    fused.scales = torch.cat([l.scales for l in layers], dim=1).contiguous()
+    fused.bias = torch.cat([l.bias for l in layers], dim=0).contiguous()
+    fused.g_idx = first.g_idx
+    fused.disable_bias = all(l.disable_bias for l in layers)
+    return fused
+
+
 def _cast_quant_buffers(model, dtype):
     for _, m in model.named_modules():
         if isinstance(m, Autograd4bitQuantLinear):
@@ -222,22 +245,29 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
         bwd   dyb = dy @ B     [M, r]   then  dx = [dy | dyb] @ [W^T ; scaling * A]
               dA  = scaling * dyb^T @ x   [r, K]        dB = scaling * dy^T @ xa   [N, r]
     A: lora_A.weight [r, K], B: lora_B.weight [N, r] (any float dtype; products run in fp16
-    with fp32 accumulation, like the reference under autocast).  The adapter matrices go to the
-    kernels as strided views: no transposed or pre-scaled copies are made."""
+    with fp32 accumulation, like the reference under autocast).  fp32 / fp16 adapter matrices are
+    read in place by the kernels through strides: no cast, transposed or pre-scaled copies."""
 
     @staticmethod
-    @custom_fwd(device_type='cuda', cast_inputs=torch.float16)
+    def _kernel_dtype(w):
+        return w if w.dtype in (torch.float16, torch.float32) else w.float()
+
+    @staticmethod
+    @custom_fwd(device_type='cuda', cast_inputs=None)
     def forward(ctx, x, qweight, scales, zeros, g_idx, bias, lora_a, lora_b, scaling, groupsize):
         K, N = qweight.shape[0] * 8, qweight.shape[1]
         x2 = x.reshape(-1, K)
         if x2.dtype != torch.float16:
             x2 = x2.half()
-        a16 = lora_a.to(torch.float16)
-        b16 = lora_b.to(torch.float16)
-        xa = torch.mm(x2, a16.t())
+        x2 = x2.contiguous()
+        if bias is not None and bias.dtype != torch.float16:
+            bias = bias.half()
+        a = AutogradMatmul4bitLora._kernel_dtype(lora_a.detach())
+        b = AutogradMatmul4bitLora._kernel_dtype(lora_b.detach())
+        xa = quant_hip.lora_down(x2, a)
         y = quant_hip.gemm_fwd(x2, qweight, zeros, scales, g_idx, groupsize, bias=bias,
-                               xa=xa, lora_bt=b16.t(), lora_scale=scaling, out_shape=tuple(x.shape[:-1]) + (N,))
-        ctx.save_for_backward(x2, xa, qweight, scales, zeros, g_idx, a16, b16)
+                               xa=xa, lora_bt=b.t(), lora_scale=scaling, out_shape=tuple(x.shape[:-1]) + (N,))
+        ctx.save_for_backward(x2, xa, qweight, scales, zeros, g_idx, a, b)
         ctx.scaling = scaling
         ctx.groupsize = groupsize
         ctx.ab_dtypes = (lora_a.dtype, lora_b.dtype)
@@ -246,20 +276,29 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
     @staticmethod
     @custom_bwd(device_type='cuda')
     def backward(ctx, grad_output):
-        x2, xa, qweight, scales, zeros, g_idx, a16, b16 = ctx.saved_tensors
+        x2, xa, qweight, scales, zeros, g_idx, a, b = ctx.saved_tensors
         N = qweight.shape[1]
         dy = grad_output.reshape(-1, N)
         if dy.dtype != torch.float16:
             dy = dy.half()
         dy = dy.contiguous()
-        dyb = torch.mm(dy, b16)
+        dyb = quant_hip.lora_down(dy, b.t())
         dx = da = db = None
         if ctx.needs_input_grad[0]:
-            dx = quant_hip.gemm_bwd_dx(dy, qweight, zeros, scales, g_idx, ctx.groupsize, dyb=dyb, lora_a=a16,
+            dx = quant_hip.gemm_bwd_dx(dy, qweight, zeros, scales, g_idx, ctx.groupsize, dyb=dyb, lora_a=a,
                                        lora_scale=ctx.scaling,
                                        out_shape=tuple(grad_output.shape[:-1]) + (qweight.shape[0] * 8,))
+        r = a.shape[0]
         if ctx.needs_input_grad[6]:
-            da = torch.addmm(a16, dyb.t(), x2, beta=0.0, alpha=ctx.scaling).to(ctx.ab_dtypes[0])
+            if r in quant_hip.LORA_GRAD_RANKS:
+                da = quant_hip.lora_grad(dyb, x2, ctx.scaling)
+            else:
+                da = torch.mm(dyb.t(), x2).float().mul_(ctx.scaling)
+            da = da.to(ctx.ab_dtypes[0])
         if ctx.needs_input_grad[7]:
-            db = torch.addmm(b16, dy.t(), xa, beta=0.0, alpha=ctx.scaling).to(ctx.ab_dtypes[1])
+            if r in quant_hip.LORA_GRAD_RANKS:
+                db = quant_hip.lora_grad(xa, dy, ctx.scaling, transposed=True)
+            else:
+                db = torch.mm(dy.t(), xa).float().mul_(ctx.scaling)
+            db = db.to(ctx.ab_dtypes[1])
         return dx, None, None, None, None, None, da, db, None, None

@@ -10,7 +10,9 @@ int q4_launch_permute_rows(const int32_t*, const int32_t*, int32_t*, int, int, h
 int q4_launch_gemv(const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, void*, int,
                    int, int, int, int, void*, hipStream_t);
 int q4_launch_gemm(int, const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, const void*,
-                   const void*, const void*, int, int, float, int, void*, int, int, int, int, hipStream_t);
+                   const void*, const void*, int, int, int, float, int, void*, int, int, int, int, hipStream_t);
+int q4_launch_lora_down(const void*, const void*, int, int, int, void*, int, int, int, hipStream_t);
+int q4_launch_lora_grad(const void*, const void*, float*, int, int, float, int, int, int, void*, hipStream_t);
 }
 
 namespace {
@@ -30,7 +32,7 @@ int check_layer(const void* qweight, const void* qzeros, const void* scales, con
 }
 }  // namespace
 
-extern "C" int q4_abi_version(void) { return 2; }
+extern "C" int q4_abi_version(void) { return 3; }
 
 extern "C" const char* q4_error_string(int code) {
     switch (code) {
@@ -79,7 +81,7 @@ extern "C" int q4_gemv_f16(const void* x, const int32_t* qweight, const int32_t*
 
 static int gemm_common(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros, const void* scales,
                        const int32_t* g_idx, int groupsize, const void* bias, const void* la, const void* lb,
-                       int lb_sr, int lb_sc, float lb_scale, int R,
+                       int lb_sr, int lb_sc, int lb_is_f32, float lb_scale, int R,
                        void* out, int M, int K, int N, int G, void* stream) {
     int rc = check_layer(qweight, qzeros, scales, g_idx, groupsize, K, N, G);
     if (rc != Q4_OK) return rc;
@@ -92,24 +94,48 @@ static int gemm_common(int fwd, const void* act, const int32_t* qweight, const i
     if ((la != nullptr) != (lb != nullptr)) return Q4_ERR_NULL_POINTER;
     if (la && (R < 8 || R > 64 || (R % 8) != 0)) return Q4_ERR_BAD_SHAPE;
     if (misaligned(act) || misaligned(out) || (la && misaligned(la))) return Q4_ERR_MISALIGNED;
-    if (lb && (reinterpret_cast<uintptr_t>(lb) & 1u)) return Q4_ERR_MISALIGNED;
+    if (lb && (reinterpret_cast<uintptr_t>(lb) & (lb_is_f32 ? 3u : 1u))) return Q4_ERR_MISALIGNED;
     if (lb && (lb_sr < 1 || lb_sc < 1)) return Q4_ERR_BAD_SHAPE;
-    return q4_launch_gemm(fwd, act, qweight, qzeros, scales, g_idx, groupsize, bias, la, lb, lb_sr, lb_sc, lb_scale, R,
-                          out, M, K, N, G, (hipStream_t)stream);
+    return q4_launch_gemm(fwd, act, qweight, qzeros, scales, g_idx, groupsize, bias, la, lb, lb_sr, lb_sc, lb_is_f32,
+                          lb_scale, R, out, M, K, N, G, (hipStream_t)stream);
 }
 
 extern "C" int q4_gemm_fwd_f16(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
                                const int32_t* g_idx, int groupsize, const void* bias,
-                               const void* xa, const void* lora_b, int ldb_r, int ldb_n, float lora_scale, int R,
-                               void* y, int M, int K, int N, int G, void* stream) {
-    return gemm_common(1, x, qweight, qzeros, scales, g_idx, groupsize, bias, xa, lora_b, ldb_r, ldb_n, lora_scale, R,
-                       y, M, K, N, G, stream);
+                               const void* xa, const void* lora_b, int ldb_r, int ldb_n, int lora_is_f32,
+                               float lora_scale, int R, void* y, int M, int K, int N, int G, void* stream) {
+    return gemm_common(1, x, qweight, qzeros, scales, g_idx, groupsize, bias, xa, lora_b, ldb_r, ldb_n, lora_is_f32,
+                       lora_scale, R, y, M, K, N, G, stream);
 }
 
 extern "C" int q4_gemm_bwd_dx_f16(const void* dy, const int32_t* qweight, const int32_t* qzeros, const void* scales,
                                   const int32_t* g_idx, int groupsize,
-                                  const void* dyb, const void* lora_a, int lda_r, int lda_k, float lora_scale, int R,
-                                  void* dx, int M, int K, int N, int G, void* stream) {
-    return gemm_common(0, dy, qweight, qzeros, scales, g_idx, groupsize, nullptr, dyb, lora_a, lda_r, lda_k, lora_scale, R,
-                       dx, M, K, N, G, stream);
+                                  const void* dyb, const void* lora_a, int lda_r, int lda_k, int lora_is_f32,
+                                  float lora_scale, int R, void* dx, int M, int K, int N, int G, void* stream) {
+    return gemm_common(0, dy, qweight, qzeros, scales, g_idx, groupsize, nullptr, dyb, lora_a, lda_r, lda_k, lora_is_f32,
+                       lora_scale, R, dx, M, K, N, G, stream);
+}
+
+extern "C" int q4_lora_down_f16(const void* in, const void* w, int w_sr, int w_sc, int w_is_f32, void* out,
+                                int M, int C, int R, void* stream) {
+    if (!in || !w || !out) return Q4_ERR_NULL_POINTER;
+    if (M < 1 || C < 32 || (C % 32) != 0 || R < 1 || R > 64 || w_sr < 1 || w_sc < 1) return Q4_ERR_BAD_SHAPE;
+    if (misaligned(in) || (reinterpret_cast<uintptr_t>(out) & 1u) || (reinterpret_cast<uintptr_t>(w) & (w_is_f32 ? 3u : 1u)))
+        return Q4_ERR_MISALIGNED;
+    return q4_launch_lora_down(in, w, w_sr, w_sc, w_is_f32, out, M, C, R, (hipStream_t)stream);
+}
+
+extern "C" size_t q4_lora_grad_workspace_bytes(int R, int C) {
+    if (R < 1 || C < 1) return 0;
+    return (size_t)R * (size_t)C * sizeof(unsigned long long);
+}
+
+extern "C" int q4_lora_grad_f32(const void* p, const void* in, float* out, int o_sr, int o_sc, float alpha,
+                                int M, int C, int R, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!p || !in || !out) return Q4_ERR_NULL_POINTER;
+    if (M < 1 || C < 8 || (C % 8) != 0 || (R != 8 && R != 16) || o_sr < 1 || o_sc < 1) return Q4_ERR_BAD_SHAPE;
+    if (misaligned(p) || misaligned(in) || (reinterpret_cast<uintptr_t>(out) & 3u)) return Q4_ERR_MISALIGNED;
+    if (!workspace || workspace_bytes < q4_lora_grad_workspace_bytes(R, C)) return Q4_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
+    return q4_launch_lora_grad(p, in, out, o_sr, o_sc, alpha, M, C, R, workspace, (hipStream_t)stream);
 }

@@ -50,14 +50,17 @@ struct GemmArgs {
     int groupsize;
     const half_t* bias;       // fwd only, [N] or null
     const half_t* la;         // fwd: xa [M,R]     bwd: dyb [M,R]   (or null)
-    const half_t* lb;         // adapter matrix, element (r, c) at lb[r*lb_sr + c*lb_sc]; fwd: c = n, bwd: c = k
-    int lb_sr, lb_sc;
+    const void* lb;           // adapter matrix (fp16 or fp32), element (r, c) at lb[r*lb_sr + c*lb_sc]; fwd: c = n, bwd: c = k
+    int lb_sr, lb_sc, lb_is_f32;
     float lb_scale;           // multiplied into the adapter matrix when it is staged in LDS
     int R;
     half_t* out;              // fwd: y [M,N]      bwd: dx [M,K]
     int M, K, N, G;
 };
 
+__device__ __forceinline__ float adapter_at(const GemmArgs& a, size_t idx) {
+    return a.lb_is_f32 ? reinterpret_cast<const float*>(a.lb)[idx] : (float)reinterpret_cast<const half_t*>(a.lb)[idx];
+}
 __device__ __forceinline__ rsrc_t make_rsrc(const void* p, unsigned bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, kRsrcFlags);
 }
@@ -176,7 +179,7 @@ struct FwdSlab {
     __device__ __forceinline__ void store_lora(const GemmArgs& a, int n0, half_t* sB, int t) const {
         for (int idx = t; idx < BN * BK; idx += NT) {
             const int r = idx >> 7, c = idx & 127;
-            sB[c * LDS_STRIDE + r] = (r < a.R) ? (half_t)(a.lb_scale * (float)a.lb[(size_t)r * a.lb_sr + (size_t)(n0 + c) * a.lb_sc])
+            sB[c * LDS_STRIDE + r] = (r < a.R) ? (half_t)(a.lb_scale * adapter_at(a, (size_t)r * a.lb_sr + (size_t)(n0 + c) * a.lb_sc))
                                                : (half_t)0.f;
         }
     }
@@ -264,7 +267,7 @@ struct BwdSlab {
     __device__ __forceinline__ void store_lora(const GemmArgs& a, int kout0, half_t* sB, int t) const {
         for (int idx = t; idx < BN * BK; idx += NT) {
             const int r = idx >> 7, c = idx & 127;
-            sB[c * LDS_STRIDE + r] = (r < a.R) ? (half_t)(a.lb_scale * (float)a.lb[(size_t)r * a.lb_sr + (size_t)(kout0 + c) * a.lb_sc])
+            sB[c * LDS_STRIDE + r] = (r < a.R) ? (half_t)(a.lb_scale * adapter_at(a, (size_t)r * a.lb_sr + (size_t)(kout0 + c) * a.lb_sc))
                                                : (half_t)0.f;
         }
     }
@@ -484,7 +487,7 @@ static hipError_t launch_gemm_cfg(int cfg, const GemmArgs& a, int nout, hipStrea
 
 extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros,
                               const void* scales, const int32_t* g_idx, int groupsize, const void* bias,
-                              const void* la, const void* lb, int lb_sr, int lb_sc, float lb_scale, int R,
+                              const void* la, const void* lb, int lb_sr, int lb_sc, int lb_is_f32, float lb_scale, int R,
                               void* out, int M, int K, int N, int G, hipStream_t stream) {
     using namespace q4;
     GemmArgs a;
@@ -496,8 +499,8 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     a.groupsize = groupsize;
     a.bias = reinterpret_cast<const half_t*>(bias);
     a.la = reinterpret_cast<const half_t*>(la);
-    a.lb = reinterpret_cast<const half_t*>(lb);
-    a.lb_sr = lb_sr; a.lb_sc = lb_sc; a.lb_scale = lb_scale;
+    a.lb = lb;
+    a.lb_sr = lb_sr; a.lb_sc = lb_sc; a.lb_is_f32 = lb_is_f32; a.lb_scale = lb_scale;
     a.R = (la && lb) ? R : 0;
     a.out = reinterpret_cast<half_t*>(out);
     a.M = M; a.K = K; a.N = N; a.G = G;

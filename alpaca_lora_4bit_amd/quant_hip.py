@@ -230,32 +230,38 @@ def gemv(x, qweight, qzeros, scales, g_idx=None, groupsize=None, out=None, accum
     return out
 
 
+def _adapter_dtype_flag(w, what):
+    _require(w.dtype in (torch.float16, torch.float32), f"{what} must be float16 or float32")
+    return int(w.dtype == torch.float32)
+
+
 def _lora_pair(la, lb, rows, cols, dev):
-    """la: [rows, R] fp16 contiguous; lb: [R, cols] fp16 with any (positive) strides."""
+    """la: [rows, R] fp16 contiguous; lb: [R, cols] fp16 or fp32 with any (positive) strides."""
     if la is None and lb is None:
-        return None, None, 0, 0, 0
+        return None, None, 0, 0, 0, 0
     _require(la is not None and lb is not None, "both LoRA operands are required")
     R = la.shape[-1]
-    _require(la.dtype == torch.float16 and lb.dtype == torch.float16, "LoRA operands must be float16")
+    _require(la.dtype == torch.float16, "the rank-R activation operand must be float16")
+    is_f32 = _adapter_dtype_flag(lb, "the adapter matrix")
     _require(tuple(la.shape) == (rows, R) and tuple(lb.shape) == (R, cols), "LoRA operand shapes do not match")
     _require(R % 8 == 0 and 8 <= R <= 64, "LoRA rank must be a multiple of 8 in [8, 64] for the fused path")
     _require(la.is_contiguous() and la.device == dev and lb.device == dev, "LoRA operands must be on the same device")
     sr, sc = lb.stride()
     _require(sr >= 1 and sc >= 1, "the adapter matrix must have positive strides")
-    return la, lb, R, int(sr), int(sc)
+    return la, lb, R, int(sr), int(sc), is_f32
 
 
 def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, xa=None, lora_bt=None,
              lora_scale=1.0, out_shape=None):
     """y fp16 [M, N] = x @ W (+ bias) (+ lora_scale * xa @ lora_bt), W dequantized tile by tile in LDS.
-    `lora_bt` is the adapter matrix as an [R, N] view with any strides (e.g. `lora_B.weight.half().t()`)."""
+    `lora_bt` is the adapter matrix as an [R, N] fp16/fp32 view with any strides (e.g. `lora_B.weight.t()`)."""
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     x2 = _flat_half(x, K, dev, "x")
     M = x2.shape[0]
     if bias is not None:
         _require(bias.dtype == torch.float16 and tuple(bias.shape) == (N,) and bias.is_contiguous()
                  and bias.device == dev, "bias must be a contiguous float16 [N] tensor on the same device")
-    xa, lora_bt, R, sr, sc = _lora_pair(xa, lora_bt, M, N, dev)
+    xa, lora_bt, R, sr, sc, f32 = _lora_pair(xa, lora_bt, M, N, dev)
     plan = _actorder_plan(qweight, scales, g_idx, groupsize, G)
     if plan is not None:
         perm, _, qweight, gs_sorted = plan
@@ -266,7 +272,7 @@ def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, 
     out = torch.empty(_out_shape(out_shape, M, N), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().q4_gemm_fwd_f16(x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
-                                        gp, gs, _ptr(bias), _ptr(xa), _ptr(lora_bt), sr, sc, float(lora_scale), R,
+                                        gp, gs, _ptr(bias), _ptr(xa), _ptr(lora_bt), sr, sc, f32, float(lora_scale), R,
                                         out.data_ptr(), M, K, N, G, _stream(dev))
     _lib.check(rc, "q4_gemm_fwd_f16")
     return out
@@ -285,14 +291,64 @@ def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=Non
         la_sorted = None if lora_a is None else lora_a.index_select(1, perm)
         dx_sorted = gemm_bwd_dx(dy2, qs, qzeros, scales, None, gs_sorted, dyb=dyb, lora_a=la_sorted, lora_scale=lora_scale)
         return dx_sorted.index_select(1, inv).reshape(_out_shape(out_shape, M, K))
-    dyb, lora_a, R, sr, sc = _lora_pair(dyb, lora_a, M, K, dev)
+    dyb, lora_a, R, sr, sc, f32 = _lora_pair(dyb, lora_a, M, K, dev)
     gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
     out = torch.empty(_out_shape(out_shape, M, K), dtype=torch.float16, device=dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().q4_gemm_bwd_dx_f16(dy2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
-                                           gp, gs, _ptr(dyb), _ptr(lora_a), sr, sc, float(lora_scale), R,
+                                           gp, gs, _ptr(dyb), _ptr(lora_a), sr, sc, f32, float(lora_scale), R,
                                            out.data_ptr(), M, K, N, G, _stream(dev))
     _lib.check(rc, "q4_gemm_bwd_dx_f16")
+    return out
+
+
+LORA_GRAD_RANKS = (8, 16)
+
+
+def lora_down(inp, w):
+    """out fp16 [M, R] = inp fp16 [M, C] @ w^T for an adapter matrix view w [R, C] (fp16/fp32, any positive
+    strides): xa = x @ A^T with w = lora_A.weight, dyb = dy @ B with w = lora_B.weight.t()  (models.py:66)."""
+    _require(inp.is_cuda and inp.dtype == torch.float16 and inp.dim() == 2 and inp.is_contiguous(),
+             "inp must be a contiguous float16 [M, C] CUDA tensor")
+    M, C = inp.shape
+    _require(w.dim() == 2 and w.shape[1] == C and w.device == inp.device, "w must be an [R, C] view on the same device")
+    R = w.shape[0]
+    _require(1 <= R <= 64 and C % 32 == 0 and M >= 1, "lora_down needs 1 <= R <= 64 and C % 32 == 0")
+    f32 = _adapter_dtype_flag(w, "w")
+    sr, sc = w.stride()
+    _require(sr >= 1 and sc >= 1, "w must have positive strides")
+    out = torch.empty((M, R), dtype=torch.float16, device=inp.device)
+    with torch.cuda.device(inp.device):
+        rc = _lib.lib().q4_lora_down_f16(inp.data_ptr(), w.data_ptr(), int(sr), int(sc), f32, out.data_ptr(),
+                                         M, C, R, _stream(inp.device))
+    _lib.check(rc, "q4_lora_down_f16")
+    return out
+
+
+def lora_grad(p, inp, alpha, transposed=False):
+    """alpha * p^T @ inp in fp32 for p fp16 [M, R], inp fp16 [M, C], R in LORA_GRAD_RANKS.  Returns [R, C], or
+    with transposed=True the same values stored as a contiguous [C, R] tensor (lora_B.weight's layout)."""
+    _require(p.is_cuda and p.dtype == torch.float16 and p.dim() == 2 and p.is_contiguous(),
+             "p must be a contiguous float16 [M, R] CUDA tensor")
+    _require(inp.dtype == torch.float16 and inp.dim() == 2 and inp.is_contiguous() and inp.device == p.device
+             and inp.shape[0] == p.shape[0], "inp must be a contiguous float16 [M, C] tensor on the same device")
+    M, R = p.shape
+    C = inp.shape[1]
+    _require(R in LORA_GRAD_RANKS and C % 8 == 0 and M >= 1, "lora_grad needs R in (8, 16) and C % 8 == 0")
+    dev = p.device
+    if transposed:
+        out = torch.empty((C, R), dtype=torch.float32, device=dev)
+        sr, sc = 1, R
+    else:
+        out = torch.empty((R, C), dtype=torch.float32, device=dev)
+        sr, sc = C, 1
+    L = _lib.lib()
+    nbytes = L.q4_lora_grad_workspace_bytes(R, C)
+    with torch.cuda.device(dev):
+        ws = _workspace(dev, nbytes)
+        rc = L.q4_lora_grad_f32(p.data_ptr(), inp.data_ptr(), out.data_ptr(), sr, sc, float(alpha), M, C, R,
+                                ws.data_ptr(), ws.numel(), _stream(dev))
+    _lib.check(rc, "q4_lora_grad_f32")
     return out
 
 

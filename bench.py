@@ -320,6 +320,9 @@ def main():
             r = bench_mlp_decode(M, max(args.steps // 2, 5), 2)
             extra[f"mlp_decode_M{M}"] = {"gbs": round(r["gbs_kernel"], 1), "us_per_gemv": round(r["avg_launch_us"], 3),
                                          "frac_hbm": round(r["gbs_kernel"] / HBM_PEAK_GBS, 4)}
+        # gate and up share x: concatenated along N they are one launch of twice the size
+        gu = bench_single_gemv(4096, 22016, 1, False, 10, 16)
+        extra["mlp_decode_M1_gate_up_fused_N22016"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in gu.items()}
         c0 = bench_single_gemv(4096, 4096, 1, False, 20, 40)
         extra["config0_K4096_N4096_M1_cold"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in c0.items()}
         c0h = bench_single_gemv(4096, 4096, 1, False, 20, 1)

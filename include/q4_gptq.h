@@ -78,16 +78,16 @@ int q4_gemv_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, co
  * Replaces vecquant4recons_v2 + torch.matmul(x, buffer) (matmul_utils_4bit.py:114-124),
  * the bias add (autograd_4bit.py:206-207) and, when xa/lora_b are given, the adapter term
  * result += lora_B(lora_A(x)) * scaling (models.py:58-66) where xa = x @ A^T.
- * The adapter matrix is addressed as Bm[r, n] = lora_b[r*ldb_r + n*ldb_n] (fp16), so both
- * lora_B.weight [N, R] (ldb_r = 1, ldb_n = R) and its transpose can be passed without a copy.
+ * The adapter matrix is addressed as Bm[r, n] = lora_b[r*ldb_r + n*ldb_n], fp16 or (lora_is_f32 != 0)
+ * fp32, so lora_B.weight [N, R] (ldb_r = 1, ldb_n = R) is passed in place: no cast, no transpose.
  * bias, xa, lora_b may be NULL; R is 0 or a multiple of 8, at most 64.
  * Both GEMM entry points need K % 128 == 0, N % 128 == 0, K*N < 2^33, and with g_idx == NULL also
  * groupsize % 64 == 0 and every |scale| < 64 (the sequential-group dequant forms s*q with a fused
  * multiply-add on 1024+q; pass g_idx to lift the restriction on the scales). */
 int q4_gemm_fwd_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                     const int32_t *g_idx, int groupsize, const void *bias,
-                    const void *xa, const void *lora_b, int ldb_r, int ldb_n, float lora_scale, int R,
-                    void *y, int M, int K, int N, int G, void *stream);
+                    const void *xa, const void *lora_b, int ldb_r, int ldb_n, int lora_is_f32, float lora_scale,
+                    int R, void *y, int M, int K, int N, int G, void *stream);
 
 /* Backward GEMM (grad of the input):
  *   dx fp16 [M, K] = dy fp16 [M, N] @ W^T  (+ lora_scale * dyb fp16 [M, R] @ Am [R, K])
@@ -97,8 +97,25 @@ int q4_gemm_fwd_f16(const void *x, const int32_t *qweight, const int32_t *qzeros
  * (lora_A.weight [R, K]: lda_r = K, lda_k = 1). */
 int q4_gemm_bwd_dx_f16(const void *dy, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                        const int32_t *g_idx, int groupsize,
-                       const void *dyb, const void *lora_a, int lda_r, int lda_k, float lora_scale, int R,
-                       void *dx, int M, int K, int N, int G, void *stream);
+                       const void *dyb, const void *lora_a, int lda_r, int lda_k, int lora_is_f32, float lora_scale,
+                       int R, void *dx, int M, int K, int N, int G, void *stream);
+
+/* Rank-R down projection of the adapter:  out fp16 [M, R] = in fp16 [M, C] @ Wm^T,
+ * Wm[j, c] = w[j*w_sr + c*w_sc] (fp16, or fp32 when w_is_f32 != 0).  xa = x @ A^T (w = lora_A.weight,
+ * w_sr = K, w_sc = 1) and dyb = dy @ B (w = lora_B.weight, w_sr = 1, w_sc = R): the two products that
+ * lora_A(x) and the backward of lora_B perform in the reference (models.py:66).  C % 32 == 0, 1 <= R <= 64. */
+int q4_lora_down_f16(const void *in, const void *w, int w_sr, int w_sc, int w_is_f32, void *out,
+                     int M, int C, int R, void *stream);
+
+/* Gradient of an adapter matrix:  out fp32 [j*o_sr + c*o_sc] = alpha * sum_m p[m, j] * in[m, c]
+ * with p fp16 [M, R] and in fp16 [M, C]:  dA = scaling * dyb^T @ x (out = [R, K], o_sr = K, o_sc = 1) and
+ * dB = scaling * dy^T @ xa (out = lora_B.weight.grad [N, R], o_sr = 1, o_sc = R) -- what torch autograd
+ * computes for the two adapter Linears of models.py:66.  R is 8 or 16, C % 8 == 0.
+ * `workspace`: q4_lora_grad_workspace_bytes(R, C) = 8*R*C bytes, 256-byte aligned, zero before first
+ * use and left zero by every call (64-bit fixed-point sums across workgroups: bit-reproducible). */
+size_t q4_lora_grad_workspace_bytes(int R, int C);
+int q4_lora_grad_f32(const void *p, const void *in, float *out, int o_sr, int o_sc, float alpha,
+                     int M, int C, int R, void *workspace, size_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

@@ -51,11 +51,20 @@ def test_error_codes_and_validation_need_no_gpu():
     assert L.q4_gemv_f16(fake, fake, fake, fake, None, 128, fake, 0, 17, 256, 128, 2, fake, 1 << 20, None) == -2
     assert L.q4_gemv_f16(fake, fake, fake, fake, None, 128, fake, 0, 1, 256, 128, 2, None, 0, None) == -3
     assert L.q4_gemv_f16(fake, fake, fake, fake, None, 128, fake, 0, 1, 256, 128, 2, fake, 8, None) == -3
-    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, None, None, 0, 0, 1.0, 0, fake, 64, 192, 128, 2, None) == -2
-    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, None, 1, 8, 1.0, 8, fake, 64, 256, 128, 2, None) == -1
-    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, fake, 1, 12, 1.0, 12, fake, 64, 256, 128, 2, None) == -2
-    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, fake, 0, 8, 1.0, 8, fake, 64, 256, 128, 2, None) == -2
-    assert L.q4_gemm_bwd_dx_f16(fake, fake, fake, fake, None, 32, None, None, 0, 0, 1.0, 0, fake, 64, 256, 128, 8, None) == -2
+    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, None, None, 0, 0, 0, 1.0, 0, fake, 64, 192, 128, 2, None) == -2
+    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, None, 1, 8, 0, 1.0, 8, fake, 64, 256, 128, 2, None) == -1
+    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, fake, 1, 12, 0, 1.0, 12, fake, 64, 256, 128, 2, None) == -2
+    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, fake, 0, 8, 1, 1.0, 8, fake, 64, 256, 128, 2, None) == -2
+    assert L.q4_gemm_bwd_dx_f16(fake, fake, fake, fake, None, 32, None, None, 0, 0, 0, 1.0, 0, fake, 64, 256, 128, 8, None) == -2
+    # adapter helpers
+    assert L.q4_lora_down_f16(fake, None, 4096, 1, 1, fake, 64, 4096, 8, None) == -1
+    assert L.q4_lora_down_f16(fake, fake, 4096, 1, 1, fake, 64, 4100, 8, None) == -2        # C % 32
+    assert L.q4_lora_down_f16(fake, fake, 4096, 1, 1, fake, 64, 4096, 65, None) == -2       # R > 64
+    assert L.q4_lora_down_f16(fake, ctypes.c_void_p(0x1002), 4096, 1, 1, fake, 64, 4096, 8, None) == -5
+    assert L.q4_lora_grad_workspace_bytes(8, 4096) == 8 * 8 * 4096
+    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 64, 4096, 12, fake, 1 << 20, None) == -2   # R not 8/16
+    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 64, 4096, 8, None, 0, None) == -3
+    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 64, 4096, 8, fake, 1024, None) == -3
     assert L.q4_gemv_workspace_bytes(16, 4096, 11008) == 16 * 11008 * 8
     assert L.q4_gemv_workspace_bytes(0, 4096, 11008) == 0
 

@@ -155,6 +155,30 @@ def test_fused_and_unfused_lora_agree(oracle):
         assert rel_err(a, b) <= TOL
 
 
+def test_fuse_quant_linears_matches_separate_layers(oracle):
+    """gate/up (or q/k/v) concatenated along N: one launch, same numbers."""
+    import torch
+    from alpaca_lora_4bit_amd.autograd_4bit import Autograd4bitQuantLinear, fuse_quant_linears
+    K = 512
+    mods, refs = [], []
+    x = oracle.make_activations(3, K, seed=9)
+    for i, N in enumerate((256, 384)):
+        layer = oracle.make_layer(K, N, 128, seed=40 + i)
+        mods.append(_fill(Autograd4bitQuantLinear(K, N, groupsize=128), layer))
+        refs.append(oracle.matmul_recons(x, layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"]))
+    fused = fuse_quant_linears(mods)
+    assert fused.out_features == 640 and fused.qweight.shape == (64, 640) and fused.qzeros.shape == (4, 80)
+    xt = torch.from_numpy(x).cuda()
+    with torch.no_grad():
+        y = fused(xt)
+        parts = torch.cat([m(xt) for m in mods], dim=-1)
+    assert torch.equal(y, parts)
+    assert rel_err(y.cpu().numpy(), np.concatenate(refs, axis=1)) <= TOL
+    bad = Autograd4bitQuantLinear(K, 128, groupsize=64)
+    with pytest.raises(ValueError):
+        fuse_quant_linears([mods[0], bad])
+
+
 def test_backend_switch_and_errors():
     from alpaca_lora_4bit_amd import autograd_4bit
     autograd_4bit.switch_backend_to("cuda")
