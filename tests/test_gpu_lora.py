@@ -1,0 +1,99 @@
+"""Parity of the rank-R adapter kernels (q4_lora_down_f16, q4_lora_grad_f32) with the numpy oracle's
+adapter products (oracle/q4_oracle.py: lora_forward / lora_backward follow models.py:58-66 of the
+reference and torch autograd over its two adapter Linears).
+
+Tolerance: 1e-2 * max|ref| as for every matmul of this path; the fp32 gradients are additionally checked
+to 1e-3 relative since they accumulate in fp32 / exact fixed point from the same fp16 inputs."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _rand16(rng, *shape, scale=1.0):
+    return (rng.standard_normal(shape) * scale).astype(np.float16)
+
+
+@pytest.mark.parametrize("M,C,R,wdtype", [
+    (2048, 4096, 8, torch.float32), (2048, 4096, 8, torch.float16), (37, 256, 16, torch.float32),
+    (1, 64, 8, torch.float16), (300, 11008, 64, torch.float32), (129, 1024, 24, torch.float16),
+    (16, 4096, 3, torch.float32),
+])
+def test_lora_down_both_layouts(M, C, R, wdtype):
+    from alpaca_lora_4bit_amd import quant_hip
+    rng = np.random.default_rng(M * 7 + C + R)
+    x = _rand16(rng, M, C)
+    w = _rand16(rng, R, C, scale=0.05)
+    ref = x.astype(np.float32) @ w.astype(np.float32).T
+    xd = torch.from_numpy(x).cuda()
+    wd = torch.from_numpy(w).cuda().to(wdtype)
+    tol = 1e-2 * np.abs(ref).max() + 1e-6
+    got = quant_hip.lora_down(xd, wd).float().cpu().numpy()                     # lora_A layout [R, C]
+    assert np.abs(got - ref).max() <= tol
+    wt = wd.t().contiguous()                                                   # lora_B layout [C, R], viewed as [R, C]
+    got_t = quant_hip.lora_down(xd, wt.t()).float().cpu().numpy()
+    assert np.abs(got_t - ref).max() <= tol
+    assert np.array_equal(got, got_t)                                           # same arithmetic either way
+
+
+@pytest.mark.parametrize("M,C,R", [(2048, 4096, 8), (2048, 11008, 8), (2048, 4096, 16), (77, 64, 8),
+                                   (1, 8, 16), (1000, 520, 8), (5000, 128, 16)])
+def test_lora_grad_matches_fp32_product(M, C, R):
+    from alpaca_lora_4bit_amd import quant_hip
+    rng = np.random.default_rng(M + C * 3 + R)
+    p = _rand16(rng, M, R, scale=0.1)
+    x = _rand16(rng, M, C)
+    alpha = 2.0
+    ref = alpha * (p.astype(np.float64).T @ x.astype(np.float64))
+    pd, xd = torch.from_numpy(p).cuda(), torch.from_numpy(x).cuda()
+    got = quant_hip.lora_grad(pd, xd, alpha)
+    got_t = quant_hip.lora_grad(pd, xd, alpha, transposed=True)
+    assert got.shape == (R, C) and got_t.shape == (C, R) and got.dtype == torch.float32
+    g = got.cpu().numpy()
+    assert np.abs(g - ref).max() <= 1e-3 * np.abs(ref).max() + 1e-6
+    assert torch.equal(got, got_t.t())                                          # strided store, same sums
+    # reproducible: the cross-workgroup sum is order-independent
+    again = quant_hip.lora_grad(pd, xd, alpha)
+    assert torch.equal(got, again)
+
+
+def test_lora_grad_leaves_workspace_zero():
+    from alpaca_lora_4bit_amd import quant_hip
+    rng = np.random.default_rng(3)
+    pd = torch.from_numpy(_rand16(rng, 2048, 8)).cuda()
+    xd = torch.from_numpy(_rand16(rng, 2048, 4096)).cuda()
+    quant_hip.lora_grad(pd, xd, 1.0)
+    torch.cuda.synchronize()
+    for ws in quant_hip._workspaces.values():
+        assert int(ws.count_nonzero()) == 0
+
+
+def test_fused_lora_function_against_oracle_fp32_adapters(oracle):
+    """Whole fused layer with fp32 adapter parameters (the usual PEFT state): y, dx, dA, dB against
+    the oracle's float64 lora_forward / lora_backward on the fp16-rounded adapter values."""
+    from alpaca_lora_4bit_amd.autograd_4bit import AutogradMatmul4bitLora
+    K, N, M, r, gs = 512, 384, 200, 8, 128
+    layer = oracle.make_layer(K, N, gs, seed=11)
+    x = oracle.make_activations(M, K, seed=5)
+    dy = oracle.make_activations(M, N, seed=6)
+    A, B = oracle.make_lora(K, N, r, seed=7)
+    B = (B * 10).astype(np.float32)                      # a trained-looking B so that every term matters
+    scaling = 2.0
+    W = oracle.dequant_v2(layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
+    A16, B16 = A.astype(np.float16), B.astype(np.float16)
+    y_ref = oracle.lora_forward(x, W, A16, B16, scaling)
+    dx_ref, dA_ref, dB_ref = oracle.lora_backward(x, dy, W, A16, B16, scaling)
+
+    t = lambda a: torch.from_numpy(a).cuda()
+    xd = t(x).requires_grad_(True)
+    Ad = t(A).requires_grad_(True)
+    Bd = t(B).requires_grad_(True)
+    y = AutogradMatmul4bitLora.apply(xd, t(layer["qweight"]), t(layer["scales"]), t(layer["qzeros"]), None, None,
+                                     Ad, Bd, scaling, gs)
+    y.backward(t(dy))
+    for got, ref in ((y, y_ref), (xd.grad, dx_ref), (Ad.grad, dA_ref), (Bd.grad, dB_ref)):
+        g = got.detach().float().cpu().numpy()
+        assert g.shape == ref.shape
+        assert np.abs(g - ref).max() <= 1e-2 * np.abs(ref).max()
+    assert Ad.grad.dtype == torch.float32 and Bd.grad.dtype == torch.float32
