@@ -13,6 +13,7 @@ int q4_launch_gemm(int, const void*, const int32_t*, const int32_t*, const void*
                    const void*, const void*, int, int, int, float, int, void*, int, int, int, int, hipStream_t);
 int q4_launch_lora_down(const void*, const void*, int, int, int, void*, int, int, int, hipStream_t);
 int q4_launch_lora_grad(const void*, const void*, float*, int, int, float, int, int, int, void*, hipStream_t);
+size_t q4_lora_grad_workspace(int, int, int);
 }
 
 namespace {
@@ -120,22 +121,29 @@ extern "C" int q4_lora_down_f16(const void* in, const void* w, int w_sr, int w_s
                                 int M, int C, int R, void* stream) {
     if (!in || !w || !out) return Q4_ERR_NULL_POINTER;
     if (M < 1 || C < 32 || (C % 32) != 0 || R < 1 || R > 64 || w_sr < 1 || w_sc < 1) return Q4_ERR_BAD_SHAPE;
+    /* 32-bit buffer offsets: the 16-row block of `in` and the span of the adapter matrix */
+    if ((long long)C * 32 >= 0x70000000ll) return Q4_ERR_BAD_SHAPE;
+    if (((long long)(R - 1) * w_sr + (long long)(C - 1) * w_sc + 1) * (w_is_f32 ? 4 : 2) >= 0x70000000ll) return Q4_ERR_BAD_SHAPE;
     if (misaligned(in) || (reinterpret_cast<uintptr_t>(out) & 1u) || (reinterpret_cast<uintptr_t>(w) & (w_is_f32 ? 3u : 1u)))
         return Q4_ERR_MISALIGNED;
     return q4_launch_lora_down(in, w, w_sr, w_sc, w_is_f32, out, M, C, R, (hipStream_t)stream);
 }
 
-extern "C" size_t q4_lora_grad_workspace_bytes(int R, int C) {
-    if (R < 1 || C < 1) return 0;
-    return (size_t)R * (size_t)C * sizeof(unsigned long long);
+extern "C" size_t q4_lora_grad_workspace_bytes(int M, int C, int R) {
+    if (M < 1 || C < 8 || (R != 8 && R != 16)) return 0;
+    return q4_lora_grad_workspace(M, C, R);
 }
 
 extern "C" int q4_lora_grad_f32(const void* p, const void* in, float* out, int o_sr, int o_sc, float alpha,
                                 int M, int C, int R, void* workspace, size_t workspace_bytes, void* stream) {
     if (!p || !in || !out) return Q4_ERR_NULL_POINTER;
     if (M < 1 || C < 8 || (C % 8) != 0 || (R != 8 && R != 16) || o_sr < 1 || o_sc < 1) return Q4_ERR_BAD_SHAPE;
+    if ((long long)M * C * 2 >= 0x70000000ll || C > (1 << 20)) return Q4_ERR_BAD_SHAPE;     /* 32-bit buffer offsets */
     if (misaligned(p) || misaligned(in) || (reinterpret_cast<uintptr_t>(out) & 3u)) return Q4_ERR_MISALIGNED;
-    if (!workspace || workspace_bytes < q4_lora_grad_workspace_bytes(R, C)) return Q4_ERR_WORKSPACE;
-    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
+    const size_t need = q4_lora_grad_workspace(M, C, R);
+    if (need > 0) {
+        if (!workspace || workspace_bytes < need) return Q4_ERR_WORKSPACE;
+        if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
+    }
     return q4_launch_lora_grad(p, in, out, o_sr, o_sc, alpha, M, C, R, workspace, (hipStream_t)stream);
 }

@@ -61,4 +61,25 @@ __device__ __forceinline__ void unpack8_natural(uint32_t w, half2_t out[4]) {
     out[3] = codes_to_half2(__builtin_amdgcn_perm(hi, lo, 0x0c070c03u));
 }
 
+// Buffer-resource loads: a 32-bit byte offset per lane plus a uniform byte offset; an access
+// past `bytes` returns zero instead of faulting, so tiles need no per-lane bounds branches.
+constexpr int kRsrcFlags = 0x00020000;
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, kRsrcFlags);
+}
+__device__ __forceinline__ uint4_t buf_load128(rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
+__device__ __forceinline__ uint2_t buf_load64(rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
+}
+__device__ __forceinline__ uint32_t buf_load32(rsrc_t r, int voff, int soff) {
+    return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
+}
+__device__ __forceinline__ uint32_t buf_load16(rsrc_t r, int voff, int soff) {
+    return (uint32_t)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0);
+}
+
 }  // namespace q4

@@ -37,9 +37,6 @@ namespace q4 {
 
 constexpr int BN = 128, BK = 64;
 constexpr int LDS_STRIDE = BK + 8;   // halves
-constexpr int kRsrcFlags = 0x00020000;
-
-typedef __amdgpu_buffer_rsrc_t rsrc_t;
 
 struct GemmArgs {
     const half_t* a;          // fwd: x [M,K]      bwd: dy [M,N]
@@ -61,22 +58,6 @@ struct GemmArgs {
 __device__ __forceinline__ float adapter_at(const GemmArgs& a, size_t idx) {
     return a.lb_is_f32 ? reinterpret_cast<const float*>(a.lb)[idx] : (float)reinterpret_cast<const half_t*>(a.lb)[idx];
 }
-__device__ __forceinline__ rsrc_t make_rsrc(const void* p, unsigned bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)bytes, kRsrcFlags);
-}
-__device__ __forceinline__ uint4_t buf_load128(rsrc_t r, int voff, int soff) {
-    return __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
-}
-__device__ __forceinline__ uint2_t buf_load64(rsrc_t r, int voff, int soff) {
-    return __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
-}
-__device__ __forceinline__ uint32_t buf_load32(rsrc_t r, int voff, int soff) {
-    return __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0);
-}
-__device__ __forceinline__ uint32_t buf_load16(rsrc_t r, int voff, int soff) {
-    return (uint32_t)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0);
-}
-
 // rn16(rn16(s*q) - zero) for a pair of codes given as (0x6400 | q): one fused multiply-add
 // computes s*(1024+q) - 1024*s = s*q with a single rounding (1024*s is exact), i.e. exactly
 // rn16(s*q); the subtraction of the zero term is the third rounding.  Needs |s| < 64 so that

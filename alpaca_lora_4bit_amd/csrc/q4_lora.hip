@@ -13,77 +13,187 @@
 
 namespace q4 {
 
-constexpr int kFracBits = 24;
-constexpr long long kBias = 1ll << 47;
-constexpr float kClamp = 4194304.0f;
+constexpr int kFarOffset = 0x70000000;      // beyond any buffer accepted here: such loads return zero, no traffic
 
-__device__ __forceinline__ half8_t load_w8(const void* w, int is_f32, size_t idx0, int stride_c) {
-    // eight consecutive-c elements W[j, c0 .. c0+7] as fp16
+__device__ __forceinline__ half8_t to_half8(float4_t a, float4_t b) {
     half8_t r;
-    if (is_f32) {
-        const float* p = reinterpret_cast<const float*>(w) + idx0;
-        if (stride_c == 1 && (idx0 & 3) == 0) {
-            const float4_t a = *reinterpret_cast<const float4_t*>(p), b = *reinterpret_cast<const float4_t*>(p + 4);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) { r[e] = (half_t)a[e]; r[4 + e] = (half_t)b[e]; }
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) r[e] = (half_t)p[(size_t)e * stride_c];
-        }
-    } else {
-        const half_t* p = reinterpret_cast<const half_t*>(w) + idx0;
-        if (stride_c == 1 && (idx0 & 7) == 0) {
-            r = *reinterpret_cast<const half8_t*>(p);
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) r[e] = p[(size_t)e * stride_c];
-        }
-    }
+    for (int e = 0; e < 4; ++e) { r[e] = (half_t)a[e]; r[4 + e] = (half_t)b[e]; }
     return r;
 }
 
 // ---- down projection -------------------------------------------------------------------
-// Workgroup = 8 wavefronts on 16 rows; wavefront w multiplies the C/8-wide slice w of those rows
+// Workgroup = 16 wavefronts on 16 rows; wavefront w multiplies the C/16-wide slice w of those rows
 // with v_mfma_f32_16x16x32_f16 (A operand = 16 rows x 32 columns of `in`, B operand = the same 32
-// columns of up to 16 rows of W), partial 16 x 16 results are added through LDS.
-// R <= 64 is handled as ceil(R/16) column blocks.
-template <int RB>   // number of 16-wide blocks of R
-__global__ __launch_bounds__(512) void lora_down_kernel(const half_t* __restrict__ in, const void* __restrict__ w,
-                                                        int w_sr, int w_sc, int w_is_f32, half_t* __restrict__ out,
-                                                        int M, int C, int R) {
-    __shared__ float red[8][RB][256];
+// columns of up to 16 rows of W); the partial 16 x 16 results are added through LDS.  R <= 64 is
+// handled as RB = ceil(R/16) column blocks.
+// All loads are buffer loads whose out-of-range lanes (rows past M, adapter rows past R, steps past
+// the wavefront's slice) return zero: no branch sits between the loads of a batch of UN steps, so they
+// are all in flight together.  Three ways to fetch W[j][c] -> the B operand (8 consecutive c per lane):
+//   kRowsT c contiguous in memory (lora_A.weight [R, C]), R <= 16: each adapter row's 256-column piece is
+//          loaded as one fully coalesced instruction (4 values per lane), converted, and passed to the
+//          operand layout through a wavefront-private LDS tile
+//   kCols  j contiguous in memory (lora_B.weight [C, R] seen as W = B^T), R <= 16, R % 4 == 0: groups of 4
+//          adapter rows are loaded coalesced and transposed through the same LDS tile
+//   kRows  c contiguous, any R <= 64: one or two 16-byte loads per lane and step straight into the operand
+//   kAny   arbitrary strides: eight scalar loads per lane and step
+enum WLayout { kRows = 0, kCols = 1, kAny = 2, kRowsT = 3 };
+constexpr int kDownWaves = 16;
+
+template <int RB, int WL, bool F32, int RQ>   // RQ: ceil(R/4) for kCols / kRowsT, else unused
+__global__ __launch_bounds__(64 * kDownWaves) void lora_down_kernel(const half_t* __restrict__ in,
+                                                                    const void* __restrict__ w, int w_sr, int w_sc,
+                                                                    half_t* __restrict__ out, int M, int C, int R) {
+    constexpr int NW = kDownWaves;
+    constexpr int UN = WL == kAny ? (RB == 1 ? 4 : RB == 2 ? 2 : 1) : (RB == 1 ? 8 : 4);   // steps whose loads are issued together
+    constexpr int ES = F32 ? 4 : 2;
+    constexpr int TRW = UN * 32 + 8;                            // padded row of the transposition tile (halves)
+    __shared__ float red[NW][RB][256];
+    constexpr bool kStaged = WL == kCols || WL == kRowsT;
+    __shared__ __attribute__((aligned(16))) half_t tr[kStaged ? NW : 1][16][kStaged ? TRW : 8];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kk = lane >> 4, c = lane & 15;
     const int m0 = blockIdx.x * 16;
-    const int row = min(m0 + c, M - 1);
     const int steps = C / 32;                                   // C is a multiple of 32
-    const int s_begin = (steps * wave) / 8, s_end = (steps * (wave + 1)) / 8;
+    const int s_begin = (steps * wave) / NW, s_end = (steps * (wave + 1)) / NW;
+    const rsrc_t rs_in = make_rsrc(in + (size_t)m0 * C, (unsigned)min(16, M - m0) * (unsigned)C * 2u);
+    const rsrc_t rs_w = make_rsrc(w, ((unsigned)(R - 1) * (unsigned)w_sr + (unsigned)(C - 1) * (unsigned)w_sc + 1u) * ES);
+    const int voff_in = (c * C + 8 * kk) * 2;
     float4_t acc[RB];
 #pragma unroll
     for (int b = 0; b < RB; ++b) acc[b] = float4_t{0.f, 0.f, 0.f, 0.f};
-    const half_t* ip = in + (size_t)row * C + 8 * kk;
-    constexpr int UN = RB == 1 ? 8 : 4;                        // steps whose loads are issued together
+
     for (int s0 = s_begin; s0 < s_end; s0 += UN) {
-        half8_t av[UN], bv[UN][RB];
+        uint4_t av[UN];
+        half8_t bv[UN][RB];
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
-            const int s = min(s0 + u, s_end - 1);               // tail steps repeat the last one and are skipped below
-            av[u] = *reinterpret_cast<const half8_t*>(ip + 32 * s);
-#pragma unroll
-            for (int b = 0; b < RB; ++b) {
-                const int j = 16 * b + c;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) bv[u][b][e] = (half_t)0.f;
-                if (j < R) bv[u][b] = load_w8(w, w_is_f32, (size_t)j * w_sr + (size_t)(32 * s + 8 * kk) * w_sc, w_sc);
-            }
+            const int s = s0 + u;
+            av[u] = buf_load128(rs_in, voff_in, s < s_end ? s * 64 : kFarOffset);
         }
+        if constexpr (WL == kRows) {
+            uint4_t raw[UN][RB][F32 ? 2 : 1];
 #pragma unroll
-        for (int u = 0; u < UN; ++u)
-            if (s0 + u < s_end)
+            for (int u = 0; u < UN; ++u) {
+                const int s = s0 + u;
+                const int soff = s < s_end ? s * 32 * ES : kFarOffset;
+#pragma unroll
+                for (int b = 0; b < RB; ++b) {
+                    const int j = 16 * b + c;
+                    const int voff = j < R ? (j * w_sr + 8 * kk) * ES : kFarOffset;
+                    raw[u][b][0] = buf_load128(rs_w, voff, soff);
+                    if constexpr (F32) raw[u][b][1] = buf_load128(rs_w, voff + 16, soff);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UN; ++u)
+#pragma unroll
+                for (int b = 0; b < RB; ++b) {
+                    if constexpr (F32) bv[u][b] = to_half8(__builtin_bit_cast(float4_t, raw[u][b][0]), __builtin_bit_cast(float4_t, raw[u][b][1]));
+                    else bv[u][b] = __builtin_bit_cast(half8_t, raw[u][b][0]);
+                }
+        } else if constexpr (kStaged) {
+            // fill the tile tr[j][column within the batch] with fp16 values of W
+            if constexpr (WL == kCols) {
+                // UN*32 columns x RQ groups of 4 adapter rows, 64 items per load instruction
+                constexpr int NT = UN * 32 * RQ / 64;
+                uint4_t raw[NT];
+                const int soff = s0 * 32 * w_sc * ES;
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const int i = lane + 64 * t, cl = i / RQ, q = i - cl * RQ;
+                    const int voff = (s0 * 32 + cl) < s_end * 32 ? (cl * w_sc + 4 * q) * ES : kFarOffset;
+                    if constexpr (F32) raw[t] = buf_load128(rs_w, voff, soff);
+                    else { const uint2_t v = buf_load64(rs_w, voff, soff); raw[t] = uint4_t{v.x, v.y, 0u, 0u}; }
+                }
+#pragma unroll
+                for (int t = 0; t < NT; ++t) {
+                    const int i = lane + 64 * t, cl = i / RQ, q = i - cl * RQ;
+                    half_t h[4];
+                    if constexpr (F32) {
+                        const float4_t f = __builtin_bit_cast(float4_t, raw[t]);
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) h[e] = (half_t)f[e];
+                    } else {
+                        const half2_t lo = as_half2(raw[t].x), hi = as_half2(raw[t].y);
+                        h[0] = lo[0]; h[1] = lo[1]; h[2] = hi[0]; h[3] = hi[1];
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) tr[wave][4 * q + e][cl] = h[e];
+                }
+            } else {
+                // 4*RQ adapter rows; per row the batch's UN*32 columns, 4 per lane
+                constexpr int NL = UN * 32 / 256;                 // load instructions per row (1 for UN = 8)
+                static_assert(NL >= 1, "a batch must cover at least 256 columns");
+                uint4_t raw[4 * RQ][NL];
+                const int soff = s0 * 32 * ES;
+#pragma unroll
+                for (int j = 0; j < 4 * RQ; ++j)
+#pragma unroll
+                    for (int t = 0; t < NL; ++t) {
+                        const int cl = 4 * (lane + 64 * t);
+                        const int voff = (j < R && (s0 * 32 + cl) < s_end * 32) ? (j * w_sr + cl) * ES : kFarOffset;
+                        if constexpr (F32) raw[j][t] = buf_load128(rs_w, voff, soff);
+                        else { const uint2_t v = buf_load64(rs_w, voff, soff); raw[j][t] = uint4_t{v.x, v.y, 0u, 0u}; }
+                    }
+#pragma unroll
+                for (int j = 0; j < 4 * RQ; ++j)
+#pragma unroll
+                    for (int t = 0; t < NL; ++t) {
+                        const int cl = 4 * (lane + 64 * t);
+                        uint2_t packed;
+                        if constexpr (F32) {
+                            const float4_t f = __builtin_bit_cast(float4_t, raw[j][t]);
+                            const half2_t lo = {(half_t)f[0], (half_t)f[1]}, hi = {(half_t)f[2], (half_t)f[3]};
+                            packed = uint2_t{as_u32(lo), as_u32(hi)};
+                        } else {
+                            packed = uint2_t{raw[j][t].x, raw[j][t].y};
+                        }
+                        *reinterpret_cast<uint2_t*>(&tr[wave][j][cl]) = packed;
+                    }
+            }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                const half8_t v = *reinterpret_cast<const half8_t*>(&tr[wave][c][32 * u + 8 * kk]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) bv[u][0][e] = c < 4 * RQ ? v[e] : (half_t)0.f;   // rows past R were never written
+            }
+            __builtin_amdgcn_wave_barrier();
+        } else {
+            uint32_t raw[UN][RB][8];
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                const int s = s0 + u;
+                const int soff = s < s_end ? s * 32 * w_sc * ES : kFarOffset;
+#pragma unroll
+                for (int b = 0; b < RB; ++b) {
+                    const int j = 16 * b + c;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int voff = j < R ? (j * w_sr + (8 * kk + e) * w_sc) * ES : kFarOffset;
+                        raw[u][b][e] = F32 ? buf_load32(rs_w, voff, soff) : buf_load16(rs_w, voff, soff);
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UN; ++u)
 #pragma unroll
                 for (int b = 0; b < RB; ++b)
-                    acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[u], bv[u][b], acc[b], 0, 0, 0);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e)
+                        bv[u][b][e] = F32 ? (half_t)__builtin_bit_cast(float, raw[u][b][e])
+                                          : __builtin_bit_cast(half_t, (uint16_t)raw[u][b][e]);
+        }
+        // steps past the slice were loaded as zeros: they add nothing
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+#pragma unroll
+            for (int b = 0; b < RB; ++b)
+                acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, av[u]), bv[u][b], acc[b], 0, 0, 0);
     }
     // acc[b][r]: row 4*kk + r, column 16*b + c
 #pragma unroll
@@ -91,156 +201,265 @@ __global__ __launch_bounds__(512) void lora_down_kernel(const half_t* __restrict
 #pragma unroll
         for (int r = 0; r < 4; ++r) red[wave][b][(4 * kk + r) * 16 + c] = acc[b][r];
     __syncthreads();
-    for (int e = threadIdx.x; e < RB * 256; e += 512) {
+    for (int e = threadIdx.x; e < RB * 256; e += 64 * NW) {
         const int b = e >> 8, i = e & 255;
         float v = 0.f;
 #pragma unroll
-        for (int wv = 0; wv < 8; ++wv) v += red[wv][b][i];
+        for (int wv = 0; wv < NW; ++wv) v += red[wv][b][i];
         const int m = m0 + (i >> 4), j = 16 * b + (i & 15);
         if (m < M && j < R) out[(size_t)m * R + j] = (half_t)v;
     }
 }
 
 // ---- gradient of an adapter matrix -------------------------------------------------------
-// out[j, c] = alpha * sum_m P[m, j] * in[m, c].  A thread owns CPT = 64/R8 adjacent columns
-// (R8 = R rounded up to 8... here R in {8, 16}: 8 or 4 columns) and R x CPT fp32 accumulators; the
-// 8 wavefronts of a workgroup share a block of 64*CPT columns and split its rows; gridDim.y
-// workgroups share a column block.  Rows of P reach the lanes as LDS broadcasts.  The reduction
-// over wavefronts goes through LDS, the one over workgroups through one 64-bit fixed-point
-// atomic per output element with an arrival count in the top byte (order-independent, hence
-// bit-reproducible; the last arrival converts, scales and stores, and zeroes the workspace).
+// out[j, c] = alpha * sum_m P[m, j] * in[m, c].  A thread owns CPT = 64/R adjacent columns (R is 8
+// or 16: 8 or 4 columns) and R x CPT fp32 accumulators; the 4 wavefronts of a workgroup share a
+// block of 64*CPT columns and split its rows 16 at a time; gridDim.y workgroups share a column
+// block.  Two rows are multiplied per instruction with v_dot2_f32_f16: rows (2i, 2i+1) of `in` are
+// interleaved in registers with two byte permutes per dword, the matching pairs of P come from
+// LDS as broadcasts.  The sum over wavefronts goes through LDS; the sum over workgroups goes
+// through fp32 partial tiles in the workspace that a second small kernel adds in a fixed order
+// (bit-reproducible, no atomics, nothing to pre-clear).
+// Partial tile layout: part[split][column block][a = j*CPT + e][lane], i.e. exactly the order the
+// workgroup produces, so both kernels read and write it fully coalesced; only the final, small
+// output goes through the caller's strides.
+constexpr int kGradWaves = 4;
+
+template <int ND, int NPP>
+struct RowRegs { uint32_t d[16][ND]; uint32_t plo[NPP], phi[NPP]; };
+
 template <int R>
-__global__ __launch_bounds__(512) void lora_grad_kernel(const half_t* __restrict__ P, const half_t* __restrict__ in,
-                                                        float* __restrict__ out, int o_sr, int o_sc, float alpha,
-                                                        int M, int C, int rows_per_wg,
-                                                        unsigned long long* __restrict__ acc64) {
+__global__ __launch_bounds__(64 * kGradWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void lora_grad_kernel(const half_t* __restrict__ P,
+                                                                    const half_t* __restrict__ in,
+                                                                    float* __restrict__ out, int o_sr, int o_sc,
+                                                                    float alpha, int M, int C, int rows_per_wg,
+                                                                    float* __restrict__ part) {
     constexpr int CPT = 64 / R;                  // columns per thread: 8 (R = 8) or 4 (R = 16)
+    constexpr int ND = CPT / 2;                  // dwords per thread and row
+    constexpr int NPP = 8 * R / 64;              // pairs of P staged per lane and 16-row block
     constexpr int NACC = R * CPT;                // 64
-    __shared__ float red[8][NACC][64];           // 128 KB
-    __shared__ __attribute__((aligned(16))) half_t ptile[8][16][R];
+    __shared__ float red[kGradWaves][NACC][64];  // 64 KB
+    __shared__ __attribute__((aligned(16))) uint32_t ppair[kGradWaves][8 * R];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int c0 = (blockIdx.x * 64 + lane) * CPT;
-    const bool col_ok = c0 < C;                  // C is a multiple of 8, so a thread's columns are all in or all out
-    const int m_begin = blockIdx.y * rows_per_wg + wave * (rows_per_wg / 8);
-    const int m_end = min(m_begin + rows_per_wg / 8, M);
+    // lanes past the last column get an offset beyond the buffer: their loads return zero
+    const int voff = c0 < C ? c0 * 2 : kFarOffset;
+    const int row_bytes = C * 2;
+    const int rows_per_wave = rows_per_wg / kGradWaves;           // a multiple of 16
+    const int m_begin = blockIdx.y * rows_per_wg + wave * rows_per_wave;
+    const int m_end = min(m_begin + rows_per_wave, M);
+    // both buffers end at this wavefront's last row: rows past it read as zero
+    const rsrc_t rs_in = make_rsrc(in, (unsigned)max(m_end, 0) * (unsigned)row_bytes);
+    const rsrc_t rs_p = make_rsrc(P, (unsigned)max(m_end, 0) * (unsigned)(R * 2));
     float acc[R][CPT];
 #pragma unroll
     for (int j = 0; j < R; ++j)
 #pragma unroll
         for (int e = 0; e < CPT; ++e) acc[j][e] = 0.f;
 
-    for (int mb = m_begin; mb < m_end; mb += 16) {
-        // stage 16 rows of P for this wavefront (wavefront-private region, LDS ops of a wave are ordered)
-        const int nrow = min(16, m_end - mb);
-        for (int i = lane; i < 16 * R; i += 64) {
-            const int rr = i / R, j = i - rr * R;
-            ptile[wave][rr][j] = rr < nrow ? P[(size_t)(mb + rr) * R + j] : (half_t)0.f;
+    // Loads of one 16-row block: first the pairs (P[2i][j], P[2i+1][j]) this lane will stage in LDS,
+    // then the 16 rows of `in`.  No branches: a block past the end is fetched from kFarOffset.
+    auto load_rows = [&](RowRegs<ND, NPP>& x, int mb) {
+        const bool live = mb < m_end;
+        const int soff_p = live ? mb * R * 2 : kFarOffset;
+        const int soff_x = live ? mb * row_bytes : kFarOffset;
+#pragma unroll
+        for (int t = 0; t < NPP; ++t) {
+            const int i = lane + 64 * t, pi = i / R, j = i - pi * R;
+            x.plo[t] = buf_load16(rs_p, (2 * pi * R + j) * 2, soff_p);
+            x.phi[t] = buf_load16(rs_p, ((2 * pi + 1) * R + j) * 2, soff_p);
         }
+#pragma unroll
+        for (int rr = 0; rr < 16; ++rr) {
+            const int soff = soff_x + rr * row_bytes;
+            if constexpr (ND == 4) {
+                const uint4_t v = buf_load128(rs_in, voff, soff);
+                x.d[rr][0] = v.x; x.d[rr][1] = v.y; x.d[rr][2] = v.z; x.d[rr][3] = v.w;
+            } else {
+                const uint2_t v = buf_load64(rs_in, voff, soff);
+                x.d[rr][0] = v.x; x.d[rr][1] = v.y;
+            }
+        }
+    };
+    auto consume = [&](const RowRegs<ND, NPP>& x) {
+        // pairs of P -> LDS (wavefront-private region; LDS operations of one wavefront are ordered)
+#pragma unroll
+        for (int t = 0; t < NPP; ++t) ppair[wave][lane + 64 * t] = x.plo[t] | (x.phi[t] << 16);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        // all 16 row loads of `in` first, then the arithmetic
-        half_t xin[16][CPT];
 #pragma unroll
-        for (int rr = 0; rr < 16; ++rr) {
-            const int m = min(mb + rr, M - 1);
-            if (col_ok) {
-                if constexpr (CPT == 8) {
-                    const half8_t v = *reinterpret_cast<const half8_t*>(in + (size_t)m * C + c0);
+        for (int pi = 0; pi < 8; ++pi) {
+            if constexpr (R > 8) __builtin_amdgcn_sched_barrier(0);   // bounds the live LDS reads (register pressure)
+            uint32_t p2[R];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) xin[rr][e] = v[e];
-                } else {
-                    const half4_t v = *reinterpret_cast<const half4_t*>(in + (size_t)m * C + c0);
+            for (int j = 0; j < R; j += 4) {
+                const uint4_t pv = *reinterpret_cast<const uint4_t*>(&ppair[wave][pi * R + j]);
+                p2[j] = pv.x; p2[j + 1] = pv.y; p2[j + 2] = pv.z; p2[j + 3] = pv.w;
+            }
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) xin[rr][e] = v[e];
+            for (int d = 0; d < ND; ++d) {
+                const uint32_t r0 = x.d[2 * pi][d], r1 = x.d[2 * pi + 1][d];
+                const half2_t xlo = as_half2(__builtin_amdgcn_perm(r1, r0, 0x05040100u));   // column 2d of both rows
+                const half2_t xhi = as_half2(__builtin_amdgcn_perm(r1, r0, 0x07060302u));   // column 2d+1
+#pragma unroll
+                for (int j = 0; j < R; ++j) {
+                    acc[j][2 * d] = __builtin_amdgcn_fdot2(as_half2(p2[j]), xlo, acc[j][2 * d], false);
+                    acc[j][2 * d + 1] = __builtin_amdgcn_fdot2(as_half2(p2[j]), xhi, acc[j][2 * d + 1], false);
                 }
-            } else {
-#pragma unroll
-                for (int e = 0; e < CPT; ++e) xin[rr][e] = (half_t)0.f;
             }
-        }
-#pragma unroll
-        for (int rr = 0; rr < 16; ++rr) {
-            half_t p[R];
-#pragma unroll
-            for (int j = 0; j < R; j += 8) {
-                const half8_t pv = *reinterpret_cast<const half8_t*>(&ptile[wave][rr][j]);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) p[j + e] = pv[e];
-            }
-#pragma unroll
-            for (int j = 0; j < R; ++j)
-#pragma unroll
-                for (int e = 0; e < CPT; ++e) acc[j][e] += (float)p[j] * (float)xin[rr][e];
         }
         __builtin_amdgcn_wave_barrier();
+    };
+
+    // rows in blocks of 16, the next block's loads in flight while the current one is consumed
+    RowRegs<ND, NPP> xa, xb;
+    load_rows(xa, m_begin);
+    for (int mb = m_begin; mb < m_end; mb += 32) {
+        load_rows(xb, mb + 16);
+        consume(xa);
+        load_rows(xa, mb + 32);
+        if (mb + 16 < m_end) consume(xb);
     }
 #pragma unroll
     for (int j = 0; j < R; ++j)
 #pragma unroll
         for (int e = 0; e < CPT; ++e) red[wave][j * CPT + e][lane] = acc[j][e];
     __syncthreads();
-    const int S = gridDim.y;
-    for (int o = threadIdx.x; o < NACC * 64; o += 512) {
+    const bool direct = gridDim.y == 1;
+    float* tile = part + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * (NACC * 64);
+    for (int o = threadIdx.x; o < NACC * 64; o += 64 * kGradWaves) {
         const int a = o >> 6, ln = o & 63;
         float v = 0.f;
 #pragma unroll
-        for (int wv = 0; wv < 8; ++wv) v += red[wv][a][ln];
-        const int j = a / CPT, cc = (blockIdx.x * 64 + ln) * CPT + (a - j * CPT);
-        if (cc >= C) continue;
-        float* op = out + (size_t)j * o_sr + (size_t)cc * o_sc;
-        if (S == 1) {
-            *op = alpha * v;
+        for (int wv = 0; wv < kGradWaves; ++wv) v += red[wv][a][ln];
+        if (direct) {
+            const int j = a / CPT, cc = (blockIdx.x * 64 + ln) * CPT + (a - j * CPT);
+            if (cc < C) out[(size_t)j * o_sr + (size_t)cc * o_sc] = alpha * v;
         } else {
-            v = fminf(fmaxf(v, -kClamp), kClamp);
-            const long long fx = __float2ll_rn(v * (float)(1 << kFracBits));
-            const unsigned long long add = (1ull << 56) + (unsigned long long)(fx + kBias);
-            unsigned long long* ap = acc64 + (size_t)j * C + cc;
-            const unsigned long long old = __hip_atomic_fetch_add(ap, add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if ((old >> 56) == (unsigned long long)(S - 1)) {
-                const long long tot = (long long)((old + add) & ((1ull << 56) - 1)) - (long long)S * kBias;
-                *op = alpha * (float)((double)tot * (1.0 / (double)(1 << kFracBits)));
-                __hip_atomic_store(ap, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
+            tile[o] = v;
         }
     }
 }
 
+// Adds the `splits` partial tiles of every column block in order and writes the scaled result.
+template <int R>
+__global__ __launch_bounds__(256) void lora_grad_reduce_kernel(const float* __restrict__ part, float* __restrict__ out,
+                                                               int o_sr, int o_sc, float alpha, int C,
+                                                               int col_blocks, int splits) {
+    constexpr int CPT = 64 / R;
+    constexpr int NACC = R * CPT;
+    const int t = blockIdx.x * 256 + threadIdx.x;         // index into one split's tiles: [column block][a][lane]
+    const int total = col_blocks * NACC * 64;
+    if (t >= total) return;
+    float v = 0.f;
+    int s = 0;
+    for (; s + 8 <= splits; s += 8) {
+        float u[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) u[i] = part[(size_t)(s + i) * total + t];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v += u[i];
+    }
+    for (; s < splits; ++s) v += part[(size_t)s * total + t];
+    const int bx = t / (NACC * 64), o = t - bx * (NACC * 64);
+    const int a = o >> 6, ln = o & 63;
+    const int j = a / CPT, cc = (bx * 64 + ln) * CPT + (a - j * CPT);
+    if (cc < C) out[(size_t)j * o_sr + (size_t)cc * o_sc] = alpha * v;
+}
+
+struct GradPlan { int col_blocks, splits, rows_per_wg; };
+inline GradPlan plan_grad(int M, int C, int R) {
+    GradPlan g;
+    const int cpt = 64 / R;
+    g.col_blocks = (C + 64 * cpt - 1) / (64 * cpt);
+    // rows per workgroup: a multiple of 64 (4 wavefronts x 16 rows); about one workgroup for each of
+    // the 256 CUs, at most 32 row splits (their partial tiles cost 2*splits*R*C*4 bytes of traffic)
+    int splits = (256 + g.col_blocks - 1) / g.col_blocks;
+    if (splits > 32) splits = 32;
+    const int unit = 16 * kGradWaves;
+    g.rows_per_wg = ((M + splits - 1) / splits + unit - 1) / unit * unit;
+    g.splits = (M + g.rows_per_wg - 1) / g.rows_per_wg;
+    return g;
+}
+
 }  // namespace q4
+
+template <int RB, int WL, bool F32, int RQ>
+static void launch_down_kernel(const q4::half_t* ip, const void* w, int w_sr, int w_sc, q4::half_t* op,
+                               int M, int C, int R, hipStream_t stream) {
+    hipLaunchKernelGGL((q4::lora_down_kernel<RB, WL, F32, RQ>), dim3((M + 15) / 16), dim3(64 * q4::kDownWaves), 0, stream,
+                       ip, w, w_sr, w_sc, op, M, C, R);
+}
+
+template <int WL, bool F32>
+static void launch_down_rb(const q4::half_t* ip, const void* w, int w_sr, int w_sc, q4::half_t* op,
+                           int M, int C, int R, hipStream_t stream) {
+    switch ((R + 15) / 16) {
+        case 1: launch_down_kernel<1, WL, F32, 0>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
+        case 2: launch_down_kernel<2, WL, F32, 0>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
+        case 3: launch_down_kernel<3, WL, F32, 0>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
+        default: launch_down_kernel<4, WL, F32, 0>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
+    }
+}
+
+template <int WL, bool F32>
+static void launch_down_staged(const q4::half_t* ip, const void* w, int w_sr, int w_sc, q4::half_t* op,
+                             int M, int C, int R, hipStream_t stream) {
+    switch ((R + 3) / 4) {
+        case 1: launch_down_kernel<1, WL, F32, 1>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
+        case 2: launch_down_kernel<1, WL, F32, 2>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
+        case 3: launch_down_kernel<1, WL, F32, 3>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
+        default: launch_down_kernel<1, WL, F32, 4>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
+    }
+}
 
 extern "C" int q4_launch_lora_down(const void* in, const void* w, int w_sr, int w_sc, int w_is_f32, void* out,
                                    int M, int C, int R, hipStream_t stream) {
     using namespace q4;
-    const dim3 grid((M + 15) / 16), block(512);
     const half_t* ip = reinterpret_cast<const half_t*>(in);
     half_t* op = reinterpret_cast<half_t*>(out);
-    switch ((R + 15) / 16) {
-        case 1: hipLaunchKernelGGL(lora_down_kernel<1>, grid, block, 0, stream, ip, w, w_sr, w_sc, w_is_f32, op, M, C, R); break;
-        case 2: hipLaunchKernelGGL(lora_down_kernel<2>, grid, block, 0, stream, ip, w, w_sr, w_sc, w_is_f32, op, M, C, R); break;
-        case 3: hipLaunchKernelGGL(lora_down_kernel<3>, grid, block, 0, stream, ip, w, w_sr, w_sc, w_is_f32, op, M, C, R); break;
-        default: hipLaunchKernelGGL(lora_down_kernel<4>, grid, block, 0, stream, ip, w, w_sr, w_sc, w_is_f32, op, M, C, R); break;
+    const bool base16 = (reinterpret_cast<uintptr_t>(w) & 15u) == 0;
+    const int vec = w_is_f32 ? 4 : 8;                       // elements per 16 bytes
+    if (w_sc == 1 && base16 && w_sr % 4 == 0 && R <= 16) {
+        if (w_is_f32) launch_down_staged<kRowsT, true>(ip, w, w_sr, w_sc, op, M, C, R, stream);
+        else launch_down_staged<kRowsT, false>(ip, w, w_sr, w_sc, op, M, C, R, stream);
+    } else if (w_sc == 1 && base16 && w_sr % vec == 0) {
+        if (w_is_f32) launch_down_rb<kRows, true>(ip, w, w_sr, w_sc, op, M, C, R, stream);
+        else launch_down_rb<kRows, false>(ip, w, w_sr, w_sc, op, M, C, R, stream);
+    } else if (w_sr == 1 && base16 && w_sc % 4 == 0 && R % 4 == 0 && R <= 16 && w_sc >= R) {
+        if (w_is_f32) launch_down_staged<kCols, true>(ip, w, w_sr, w_sc, op, M, C, R, stream);
+        else launch_down_staged<kCols, false>(ip, w, w_sr, w_sc, op, M, C, R, stream);
+    } else {
+        if (w_is_f32) launch_down_rb<kAny, true>(ip, w, w_sr, w_sc, op, M, C, R, stream);
+        else launch_down_rb<kAny, false>(ip, w, w_sr, w_sc, op, M, C, R, stream);
     }
     return hipGetLastError() == hipSuccess ? 0 : -4;
+}
+
+extern "C" size_t q4_lora_grad_workspace(int M, int C, int R) {
+    const q4::GradPlan g = q4::plan_grad(M, C, R);
+    return g.splits == 1 ? 0 : (size_t)g.splits * g.col_blocks * 64 * 64 * sizeof(float);
 }
 
 extern "C" int q4_launch_lora_grad(const void* P, const void* in, float* out, int o_sr, int o_sc, float alpha,
                                    int M, int C, int R, void* workspace, hipStream_t stream) {
     using namespace q4;
-    const int cpt = 64 / R;
-    const int col_blocks = (C + 64 * cpt - 1) / (64 * cpt);
-    // rows per workgroup: a multiple of 128 (8 wavefronts x 16 rows); the LDS footprint allows one
-    // workgroup per CU, so aim at about one workgroup for each of the 256 CUs
-    int splits = (256 + col_blocks - 1) / col_blocks;
-    int rows_per_wg = ((M + splits - 1) / splits + 127) / 128 * 128;
-    if (rows_per_wg < 128) rows_per_wg = 128;
-    splits = (M + rows_per_wg - 1) / rows_per_wg;
-    if (splits > 255) { rows_per_wg = ((M + 254) / 255 + 127) / 128 * 128; splits = (M + rows_per_wg - 1) / rows_per_wg; }
-    const dim3 grid(col_blocks, splits), block(512);
+    const GradPlan g = plan_grad(M, C, R);
+    const dim3 grid(g.col_blocks, g.splits), block(64 * kGradWaves);
     const half_t* pp = reinterpret_cast<const half_t*>(P);
     const half_t* ip = reinterpret_cast<const half_t*>(in);
-    unsigned long long* ws = reinterpret_cast<unsigned long long*>(workspace);
-    if (R == 8) hipLaunchKernelGGL(lora_grad_kernel<8>, grid, block, 0, stream, pp, ip, out, o_sr, o_sc, alpha, M, C, rows_per_wg, ws);
-    else hipLaunchKernelGGL(lora_grad_kernel<16>, grid, block, 0, stream, pp, ip, out, o_sr, o_sc, alpha, M, C, rows_per_wg, ws);
+    float* ws = reinterpret_cast<float*>(workspace);
+    const int rblocks = (g.col_blocks * 64 * 64 + 255) / 256;
+    if (R == 8) {
+        hipLaunchKernelGGL(lora_grad_kernel<8>, grid, block, 0, stream, pp, ip, out, o_sr, o_sc, alpha, M, C, g.rows_per_wg, ws);
+        if (g.splits > 1)
+            hipLaunchKernelGGL(lora_grad_reduce_kernel<8>, dim3(rblocks), dim3(256), 0, stream, ws, out, o_sr, o_sc, alpha, C, g.col_blocks, g.splits);
+    } else {
+        hipLaunchKernelGGL(lora_grad_kernel<16>, grid, block, 0, stream, pp, ip, out, o_sr, o_sc, alpha, M, C, g.rows_per_wg, ws);
+        if (g.splits > 1)
+            hipLaunchKernelGGL(lora_grad_reduce_kernel<16>, dim3(rblocks), dim3(256), 0, stream, ws, out, o_sr, o_sc, alpha, C, g.col_blocks, g.splits);
+    }
     return hipGetLastError() == hipSuccess ? 0 : -4;
 }

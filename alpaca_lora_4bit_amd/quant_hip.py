@@ -23,6 +23,7 @@ _lib.lib()  # fail at import time, loudly, if the HIP library is missing
 
 MAX_GEMV_ROWS = 16
 _workspaces = {}
+_scratch_bufs = {}
 
 # Act-order layers (g_idx a real permutation): sort the packed rows by group once per layer and
 # run the sequential-group kernels on the sorted copy, gathering x through the permutation.
@@ -162,6 +163,16 @@ def _workspace(device, nbytes):
         ws = torch.zeros(max(nbytes, 1 << 22), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
+
+
+def _scratch(device, nbytes):
+    """Uninitialised scratch (partial sums); kept apart from the zero-on-entry split-K workspace."""
+    key = (device.index, _stream(device))
+    buf = _scratch_bufs.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 22), dtype=torch.uint8, device=device)
+        _scratch_bufs[key] = buf
+    return buf
 
 
 def _out_shape(out_shape, rows, cols):
@@ -343,9 +354,9 @@ def lora_grad(p, inp, alpha, transposed=False):
         out = torch.empty((R, C), dtype=torch.float32, device=dev)
         sr, sc = C, 1
     L = _lib.lib()
-    nbytes = L.q4_lora_grad_workspace_bytes(R, C)
+    nbytes = L.q4_lora_grad_workspace_bytes(M, C, R)
     with torch.cuda.device(dev):
-        ws = _workspace(dev, nbytes)
+        ws = _scratch(dev, nbytes)
         rc = L.q4_lora_grad_f32(p.data_ptr(), inp.data_ptr(), out.data_ptr(), sr, sc, float(alpha), M, C, R,
                                 ws.data_ptr(), ws.numel(), _stream(dev))
     _lib.check(rc, "q4_lora_grad_f32")

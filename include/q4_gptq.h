@@ -111,9 +111,10 @@ int q4_lora_down_f16(const void *in, const void *w, int w_sr, int w_sc, int w_is
  * with p fp16 [M, R] and in fp16 [M, C]:  dA = scaling * dyb^T @ x (out = [R, K], o_sr = K, o_sc = 1) and
  * dB = scaling * dy^T @ xa (out = lora_B.weight.grad [N, R], o_sr = 1, o_sc = R) -- what torch autograd
  * computes for the two adapter Linears of models.py:66.  R is 8 or 16, C % 8 == 0.
- * `workspace`: q4_lora_grad_workspace_bytes(R, C) = 8*R*C bytes, 256-byte aligned, zero before first
- * use and left zero by every call (64-bit fixed-point sums across workgroups: bit-reproducible). */
-size_t q4_lora_grad_workspace_bytes(int R, int C);
+ * `workspace`: q4_lora_grad_workspace_bytes(M, C, R) bytes (0 for small M: then it may be NULL), 256-byte
+ * aligned, contents irrelevant before and after the call: it carries fp32 partial sums of row blocks,
+ * which a second kernel adds in a fixed order (bit-reproducible). */
+size_t q4_lora_grad_workspace_bytes(int M, int C, int R);
 int q4_lora_grad_f32(const void *p, const void *in, float *out, int o_sr, int o_sc, float alpha,
                      int M, int C, int R, void *workspace, size_t workspace_bytes, void *stream);
 

@@ -61,10 +61,12 @@ def test_error_codes_and_validation_need_no_gpu():
     assert L.q4_lora_down_f16(fake, fake, 4096, 1, 1, fake, 64, 4100, 8, None) == -2        # C % 32
     assert L.q4_lora_down_f16(fake, fake, 4096, 1, 1, fake, 64, 4096, 65, None) == -2       # R > 64
     assert L.q4_lora_down_f16(fake, ctypes.c_void_p(0x1002), 4096, 1, 1, fake, 64, 4096, 8, None) == -5
-    assert L.q4_lora_grad_workspace_bytes(8, 4096) == 8 * 8 * 4096
+    assert L.q4_lora_grad_workspace_bytes(64, 4096, 8) == 0            # one row block: no partial sums
+    assert L.q4_lora_grad_workspace_bytes(2048, 4096, 8) == 32 * 8 * 64 * 64 * 4
+    assert L.q4_lora_grad_workspace_bytes(2048, 4096, 12) == 0
     assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 64, 4096, 12, fake, 1 << 20, None) == -2   # R not 8/16
-    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 64, 4096, 8, None, 0, None) == -3
-    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 64, 4096, 8, fake, 1024, None) == -3
+    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 2048, 4096, 8, None, 0, None) == -3
+    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 2048, 4096, 8, fake, 1024, None) == -3
     assert L.q4_gemv_workspace_bytes(16, 4096, 11008) == 16 * 11008 * 8
     assert L.q4_gemv_workspace_bytes(0, 4096, 11008) == 0
 

@@ -35,6 +35,10 @@ def test_lora_down_both_layouts(M, C, R, wdtype):
     got_t = quant_hip.lora_down(xd, wt.t()).float().cpu().numpy()
     assert np.abs(got_t - ref).max() <= tol
     assert np.array_equal(got, got_t)                                           # same arithmetic either way
+    big = torch.zeros((R, C + 3), dtype=wdtype, device="cuda")                 # odd row pitch, unaligned start
+    big[:, 1:C + 1] = wd
+    got_v = quant_hip.lora_down(xd, big[:, 1:C + 1]).float().cpu().numpy()
+    assert np.array_equal(got, got_v)
 
 
 @pytest.mark.parametrize("M,C,R", [(2048, 4096, 8), (2048, 11008, 8), (2048, 4096, 16), (77, 64, 8),
@@ -58,13 +62,21 @@ def test_lora_grad_matches_fp32_product(M, C, R):
     assert torch.equal(got, again)
 
 
-def test_lora_grad_leaves_workspace_zero():
+def test_lora_grad_does_not_disturb_gemv_workspace(oracle):
+    """The gradient's partial sums live in their own scratch: a GEMV (whose split-K workspace must stay
+    zero between calls) gives the same result before and after."""
     from alpaca_lora_4bit_amd import quant_hip
     rng = np.random.default_rng(3)
-    pd = torch.from_numpy(_rand16(rng, 2048, 8)).cuda()
-    xd = torch.from_numpy(_rand16(rng, 2048, 4096)).cuda()
+    layer = oracle.make_layer(4096, 256, 128, seed=2)
+    t = lambda a: torch.from_numpy(a).cuda()
+    q, z, sc = t(layer["qweight"]), t(layer["qzeros"]), t(layer["scales"])
+    x = t(oracle.make_activations(1, 4096, seed=9))
+    y0 = quant_hip.gemv(x, q, z, sc, None, 128).clone()
+    pd = t(_rand16(rng, 2048, 8))
+    xd = t(_rand16(rng, 2048, 4096))
     quant_hip.lora_grad(pd, xd, 1.0)
-    torch.cuda.synchronize()
+    y1 = quant_hip.gemv(x, q, z, sc, None, 128)
+    assert torch.equal(y0, y1)
     for ws in quant_hip._workspaces.values():
         assert int(ws.count_nonzero()) == 0
 
