@@ -276,6 +276,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy: a kernel of known traffic for scaling rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--lora-step-only", action="store_true",
+                    help="run only the config-2 LoRA layer step (forward + backward, M=2048) and print its figures: "
+                         "a short run for profiling the GEMM and adapter kernels")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU's share of the path only; --gpus must be 1 "
@@ -287,6 +290,10 @@ def main():
     torch.cuda.set_device(0)
     from alpaca_lora_4bit_amd import quant_hip  # noqa: F401  (fails loudly if the HIP library is missing)
 
+    if args.lora_step_only:
+        r = bench_lora_step(max(args.steps, 5))
+        print(json.dumps({"workload": "config2_lora_fwd_bwd_M2048", **{k: round(v, 4) for k, v in r.items()}}))
+        return
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
         dst = torch.empty_like(src)
