@@ -53,7 +53,36 @@ struct GemmArgs {
     int R;
     half_t* out;              // fwd: y [M,N]      bwd: dx [M,K]
     int M, K, N, G;
+    int phase_step;           // rotation of the reduction loop per row tile, in steps of 64
 };
+
+// Which output tile a workgroup computes, and where in the reduction it starts.
+//  * Workgroups are handed to the 8 XCDs round-robin in dispatch order.  The ids are permuted so that one
+//    XCD owns a contiguous range of tiles in column-major order: a few column tiles for all row tiles.
+//    Its L2 then holds few columns of W, spread over several L2 channels, and each slab of activations
+//    is fetched once per XCD and shared by its column tiles.
+//  * Activation rows of a power-of-two pitch (K = 4096: 8 KB) put one reduction slab of ALL rows into
+//    a single L2 channel; workgroups marching through the reduction in lockstep then queue on that one
+//    channel.  Row tile r therefore starts its (cyclic) reduction loop phase_step * r steps later.
+struct TileMap {
+    int tile_c, tile_r, phase;
+};
+__device__ __forceinline__ TileMap map_tile(int phase_step, int nsteps) {
+    const int nc = gridDim.x, nr = gridDim.y, total = nc * nr;
+    int id = blockIdx.y * nc + blockIdx.x;
+    if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
+    TileMap m;
+    m.tile_c = id / nr;
+    m.tile_r = id - m.tile_c * nr;
+    m.phase = (m.tile_r * phase_step) % nsteps;
+    return m;
+}
+// reduction offset of pipeline stage `stage` (stages past the end repeat the last one: harmless reloads)
+__device__ __forceinline__ int red_of(int stage, int nsteps, int phase) {
+    int v = min(stage, nsteps - 1) + phase;
+    if (v >= nsteps) v -= nsteps;
+    return v * BK;
+}
 
 __device__ __forceinline__ float adapter_at(const GemmArgs& a, size_t idx) {
     return a.lb_is_f32 ? reinterpret_cast<const float*>(a.lb)[idx] : (float)reinterpret_cast<const half_t*>(a.lb)[idx];
@@ -105,16 +134,21 @@ struct FwdSlab {
         voff_s = (n0 + col) * 2;
         voff_z = ((n0 + col) >> 3) * 4;
     }
-    // raw loads only: any arithmetic on the loaded values here would wait for them before the MFMAs
-    __device__ __forceinline__ void load(const GemmArgs& a, const SlabRsrc& r, int, int kred0) {
-        const int soff = (kred0 >> 3) * a.N * 4;
-#pragma unroll
-        for (int i = 0; i < NW; ++i) w[i] = buf_load32(r.w, voff_w + i * wstride, soff);
-        if (!GIDX) {
-            const int g = kred0 / a.groupsize;
-            s_raw = buf_load16(r.s, voff_s, g * a.N * 2);
-            z_raw = buf_load32(r.z, voff_z, g * (a.N >> 3) * 4);
+    // raw loads only: any arithmetic on the loaded values here would wait for them before the MFMAs.
+    // The loads of a slab are kLoads separate pieces so that the main loop can issue them one at a time.
+    static constexpr int kLoads = GIDX ? NW : NW + 2;
+    template <int I>
+    __device__ __forceinline__ void load_part(const GemmArgs& a, const SlabRsrc& r, int kred0) {
+        if constexpr (I < NW) {
+            w[I] = buf_load32(r.w, voff_w + I * wstride, (kred0 >> 3) * a.N * 4);
+        } else if constexpr (I == NW) {
+            s_raw = buf_load16(r.s, voff_s, (kred0 / a.groupsize) * a.N * 2);
+        } else {
+            z_raw = buf_load32(r.z, voff_z, (kred0 / a.groupsize) * (a.N >> 3) * 4);
         }
+    }
+    __device__ __forceinline__ void load(const GemmArgs& a, const SlabRsrc& r, int, int kred0) {
+        static_for<0, kLoads>([&](auto ic) { load_part<decltype(ic)::value>(a, r, kred0); });
     }
     template <int I>
     __device__ __forceinline__ void store_slice(const GemmArgs& a, int n0, int kred0, half_t* sB) {
@@ -188,12 +222,15 @@ struct BwdSlab {
         voff_s = (g * a.N + 4 * n4) * 2;
         voff_z = (g * (a.N >> 3) + (n4 >> 1)) * 4;
     }
-    __device__ __forceinline__ void load(const GemmArgs&, const SlabRsrc& r, int, int nred0) {
-        w = buf_load128(r.w, voff_w, nred0 * 4);
-        if (!GIDX) {
-            sv = buf_load64(r.s, voff_s, nred0 * 2);
-            zw = buf_load32(r.z, voff_z, (nred0 >> 3) * 4);       // shifted in the slices: no ALU on loaded data here
-        }
+    static constexpr int kLoads = GIDX ? 1 : 3;
+    template <int I>
+    __device__ __forceinline__ void load_part(const GemmArgs&, const SlabRsrc& r, int nred0) {
+        if constexpr (I == 0) w = buf_load128(r.w, voff_w, nred0 * 4);
+        else if constexpr (I == 1) sv = buf_load64(r.s, voff_s, nred0 * 2);
+        else zw = buf_load32(r.z, voff_z, (nred0 >> 3) * 4);     // shifted in the slices: no ALU on loaded data here
+    }
+    __device__ __forceinline__ void load(const GemmArgs& a, const SlabRsrc& r, int, int nred0) {
+        static_for<0, kLoads>([&](auto ic) { load_part<decltype(ic)::value>(a, r, nred0); });
     }
     template <int I>
     __device__ __forceinline__ void store_slice(const GemmArgs& a, int kout0, int nred0, half_t* sB) {
@@ -276,8 +313,10 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     const int wm = wave >> 1, wn = wave & 1;
     const int NOUT = FWD ? a.N : a.K;
     const int RED = FWD ? a.K : a.N;
-    const int m0 = blockIdx.y * BM;
-    const int c0 = blockIdx.x * BN;          // first output column of the tile
+    const int nsteps = RED / BK;              // even: RED is a multiple of 128
+    const TileMap tm = map_tile(a.phase_step, nsteps);
+    const int m0 = tm.tile_r * BM;
+    const int c0 = tm.tile_c * BN;           // first output column of the tile
     const int rows_valid = min(BM, a.M - m0);
 
     // buffer descriptors: activations of this workgroup's rows (rows beyond M read as zero), weights
@@ -330,8 +369,6 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
             bf[j] = *reinterpret_cast<const half8_t*>(pb + b_off + 32 * j * LDS_STRIDE + 16 * ks);
     };
 
-    const int nsteps = RED / BK;              // even: RED is a multiple of 128
-    const int last = (nsteps - 1) * BK;
     half8_t af[2][TM], bf[2][2];              // operand fragments, double buffered over the sub-steps
 
     // One pipeline step, branch-free.  CUR = LDS buffer / register set of the stage being multiplied:
@@ -341,13 +378,20 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     auto step = [&](int s, auto cur_tag) {
         constexpr int CUR = decltype(cur_tag)::value;
         constexpr int NM = TM * 2 * KS;                        // MFMAs per step
-        constexpr int NITEM = 2 + NSL + NA;                    // side-work items per step
         constexpr int BAR = NM - 4;                            // MFMA index after which the barrier sits
+        // Side work of a step: NL global loads (stage s+2 -> register set CUR) and NC consumer items
+        // (stage s+1: register set CUR^1 -> LDS[CUR^1]; NSL dequantization slices with the NA activation
+        // stores spread evenly among them).  One load per MFMA slot from slot 0 on (never a burst: eight
+        // wavefronts issuing ten loads each at once stall on the address unit), the consumers spread over
+        // slots 0..BAR-2 so that the last LDS stores have two MFMAs to drain before the barrier.
+        constexpr int NLS = Slab::kLoads, NL = NLS + NA, NC = NSL + NA;
+        constexpr int SLOTS = BAR - 1;
+        static_assert(SLOTS >= 1, "too few MFMAs per step");
         // fragment set 0 is reloaded right after the barrier: every MFMA of sub-step KS-2 (its last
         // user in this step) must have been issued by then
         static_assert(BAR >= (KS - 1) * TM * 2 - 1, "barrier placed before the last use of fragment set 0");
-        const int red_next2 = min((s + 2) * BK, last);
-        const int red_next1 = min((s + 1) * BK, last);
+        const int red_next2 = red_of(s + 2, nsteps, tm.phase);
+        const int red_next1 = red_of(s + 1, nsteps, tm.phase);
         const half_t* const a_cur = CUR ? sA1 : sA0;
         const half_t* const b_cur = CUR ? sB1 : sB0;
         half_t* const a_nxt = CUR ? sA0 : sA1;
@@ -358,17 +402,24 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
             if constexpr (r == 0 && ks + 1 < KS)
                 read_frags(af[(ks + 1) & 1], bf[(ks + 1) & 1], a_cur, b_cur, ks + 1);
             acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[ks & 1][ti], bf[ks & 1][tj], acc[ti][tj], 0, 0, 0);
-            // side work is spread over MFMAs 0..BAR so that it is complete when the barrier comes
-            constexpr int j_lo = i <= BAR ? (i * NITEM) / (BAR + 1) : NITEM;
-            constexpr int j_hi = i <= BAR ? ((i + 1) * NITEM) / (BAR + 1) : NITEM;
-            static_for<j_lo, j_hi>([&](auto jc) {
-                constexpr int j = decltype(jc)::value;
-                if constexpr (j == 0) slab[CUR].load(a, rs, c0, red_next2);
-                else if constexpr (j == 1) load_a(areg[CUR], red_next2);
-                else if constexpr (j < 2 + NSL) slab[CUR ^ 1].template store_slice<j - 2>(a, c0, red_next1, b_nxt);
+            // loads l with l*SLOTS/NL == i, consumers q with q*SLOTS/NC == i
+            constexpr int l_lo = i < SLOTS ? (i * NL + SLOTS - 1) / SLOTS : NL;
+            constexpr int l_hi = i < SLOTS ? ((i + 1) * NL + SLOTS - 1) / SLOTS : NL;
+            static_for<l_lo, l_hi>([&](auto lc) {
+                constexpr int l = decltype(lc)::value;
+                if constexpr (l < NLS) slab[CUR].template load_part<l>(a, rs, red_next2);
+                else areg[CUR][l - NLS] = buf_load128(rs_a, voff_a + (l - NLS) * astride, red_next2 * 2);
+            });
+            constexpr int q_lo = i < SLOTS ? (i * NC + SLOTS - 1) / SLOTS : NC;
+            constexpr int q_hi = i < SLOTS ? ((i + 1) * NC + SLOTS - 1) / SLOTS : NC;
+            static_for<q_lo, q_hi>([&](auto qc) {
+                constexpr int q = decltype(qc)::value;
+                constexpr int na_before = q * NA / NC;                       // activation stores among items 0..q-1
+                constexpr bool is_a = (q + 1) * NA / NC > na_before;
+                if constexpr (is_a)
+                    *reinterpret_cast<uint4_t*>(a_nxt + (arow + APASS * na_before) * LDS_STRIDE + acol) = areg[CUR ^ 1][na_before];
                 else
-                    *reinterpret_cast<uint4_t*>(a_nxt + (arow + APASS * (j - 2 - NSL)) * LDS_STRIDE + acol) =
-                        areg[CUR ^ 1][j - 2 - NSL];
+                    slab[CUR ^ 1].template store_slice<q - na_before>(a, c0, red_next1, b_nxt);
             });
             if constexpr (i == BAR) {
                 // every wavefront has finished reading LDS[CUR] (the last fragments were fetched at
@@ -380,12 +431,13 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
         });
     };
 
-    load_a(areg[0], 0);
-    slab[0].load(a, rs, c0, 0);
-    load_a(areg[1], min(BK, last));
-    slab[1].load(a, rs, c0, min(BK, last));
+    const int red0 = red_of(0, nsteps, tm.phase), red1 = red_of(1, nsteps, tm.phase);
+    load_a(areg[0], red0);
+    slab[0].load(a, rs, c0, red0);
+    load_a(areg[1], red1);
+    slab[1].load(a, rs, c0, red1);
     store_a(areg[0], sA0);
-    static_for<0, NSL>([&](auto jc) { slab[0].template store_slice<decltype(jc)::value>(a, c0, 0, sB0); });
+    static_for<0, NSL>([&](auto jc) { slab[0].template store_slice<decltype(jc)::value>(a, c0, red0, sB0); });
     __syncthreads();
     read_frags(af[0], bf[0], sA0, sB0, 0);
     for (int s = 0; s < nsteps; s += 2) {
@@ -485,6 +537,8 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     a.R = (la && lb) ? R : 0;
     a.out = reinterpret_cast<half_t*>(out);
     a.M = M; a.K = K; a.N = N; a.G = G;
+    static const int env_phase = getenv("Q4_GEMM_PHASE") ? atoi(getenv("Q4_GEMM_PHASE")) : 2;
+    a.phase_step = env_phase < 0 ? 0 : env_phase;
     const int nout = fwd ? N : K;
     const bool gidx = g_idx != nullptr;
     // tile configuration: 256-row tiles once they still give every CU a workgroup
