@@ -302,3 +302,16 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
                 db = torch.mm(dy.t(), xa).float().mul_(ctx.scaling)
             db = db.to(ctx.ab_dtypes[1])
         return dx, None, None, None, None, None, da, db, None, None
+
+
+_LOADER_NAMES = ('load_llama_model_4bit_low_ram', 'load_llama_model_4bit_low_ram_and_offload',
+                 'load_llama_model_4bit_low_ram_and_offload_to_cpu')
+
+
+def __getattr__(name):
+    # the reference defines its loaders in this module (autograd_4bit.py:250-360); here they live in
+    # loaders.py (which imports this module) and are resolved lazily under the same names
+    if name in _LOADER_NAMES:
+        from . import loaders
+        return getattr(loaders, name)
+    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
