@@ -84,3 +84,30 @@ def test_loaded_model_logits_match_dense_reference(tmp_path, oracle, act_order):
     out = model.generate(ids.cuda(), max_new_tokens=3, do_sample=False)
     assert out.shape == (1, 27)
     assert int(out[0, 24]) == int(ref[0, -1].argmax())
+
+
+@pytest.mark.gpu
+def test_fused_qkv_and_gate_up_keep_the_logits(tmp_path, oracle):
+    """make_quant_attn / make_fused_mlp (model_attn_mlp_patch.py:73-247 of the reference): three / two projections
+    become one launch each; the model's own attention and MLP code keeps running on slice views."""
+    from alpaca_lora_4bit_amd import autograd_4bit as ag
+    from alpaca_lora_4bit_amd.model_attn_mlp_patch import FusedProjectionSlice, make_fused_mlp, make_quant_attn
+    path = str(tmp_path / "ckpt")
+    build(path, oracle, seed=4, with_tokenizer=True)
+    model, _ = ag.load_llama_model_4bit_low_ram(path, os.path.join(path, "model.safetensors"), groupsize=GROUPSIZE,
+                                                half=True, device_map={"": 0})
+    ids = torch.tensor([[1] + [5 + (7 * i) % 200 for i in range(23)]]).cuda()
+    with torch.no_grad():
+        before, before1 = model(ids).logits.float(), model(ids[:, :1]).logits.float()
+    n_quant = sum(isinstance(m, ag.Autograd4bitQuantLinear) for m in model.modules())
+    assert make_quant_attn(model) == 2 and make_fused_mlp(model) == 2
+    layer0 = model.model.layers[0]
+    assert isinstance(layer0.self_attn.q_proj, FusedProjectionSlice) and isinstance(layer0.mlp.up_proj, FusedProjectionSlice)
+    assert layer0.self_attn.qkv_proj.out_features == 3 * 256 and layer0.mlp.gate_up_proj.out_features == 2 * 512
+    assert sum(isinstance(m, ag.Autograd4bitQuantLinear) for m in model.modules()) == n_quant - 2 * 3   # 5 -> 2 per block
+    assert not any(k.endswith("q_proj.qweight") for k in model.state_dict())                          # no duplicate state
+    with torch.no_grad():
+        after, after1 = model(ids).logits.float(), model(ids[:, :1]).logits.float()
+    for a, b in ((after, before), (after1, before1)):
+        assert (a - b).abs().max().item() <= 2e-3 * b.abs().max().item()
+    assert make_quant_attn(model) == 0                       # idempotent: nothing left to fuse
