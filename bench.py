@@ -207,6 +207,88 @@ def bench_lora_step(reps, seed=5):
                 eager_ms=eager * 1e3, eager_tokens_per_s=M / eager)
 
 
+def bench_llama7b_lora_train_step(reps=4, seed=11, n_layers=32, batch=4, seq=256):
+    """BASELINE configs[4]: random-init 32-layer LLaMA-7B decoder, every q/k/v/o/gate/up/down projection a 4-bit
+    GPTQ layer (groupsize 128), LoRA r=8 alpha=16 on q_proj / v_proj, one forward + backward + AdamW step on
+    batch 4 x seq 256 random token ids under fp16 autocast, gradient checkpointing off.  Eager PyTorch around
+    the HIP kernels (attention = torch SDPA, lm_head = library GEMM)."""
+    import torch
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from alpaca_lora_4bit_amd import autograd_4bit as ag
+    from alpaca_lora_4bit_amd.models import inject_lora_layers
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    config = LlamaConfig(vocab_size=32000, hidden_size=4096, intermediate_size=11008, num_hidden_layers=n_layers,
+                         num_attention_heads=32, num_key_value_heads=32, max_position_embeddings=2048,
+                         tie_word_embeddings=False)
+    with torch.device("meta"):
+        model = LlamaForCausalLM(config)
+    layers = ag.find_layers(model)
+    layers.pop("lm_head", None)
+    ag.make_quant_for_4bit_autograd(model, layers, groupsize=128)
+    model = model.to_empty(device="cuda")
+    with torch.no_grad():
+        for name, mod in model.named_modules():
+            if isinstance(mod, ag.Autograd4bitQuantLinear):
+                K, N = mod.in_features, mod.out_features
+                lay = make_layer_gpu(K, N, 128, gen)
+                mod.qweight, mod.qzeros = lay["qweight"], lay["qzeros"]
+                # about unit gain per layer (W entries ~ 6.5 * scale): activations stay finite through 32 layers
+                mod.scales = (lay["scales"].float() * (0.15 / K ** 0.5 / 0.0125)).half()
+                mod.g_idx = (torch.arange(K, device="cuda") // 128).to(torch.int32)
+                mod.bias = torch.zeros(N, dtype=torch.float16, device="cuda")
+        for name, p_ in model.named_parameters():
+            if p_.dim() >= 2:
+                p_.normal_(0, 0.02, generator=gen)
+            else:
+                p_.fill_(1.0)
+    ag.model_to_half(model)
+    head_dim = config.hidden_size // config.num_attention_heads
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, head_dim, 2, device="cuda", dtype=torch.float32) / head_dim))
+    for mod in model.modules():                      # rotary tables are plain buffers that to_empty left blank
+        if hasattr(mod, "inv_freq"):
+            mod.inv_freq = inv_freq.clone()
+            if hasattr(mod, "original_inv_freq"):
+                mod.original_inv_freq = inv_freq.clone()
+    lora = inject_lora_layers(model, target_modules=("q_proj", "v_proj"), r=8, lora_alpha=16)
+    with torch.no_grad():
+        for l in lora.values():
+            l.lora_B["default"].weight.normal_(0, 0.02, generator=gen)
+    params = [p_ for p_ in model.parameters() if p_.requires_grad]
+    opt = torch.optim.AdamW(params, lr=1e-4)
+    ids = torch.randint(0, 32000, (batch, seq), device="cuda", generator=gen)
+    model.train()
+    model.config.use_cache = False
+
+    def step():
+        opt.zero_grad(set_to_none=True)
+        with torch.amp.autocast(device_type="cuda", dtype=torch.float16):
+            loss = model(input_ids=ids, labels=ids).loss
+        (loss * 1024.0).backward()
+        opt.step()
+        return loss
+
+    for _ in range(2):
+        loss = step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        loss = step()
+    e1.record()
+    torch.cuda.synchronize()
+    per = e0.elapsed_time(e1) * 1e-3 / reps
+    tokens = batch * seq
+    n_quant = sum(m.in_features * m.out_features for m in model.modules() if isinstance(m, ag.Autograd4bitQuantLinear))
+    flop = 2 * 2 * tokens * n_quant                  # forward + grad-input products of the 4-bit layers
+    out = dict(ms_per_step=per * 1e3, tokens_per_s=tokens / per, loss=float(loss.detach()), lora_layers=len(lora),
+               quant_params=n_quant, tflops_4bit_layers=flop / per / 1e12,
+               frac_mfma_4bit_layers=flop / per / 1e12 / MFMA_FP16_PEAK_TFLOPS,
+               gpu_mem_gb=torch.cuda.max_memory_allocated() / 1e9)
+    del model, opt, params, lora
+    torch.cuda.empty_cache()
+    return out
+
+
 def bench_gemm_only(M, K, N, act_order, reps, seed=7):
     import torch
     from alpaca_lora_4bit_amd import quant_hip
@@ -276,6 +358,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy: a kernel of known traffic for scaling rocprofv3 "
                          "FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--llama7b-step-only", action="store_true",
+                    help="run only the config-4 full-model LoRA training step (32-layer LLaMA-7B shapes, random init)")
     ap.add_argument("--lora-step-only", action="store_true",
                     help="run only the config-2 LoRA layer step (forward + backward, M=2048) and print its figures: "
                          "a short run for profiling the GEMM and adapter kernels")
@@ -290,6 +374,10 @@ def main():
     torch.cuda.set_device(0)
     from alpaca_lora_4bit_amd import quant_hip  # noqa: F401  (fails loudly if the HIP library is missing)
 
+    if args.llama7b_step_only:
+        r = bench_llama7b_lora_train_step(max(args.steps, 2))
+        print(json.dumps({"workload": "config4_llama7b_lora_train_step_b4_s256", **{k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()}}))
+        return
     if args.lora_step_only:
         r = bench_lora_step(max(args.steps, 5))
         print(json.dumps({"workload": "config2_lora_fwd_bwd_M2048", **{k: round(v, 4) for k, v in r.items()}}))
@@ -347,6 +435,12 @@ def main():
         extra["config2_gemm_kernels"] = {k: {kk: round(vv, 4) for kk, vv in v.items()} for k, v in gm.items()}
         g3 = bench_gemm_only(512, 5120, 13824, True, 10)
         extra["config3_actorder_M512"] = {k: {kk: round(vv, 4) for kk, vv in v.items()} for k, v in g3.items()}
+        try:
+            c4 = bench_llama7b_lora_train_step(4)
+            extra["config4_llama7b_lora_train_step_b4_s256"] = {k: (round(v, 4) if isinstance(v, float) else v)
+                                                                  for k, v in c4.items()}
+        except Exception as e:                       # the headline line must not depend on the installed transformers
+            extra["config4_llama7b_lora_train_step_b4_s256"] = {"error": f"{type(e).__name__}: {e}"[:300]}
         out["extra"] = extra
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
