@@ -6,7 +6,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libq4gptq.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _lib = None
 
@@ -19,8 +19,9 @@ SIGNATURES = {
     "q4_permute_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "q4_gemv_workspace_bytes": (_sz, [_i, _i, _i]),
     "q4_gemv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
-    "q4_gemm_fwd_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _i, _vp, _i, _i, _i, _i, _vp]),
-    "q4_gemm_bwd_dx_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _i, _vp, _i, _i, _i, _i, _vp]),
+    "q4_gemm_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "q4_gemm_fwd_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _i, _vp, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "q4_gemm_bwd_dx_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _i, _vp, _i, _i, _i, _i, _vp, _sz, _vp]),
     "q4_lora_down_f16": (_i, [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp]),
     "q4_lora_grad_workspace_bytes": (_sz, [_i, _i, _i]),
     "q4_lora_grad_f32": (_i, [_vp, _vp, _vp, _i, _i, _f, _i, _i, _i, _vp, _sz, _vp]),

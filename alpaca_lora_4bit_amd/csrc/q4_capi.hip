@@ -10,7 +10,8 @@ int q4_launch_permute_rows(const int32_t*, const int32_t*, int32_t*, int, int, h
 int q4_launch_gemv(const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, void*, int,
                    int, int, int, int, void*, hipStream_t);
 int q4_launch_gemm(int, const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, const void*,
-                   const void*, const void*, int, int, int, float, int, void*, int, int, int, int, hipStream_t);
+                   const void*, const void*, int, int, int, float, int, void*, int, int, int, int, void*, size_t, hipStream_t);
+size_t q4_gemm_plan_workspace(int, int, int, int);
 int q4_launch_lora_down(const void*, const void*, int, int, int, void*, int, int, int, hipStream_t);
 int q4_launch_lora_grad(const void*, const void*, float*, int, int, float, int, int, int, void*, hipStream_t);
 size_t q4_lora_grad_workspace(int, int, int);
@@ -33,7 +34,7 @@ int check_layer(const void* qweight, const void* qzeros, const void* scales, con
 }
 }  // namespace
 
-extern "C" int q4_abi_version(void) { return 3; }
+extern "C" int q4_abi_version(void) { return 4; }
 
 extern "C" const char* q4_error_string(int code) {
     switch (code) {
@@ -83,7 +84,7 @@ extern "C" int q4_gemv_f16(const void* x, const int32_t* qweight, const int32_t*
 static int gemm_common(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros, const void* scales,
                        const int32_t* g_idx, int groupsize, const void* bias, const void* la, const void* lb,
                        int lb_sr, int lb_sc, int lb_is_f32, float lb_scale, int R,
-                       void* out, int M, int K, int N, int G, void* stream) {
+                       void* out, int M, int K, int N, int G, void* workspace, size_t workspace_bytes, void* stream) {
     int rc = check_layer(qweight, qzeros, scales, g_idx, groupsize, K, N, G);
     if (rc != Q4_OK) return rc;
     if (!act || !out) return Q4_ERR_NULL_POINTER;
@@ -97,24 +98,32 @@ static int gemm_common(int fwd, const void* act, const int32_t* qweight, const i
     if (misaligned(act) || misaligned(out) || (la && misaligned(la))) return Q4_ERR_MISALIGNED;
     if (lb && (reinterpret_cast<uintptr_t>(lb) & (lb_is_f32 ? 3u : 1u))) return Q4_ERR_MISALIGNED;
     if (lb && (lb_sr < 1 || lb_sc < 1)) return Q4_ERR_BAD_SHAPE;
+    if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
     return q4_launch_gemm(fwd, act, qweight, qzeros, scales, g_idx, groupsize, bias, la, lb, lb_sr, lb_sc, lb_is_f32,
-                          lb_scale, R, out, M, K, N, G, (hipStream_t)stream);
+                          lb_scale, R, out, M, K, N, G, workspace, workspace ? workspace_bytes : 0, (hipStream_t)stream);
 }
 
 extern "C" int q4_gemm_fwd_f16(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
                                const int32_t* g_idx, int groupsize, const void* bias,
                                const void* xa, const void* lora_b, int ldb_r, int ldb_n, int lora_is_f32,
-                               float lora_scale, int R, void* y, int M, int K, int N, int G, void* stream) {
+                               float lora_scale, int R, void* y, int M, int K, int N, int G,
+                               void* workspace, size_t workspace_bytes, void* stream) {
     return gemm_common(1, x, qweight, qzeros, scales, g_idx, groupsize, bias, xa, lora_b, ldb_r, ldb_n, lora_is_f32,
-                       lora_scale, R, y, M, K, N, G, stream);
+                       lora_scale, R, y, M, K, N, G, workspace, workspace_bytes, stream);
 }
 
 extern "C" int q4_gemm_bwd_dx_f16(const void* dy, const int32_t* qweight, const int32_t* qzeros, const void* scales,
                                   const int32_t* g_idx, int groupsize,
                                   const void* dyb, const void* lora_a, int lda_r, int lda_k, int lora_is_f32,
-                                  float lora_scale, int R, void* dx, int M, int K, int N, int G, void* stream) {
+                                  float lora_scale, int R, void* dx, int M, int K, int N, int G,
+                                  void* workspace, size_t workspace_bytes, void* stream) {
     return gemm_common(0, dy, qweight, qzeros, scales, g_idx, groupsize, nullptr, dyb, lora_a, lda_r, lda_k, lora_is_f32,
-                       lora_scale, R, dx, M, K, N, G, stream);
+                       lora_scale, R, dx, M, K, N, G, workspace, workspace_bytes, stream);
+}
+
+extern "C" size_t q4_gemm_workspace_bytes(int fwd, int M, int K, int N) {
+    if (M < 1 || K < 128 || N < 128) return 0;
+    return q4_gemm_plan_workspace(fwd, M, K, N);
 }
 
 extern "C" int q4_lora_down_f16(const void* in, const void* w, int w_sr, int w_sc, int w_is_f32, void* out,

@@ -54,6 +54,7 @@ struct GemmArgs {
     half_t* out;              // fwd: y [M,N]      bwd: dx [M,K]
     int M, K, N, G;
     int phase_step;           // rotation of the reduction loop per row tile, in steps of 64
+    float* part;              // split-K: fp32 partial outputs [gridDim.z][M][NOUT] (gridDim.z > 1 only)
 };
 
 // Which output tile a workgroup computes, and where in the reduction it starts.
@@ -67,7 +68,7 @@ struct GemmArgs {
 struct TileMap {
     int tile_c, tile_r, phase;
 };
-__device__ __forceinline__ TileMap map_tile(int phase_step, int nsteps) {
+__device__ __forceinline__ TileMap map_tile(int phase_step, int nsteps) {   // nsteps: steps of THIS workgroup
     const int nc = gridDim.x, nr = gridDim.y, total = nc * nr;
     int id = blockIdx.y * nc + blockIdx.x;
     if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
@@ -77,11 +78,23 @@ __device__ __forceinline__ TileMap map_tile(int phase_step, int nsteps) {
     m.phase = (m.tile_r * phase_step) % nsteps;
     return m;
 }
+// Split-K: gridDim.z workgroups share an output tile; workgroup z owns `cnt` consecutive steps from `begin`.
+struct StepRange {
+    int begin, cnt;
+};
+__device__ __forceinline__ StepRange split_steps(int nsteps) {
+    const int S = gridDim.z, z = blockIdx.z;
+    const int base = nsteps / S, rem = nsteps - base * S;
+    StepRange r;
+    r.cnt = base + (z < rem ? 1 : 0);
+    r.begin = z * base + min(z, rem);
+    return r;
+}
 // reduction offset of pipeline stage `stage` (stages past the end repeat the last one: harmless reloads)
-__device__ __forceinline__ int red_of(int stage, int nsteps, int phase) {
-    int v = min(stage, nsteps - 1) + phase;
-    if (v >= nsteps) v -= nsteps;
-    return v * BK;
+__device__ __forceinline__ int red_of(int stage, StepRange sr, int phase) {
+    int v = min(stage, sr.cnt - 1) + phase;
+    if (v >= sr.cnt) v -= sr.cnt;
+    return (sr.begin + v) * BK;
 }
 
 __device__ __forceinline__ float adapter_at(const GemmArgs& a, size_t idx) {
@@ -313,8 +326,8 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     const int wm = wave >> 1, wn = wave & 1;
     const int NOUT = FWD ? a.N : a.K;
     const int RED = FWD ? a.K : a.N;
-    const int nsteps = RED / BK;              // even: RED is a multiple of 128
-    const TileMap tm = map_tile(a.phase_step, nsteps);
+    const StepRange sr = split_steps(RED / BK);
+    const TileMap tm = map_tile(a.phase_step, sr.cnt);
     const int m0 = tm.tile_r * BM;
     const int c0 = tm.tile_c * BN;           // first output column of the tile
     const int rows_valid = min(BM, a.M - m0);
@@ -390,8 +403,8 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
         // fragment set 0 is reloaded right after the barrier: every MFMA of sub-step KS-2 (its last
         // user in this step) must have been issued by then
         static_assert(BAR >= (KS - 1) * TM * 2 - 1, "barrier placed before the last use of fragment set 0");
-        const int red_next2 = red_of(s + 2, nsteps, tm.phase);
-        const int red_next1 = red_of(s + 1, nsteps, tm.phase);
+        const int red_next2 = red_of(s + 2, sr, tm.phase);
+        const int red_next1 = red_of(s + 1, sr, tm.phase);
         const half_t* const a_cur = CUR ? sA1 : sA0;
         const half_t* const b_cur = CUR ? sB1 : sB0;
         half_t* const a_nxt = CUR ? sA0 : sA1;
@@ -431,7 +444,7 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
         });
     };
 
-    const int red0 = red_of(0, nsteps, tm.phase), red1 = red_of(1, nsteps, tm.phase);
+    const int red0 = red_of(0, sr, tm.phase), red1 = red_of(1, sr, tm.phase);
     load_a(areg[0], red0);
     slab[0].load(a, rs, c0, red0);
     load_a(areg[1], red1);
@@ -440,11 +453,12 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     static_for<0, NSL>([&](auto jc) { slab[0].template store_slice<decltype(jc)::value>(a, c0, red0, sB0); });
     __syncthreads();
     read_frags(af[0], bf[0], sA0, sB0, 0);
-    for (int s = 0; s < nsteps; s += 2) {
+    for (int s = 0; s + 1 < sr.cnt; s += 2) {
         step(s, std::integral_constant<int, 0>{});
         step(s + 1, std::integral_constant<int, 1>{});
     }
-    if (a.R > 0) {
+    if (sr.cnt & 1) step(sr.cnt - 1, std::integral_constant<int, 0>{});   // an even number of steps precedes it: LDS[0]
+    if (a.R > 0 && blockIdx.z == 0) {
         // rank-R adapter step: activations [M, R] (columns beyond R are zero), adapter matrix from lb
         __syncthreads();
         const rsrc_t rs_l = make_rsrc(a.la + (size_t)m0 * a.R, (unsigned)rows_valid * (unsigned)a.R * 2u);
@@ -469,9 +483,27 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     // epilogue: acc[i][j][r] is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of its 32x32 tile.
     // Each wavefront transposes one 32 x 64 block at a time through its own 4.5 KB of LDS
     // (row stride 72 halves) and writes it as 16-byte pieces: 8 lanes cover one 128-byte row segment.
+    const int lc = lane & 31, lrow = (lane >> 5) * 4;
+    if (gridDim.z > 1) {
+        // split-K: fp32 partial sums straight from the accumulators (32 lanes cover one 128-byte row segment);
+        // the bias rides with split 0, the reduction kernel adds the splits in order and rounds once
+        float* const pz = a.part + (size_t)blockIdx.z * a.M * NOUT;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int col = c0 + wn * 64 + 32 * j + lc;
+                const float bv = (FWD && a.bias && blockIdx.z == 0) ? (float)a.bias[col] : 0.f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int m = m0 + wm * WROWS + 32 * i + 8 * (r >> 2) + lrow + (r & 3);
+                    if (m < a.M) pz[(size_t)m * NOUT + col] = acc[i][j][r] + bv;
+                }
+            }
+        return;
+    }
     __syncthreads();
     half_t* stage = sA0 + wave * (32 * LDS_STRIDE);
-    const int lc = lane & 31, lrow = (lane >> 5) * 4;
     const int orow = lane >> 3, ocol = (lane & 7) * 8;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -500,20 +532,66 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     }
 }
 
+// out fp16 [n] = sum over the splits of part[s][n], added in order (bit-reproducible), rounded once.
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ part, half_t* __restrict__ out,
+                                                                 long total, int splits) {
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= total) return;                       // total is a multiple of 4 (NOUT % 128 == 0)
+    float4_t v = *reinterpret_cast<const float4_t*>(part + i);
+    for (int s = 1; s < splits; ++s) {
+        const float4_t u = *reinterpret_cast<const float4_t*>(part + (size_t)s * total + i);
+        v[0] += u[0]; v[1] += u[1]; v[2] += u[2]; v[3] += u[3];
+    }
+    half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+    *reinterpret_cast<half4_t*>(out + i) = h;
+}
+
 template <int BM, int WGM, bool FWD, bool GIDX>
-static hipError_t launch_gemm(const GemmArgs& a, int nout, hipStream_t stream) {
-    const dim3 grid(nout / BN, (a.M + BM - 1) / BM);
+static hipError_t launch_gemm(const GemmArgs& a, int nout, int splits, hipStream_t stream) {
+    const dim3 grid(nout / BN, (a.M + BM - 1) / BM, splits);
     hipLaunchKernelGGL((gemm_kernel<BM, WGM, FWD, GIDX>), grid, dim3(128 * WGM), 0, stream, a);
+    if (splits > 1) {
+        const long total = (long)a.M * nout;
+        hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream,
+                           a.part, a.out, total, splits);
+    }
     return hipGetLastError();
 }
 
 template <bool FWD, bool GIDX>
-static hipError_t launch_gemm_cfg(int cfg, const GemmArgs& a, int nout, hipStream_t stream) {
+static hipError_t launch_gemm_cfg(int cfg, const GemmArgs& a, int nout, int splits, hipStream_t stream) {
     switch (cfg) {
-        case 0: return launch_gemm<128, 2, FWD, GIDX>(a, nout, stream);    // 128 x 128, 4 wavefronts of 64 x 64
-        case 1: return launch_gemm<256, 2, FWD, GIDX>(a, nout, stream);    // 256 x 128, 4 wavefronts of 128 x 64
-        default: return launch_gemm<256, 4, FWD, GIDX>(a, nout, stream);   // 256 x 128, 8 wavefronts of 64 x 64
+        case 0: return launch_gemm<128, 2, FWD, GIDX>(a, nout, splits, stream);    // 128 x 128, 4 wavefronts of 64 x 64
+        case 1: return launch_gemm<256, 2, FWD, GIDX>(a, nout, splits, stream);    // 256 x 128, 4 wavefronts of 128 x 64
+        default: return launch_gemm<256, 4, FWD, GIDX>(a, nout, splits, stream);   // 256 x 128, 8 wavefronts of 64 x 64
     }
+}
+
+// Launch plan shared by q4_launch_gemm and q4_gemm_plan_workspace.  Few output tiles (small M) leave most CUs
+// idle while each tile walks the whole reduction: the reduction is then split over gridDim.z workgroups that
+// write fp32 partial tiles, about 1.5 workgroups per CU in total.
+struct GemmPlan {
+    int cfg, splits;
+};
+static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
+    static const int env_cfg = getenv("Q4_GEMM_CFG") ? atoi(getenv("Q4_GEMM_CFG")) : -1;
+    static const int env_splits = getenv("Q4_GEMM_SPLITS") ? atoi(getenv("Q4_GEMM_SPLITS")) : 0;
+    GemmPlan p;
+    const bool tall = (long)(nout / BN) * ((M + 255) / 256) >= 200;
+    p.cfg = env_cfg >= 0 ? env_cfg : (tall ? 2 : 0);
+    const int bm = p.cfg == 0 ? 128 : 256;
+    const long tiles = (long)(nout / BN) * ((M + bm - 1) / bm);
+    const int nsteps = red / BK;
+    int splits = 1;
+    if (tiles < 192) {
+        splits = (int)((384 + tiles - 1) / tiles);
+        if (splits > 8) splits = 8;                            // measured: more splits only add prologues and partial tiles
+        if (splits > nsteps / 4) splits = nsteps / 4;          // at least four steps per workgroup
+    }
+    if (env_splits > 0) splits = env_splits > nsteps ? nsteps : env_splits;
+    while (splits > 1 && (size_t)splits * (size_t)M * (size_t)nout * sizeof(float) > workspace_bytes) --splits;
+    p.splits = splits < 1 ? 1 : splits;
+    return p;
 }
 
 }  // namespace q4
@@ -521,7 +599,8 @@ static hipError_t launch_gemm_cfg(int cfg, const GemmArgs& a, int nout, hipStrea
 extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros,
                               const void* scales, const int32_t* g_idx, int groupsize, const void* bias,
                               const void* la, const void* lb, int lb_sr, int lb_sc, int lb_is_f32, float lb_scale, int R,
-                              void* out, int M, int K, int N, int G, hipStream_t stream) {
+                              void* out, int M, int K, int N, int G, void* workspace, size_t workspace_bytes,
+                              hipStream_t stream) {
     using namespace q4;
     GemmArgs a;
     a.a = reinterpret_cast<const half_t*>(act);
@@ -541,12 +620,19 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     a.phase_step = env_phase < 0 ? 0 : env_phase;
     const int nout = fwd ? N : K;
     const bool gidx = g_idx != nullptr;
-    // tile configuration: 256-row tiles once they still give every CU a workgroup
-    static const int env_cfg = getenv("Q4_GEMM_CFG") ? atoi(getenv("Q4_GEMM_CFG")) : -1;
-    const bool tall = (long)(nout / BN) * ((M + 255) / 256) >= 200;
-    const int cfg = env_cfg >= 0 ? env_cfg : (tall ? 2 : 0);
+    // tile configuration: 256-row tiles once they still give every CU a workgroup; split-K for few tiles
+    const GemmPlan p = plan_gemm(M, fwd ? K : N, nout, workspace ? workspace_bytes : 0);
+    a.part = reinterpret_cast<float*>(workspace);
     hipError_t e;
-    if (fwd) e = gidx ? launch_gemm_cfg<true, true>(cfg, a, nout, stream) : launch_gemm_cfg<true, false>(cfg, a, nout, stream);
-    else e = gidx ? launch_gemm_cfg<false, true>(cfg, a, nout, stream) : launch_gemm_cfg<false, false>(cfg, a, nout, stream);
+    if (fwd) e = gidx ? launch_gemm_cfg<true, true>(p.cfg, a, nout, p.splits, stream) : launch_gemm_cfg<true, false>(p.cfg, a, nout, p.splits, stream);
+    else e = gidx ? launch_gemm_cfg<false, true>(p.cfg, a, nout, p.splits, stream) : launch_gemm_cfg<false, false>(p.cfg, a, nout, p.splits, stream);
     return e == hipSuccess ? 0 : -4;
+}
+
+// Workspace that lets q4_launch_gemm use its preferred split for this shape (0: no split wanted).
+extern "C" size_t q4_gemm_plan_workspace(int fwd, int M, int K, int N) {
+    using namespace q4;
+    const int nout = fwd ? N : K;
+    const GemmPlan p = plan_gemm(M, fwd ? K : N, nout, ~(size_t)0);
+    return p.splits > 1 ? (size_t)p.splits * (size_t)M * (size_t)nout * sizeof(float) : 0;
 }

@@ -175,6 +175,15 @@ def _scratch(device, nbytes):
     return buf
 
 
+def _gemm_scratch(L, device, fwd, M, K, N):
+    """(pointer, bytes) of the split-K scratch the GEMM would like for this shape, or (None, 0)."""
+    nbytes = L.q4_gemm_workspace_bytes(fwd, M, K, N)
+    if nbytes == 0:
+        return None, 0
+    buf = _scratch(device, nbytes)
+    return buf.data_ptr(), buf.numel()
+
+
 def _out_shape(out_shape, rows, cols):
     if out_shape is None:
         return (rows, cols)
@@ -281,10 +290,12 @@ def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, 
     else:
         gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
     out = torch.empty(_out_shape(out_shape, M, N), dtype=torch.float16, device=dev)
+    L = _lib.lib()
     with torch.cuda.device(dev):
-        rc = _lib.lib().q4_gemm_fwd_f16(x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
-                                        gp, gs, _ptr(bias), _ptr(xa), _ptr(lora_bt), sr, sc, f32, float(lora_scale), R,
-                                        out.data_ptr(), M, K, N, G, _stream(dev))
+        wp, wn = _gemm_scratch(L, dev, 1, M, K, N)
+        rc = L.q4_gemm_fwd_f16(x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
+                               gp, gs, _ptr(bias), _ptr(xa), _ptr(lora_bt), sr, sc, f32, float(lora_scale), R,
+                               out.data_ptr(), M, K, N, G, wp, wn, _stream(dev))
     _lib.check(rc, "q4_gemm_fwd_f16")
     return out
 
@@ -305,10 +316,12 @@ def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=Non
     dyb, lora_a, R, sr, sc, f32 = _lora_pair(dyb, lora_a, M, K, dev)
     gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
     out = torch.empty(_out_shape(out_shape, M, K), dtype=torch.float16, device=dev)
+    L = _lib.lib()
     with torch.cuda.device(dev):
-        rc = _lib.lib().q4_gemm_bwd_dx_f16(dy2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
-                                           gp, gs, _ptr(dyb), _ptr(lora_a), sr, sc, f32, float(lora_scale), R,
-                                           out.data_ptr(), M, K, N, G, _stream(dev))
+        wp, wn = _gemm_scratch(L, dev, 0, M, K, N)
+        rc = L.q4_gemm_bwd_dx_f16(dy2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
+                                  gp, gs, _ptr(dyb), _ptr(lora_a), sr, sc, f32, float(lora_scale), R,
+                                  out.data_ptr(), M, K, N, G, wp, wn, _stream(dev))
     _lib.check(rc, "q4_gemm_bwd_dx_f16")
     return out
 

@@ -83,11 +83,17 @@ int q4_gemv_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, co
  * bias, xa, lora_b may be NULL; R is 0 or a multiple of 8, at most 64.
  * Both GEMM entry points need K % 128 == 0, N % 128 == 0, K*N < 2^33, and with g_idx == NULL also
  * groupsize % 64 == 0 and every |scale| < 64 (the sequential-group dequant forms s*q with a fused
- * multiply-add on 1024+q; pass g_idx to lift the restriction on the scales). */
+ * multiply-add on 1024+q; pass g_idx to lift the restriction on the scales).
+ * `workspace` (optional, may be NULL; 256-byte aligned, contents irrelevant): with few output tiles (small M)
+ * the reduction is split over several workgroups per tile that leave fp32 partial tiles in it, added in a
+ * fixed order by a second kernel.  q4_gemm_workspace_bytes(fwd, M, K, N) is the size that allows the
+ * preferred split (0 when none is wanted); a smaller workspace means fewer splits, none means no split. */
+size_t q4_gemm_workspace_bytes(int fwd, int M, int K, int N);
 int q4_gemm_fwd_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                     const int32_t *g_idx, int groupsize, const void *bias,
                     const void *xa, const void *lora_b, int ldb_r, int ldb_n, int lora_is_f32, float lora_scale,
-                    int R, void *y, int M, int K, int N, int G, void *stream);
+                    int R, void *y, int M, int K, int N, int G,
+                    void *workspace, size_t workspace_bytes, void *stream);
 
 /* Backward GEMM (grad of the input):
  *   dx fp16 [M, K] = dy fp16 [M, N] @ W^T  (+ lora_scale * dyb fp16 [M, R] @ Am [R, K])
@@ -98,7 +104,8 @@ int q4_gemm_fwd_f16(const void *x, const int32_t *qweight, const int32_t *qzeros
 int q4_gemm_bwd_dx_f16(const void *dy, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                        const int32_t *g_idx, int groupsize,
                        const void *dyb, const void *lora_a, int lda_r, int lda_k, int lora_is_f32, float lora_scale,
-                       int R, void *dx, int M, int K, int N, int G, void *stream);
+                       int R, void *dx, int M, int K, int N, int G,
+                       void *workspace, size_t workspace_bytes, void *stream);
 
 /* Rank-R down projection of the adapter:  out fp16 [M, R] = in fp16 [M, C] @ Wm^T,
  * Wm[j, c] = w[j*w_sr + c*w_sc] (fp16, or fp32 when w_is_f32 != 0).  xa = x @ A^T (w = lora_A.weight,

@@ -51,11 +51,15 @@ def test_error_codes_and_validation_need_no_gpu():
     assert L.q4_gemv_f16(fake, fake, fake, fake, None, 128, fake, 0, 17, 256, 128, 2, fake, 1 << 20, None) == -2
     assert L.q4_gemv_f16(fake, fake, fake, fake, None, 128, fake, 0, 1, 256, 128, 2, None, 0, None) == -3
     assert L.q4_gemv_f16(fake, fake, fake, fake, None, 128, fake, 0, 1, 256, 128, 2, fake, 8, None) == -3
-    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, None, None, 0, 0, 0, 1.0, 0, fake, 64, 192, 128, 2, None) == -2
-    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, None, 1, 8, 0, 1.0, 8, fake, 64, 256, 128, 2, None) == -1
-    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, fake, 1, 12, 0, 1.0, 12, fake, 64, 256, 128, 2, None) == -2
-    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, fake, 0, 8, 1, 1.0, 8, fake, 64, 256, 128, 2, None) == -2
-    assert L.q4_gemm_bwd_dx_f16(fake, fake, fake, fake, None, 32, None, None, 0, 0, 0, 1.0, 0, fake, 64, 256, 128, 8, None) == -2
+    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, None, None, 0, 0, 0, 1.0, 0, fake, 64, 192, 128, 2, None, 0, None) == -2
+    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, None, 1, 8, 0, 1.0, 8, fake, 64, 256, 128, 2, None, 0, None) == -1
+    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, fake, 1, 12, 0, 1.0, 12, fake, 64, 256, 128, 2, None, 0, None) == -2
+    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, fake, 0, 8, 1, 1.0, 8, fake, 64, 256, 128, 2, None, 0, None) == -2
+    assert L.q4_gemm_bwd_dx_f16(fake, fake, fake, fake, None, 32, None, None, 0, 0, 0, 1.0, 0, fake, 64, 256, 128, 8, None, 0, None) == -2
+    assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, None, None, 0, 0, 0, 1.0, 0, fake, 64, 256, 128, 2, ctypes.c_void_p(0x1010), 1 << 20, None) == -5
+    assert L.q4_gemm_workspace_bytes(1, 2048, 4096, 4096) == 0            # enough tiles: no split
+    assert L.q4_gemm_workspace_bytes(1, 64, 4096, 4096) == 8 * 64 * 4096 * 4    # 32 tiles -> 8 splits of fp32 partials
+    assert L.q4_gemm_workspace_bytes(0, 64, 4096, 11008) == 8 * 64 * 4096 * 4
     # adapter helpers
     assert L.q4_lora_down_f16(fake, None, 4096, 1, 1, fake, 64, 4096, 8, None) == -1
     assert L.q4_lora_down_f16(fake, fake, 4096, 1, 1, fake, 64, 4100, 8, None) == -2        # C % 32

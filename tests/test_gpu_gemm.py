@@ -15,7 +15,8 @@ def _t(a):
 
 
 @pytest.mark.parametrize("K,N,gs,act", [(256, 128, 128, False), (256, 256, 64, False), (512, 384, 128, True),
-                                        (4096, 4096, 128, False), (1024, 256, 1024, False)])
+                                        (4096, 4096, 128, False), (1024, 256, 1024, False),
+                                        (1408, 256, 128, False), (1408, 256, 128, True)])   # 22 steps: uneven split-K
 @pytest.mark.parametrize("M", [17, 128, 300])
 def test_gemm_forward(oracle, K, N, gs, act, M):
     import torch
@@ -31,7 +32,7 @@ def test_gemm_forward(oracle, K, N, gs, act, M):
 
 
 @pytest.mark.parametrize("K,N,gs,act", [(256, 128, 128, False), (256, 256, 64, False), (512, 384, 128, True),
-                                        (4096, 4096, 128, False)])
+                                        (4096, 4096, 128, False), (256, 1408, 128, False)])   # reduction of 22 steps
 @pytest.mark.parametrize("M", [17, 128, 300])
 def test_gemm_backward_dx(oracle, K, N, gs, act, M):
     import torch
@@ -110,3 +111,22 @@ def test_gemm_rejects_unsupported_shapes(oracle):
     x = _t(oracle.make_activations(32, 192, seed=1))
     with pytest.raises(quant_hip.Q4Error):
         quant_hip.gemm_fwd(x, t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 64)
+
+
+def test_split_k_is_reproducible_and_matches_unsplit(oracle):
+    """Few tiles: the reduction is split and the fp32 partial tiles are added in a fixed order."""
+    import torch
+    from alpaca_lora_4bit_amd import _lib, quant_hip
+    K, N, M = 4096, 512, 40
+    assert _lib.lib().q4_gemm_workspace_bytes(1, M, K, N) > 0            # this shape does get split
+    layer = oracle.make_layer(K, N, 128, seed=77)
+    t = to_cuda_layer(layer)
+    x = torch.from_numpy(oracle.make_activations(M, K, seed=4)).cuda()
+    bias = torch.randn(N, device="cuda").half()
+    y1 = quant_hip.gemm_fwd(x, t["qweight"], t["qzeros"], t["scales"], None, 128, bias=bias)
+    y2 = quant_hip.gemm_fwd(x, t["qweight"], t["qzeros"], t["scales"], None, 128, bias=bias)
+    assert torch.equal(y1, y2)
+    ref = oracle.matmul_recons(x.cpu().numpy(), layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
+    ref = ref + bias.float().cpu().numpy()
+    err = np.abs(y1.float().cpu().numpy() - ref).max()
+    assert err <= 1e-2 * np.abs(ref).max()
