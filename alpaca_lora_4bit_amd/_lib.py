@@ -19,6 +19,8 @@ SIGNATURES = {
     "q4_permute_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "q4_gemv_workspace_bytes": (_sz, [_i, _i, _i]),
     "q4_gemv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "q4_dequant_v1_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
+    "q4_dequant2_f16": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp]),
     "q4_gemm_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "q4_gemm_fwd_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _i, _vp, _i, _i, _i, _i, _vp, _sz, _vp]),
     "q4_gemm_bwd_dx_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _i, _vp, _i, _i, _i, _i, _vp, _sz, _vp]),

@@ -47,8 +47,10 @@ try:
         @staticmethod
         @custom_fwd(device_type='cuda', cast_inputs=torch.float16)
         def forward(ctx, x, qweight, scales, zeros, g_idx, bits, maxq):
-            if g_idx is None or zeros.dtype != torch.int32:
-                mm4b._v1_unsupported()
+            ctx.is_v1 = zeros.dtype != torch.int32
+            if ctx.is_v1:                                   # per-column fp zeros: dense dequant + library GEMM
+                ctx.save_for_backward(qweight, scales, zeros)
+                return mm4b._matmul4bit_v1_recons(x, qweight, scales, zeros)
             ctx.save_for_backward(qweight, scales, zeros, g_idx)
             rows = x.numel() // x.shape[-1]
             if 1 <= rows <= quant_hip.MAX_GEMV_ROWS:
@@ -58,22 +60,35 @@ try:
         @staticmethod
         @custom_bwd(device_type='cuda')
         def backward(ctx, grad_output):
-            qweight, scales, zeros, g_idx = ctx.saved_tensors
             grad = None
+            if ctx.is_v1:
+                qweight, scales, zeros = ctx.saved_tensors
+                if ctx.needs_input_grad[0]:
+                    grad = mm4b._matmul4bit_v1_recons(grad_output, qweight, scales, zeros, transpose=True)
+                return grad, None, None, None, None, None, None
+            qweight, scales, zeros, g_idx = ctx.saved_tensors
             if ctx.needs_input_grad[0]:
                 grad = mm4b._matmul4bit_v2_recons(grad_output, qweight, scales, zeros, g_idx, transpose=True)
             return grad, None, None, None, None, None, None
 
     class AutogradMatmul2bitCuda(torch.autograd.Function):
-        """2-bit checkpoints are outside what is built for gfx950."""
+        """2-bit v2 layers: dense dequant on the GPU + library GEMM, forward and backward
+        (autograd_4bit.py:56-72)."""
 
         @staticmethod
+        @custom_fwd(device_type='cuda', cast_inputs=torch.float16)
         def forward(ctx, x, qweight, scales, zeros, g_idx, bits, maxq):
-            mm4b._v1_unsupported()
+            ctx.save_for_backward(qweight, scales, zeros, g_idx)
+            return mm4b._matmul2bit_v2_recons(x, qweight, scales, zeros, g_idx)
 
         @staticmethod
+        @custom_bwd(device_type='cuda')
         def backward(ctx, grad_output):
-            mm4b._v1_unsupported()
+            qweight, scales, zeros, g_idx = ctx.saved_tensors
+            grad = None
+            if ctx.needs_input_grad[0]:
+                grad = mm4b._matmul2bit_v2_recons(grad_output, qweight, scales, zeros, g_idx, transpose=True)
+            return grad, None, None, None, None, None, None
 
     gptq_backend_loaded = True
 except ImportError:

@@ -58,6 +58,29 @@ extern "C" int q4_dequant_f16(const int32_t* qweight, const int32_t* qzeros, con
     return q4_launch_dequant(qweight, qzeros, scales, g_idx, groupsize, out, K, N, (hipStream_t)stream);
 }
 
+extern "C" {
+int q4_launch_dequant_v1(const int32_t*, const void*, const void*, void*, int, int, hipStream_t);
+int q4_launch_dequant2(const int32_t*, const int32_t*, const void*, const int32_t*, int, void*, int, int, hipStream_t);
+}
+
+extern "C" int q4_dequant_v1_f16(const int32_t* qweight, const void* scales, const void* zeros, void* out,
+                                 int K, int N, void* stream) {
+    if (!qweight || !scales || !zeros || !out) return Q4_ERR_NULL_POINTER;
+    if (K < 8 || N < 64 || (K % 8) != 0 || (N % 64) != 0) return Q4_ERR_BAD_SHAPE;
+    if (misaligned(qweight) || misaligned(scales) || misaligned(zeros) || misaligned(out)) return Q4_ERR_MISALIGNED;
+    return q4_launch_dequant_v1(qweight, scales, zeros, out, K, N, (hipStream_t)stream);
+}
+
+extern "C" int q4_dequant2_f16(const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                               const int32_t* g_idx, int groupsize, void* out, int K, int N, int G, void* stream) {
+    if (!qweight || !qzeros || !scales || !out) return Q4_ERR_NULL_POINTER;
+    if (K < 16 || N < 64 || (K % 16) != 0 || (N % 64) != 0 || G < 1) return Q4_ERR_BAD_SHAPE;
+    if (!g_idx && (groupsize < 16 || (groupsize % 16) != 0 || (long long)G * groupsize < K)) return Q4_ERR_BAD_SHAPE;
+    if (misaligned(qweight) || misaligned(scales) || misaligned(out) || (reinterpret_cast<uintptr_t>(qzeros) & 3u))
+        return Q4_ERR_MISALIGNED;
+    return q4_launch_dequant2(qweight, qzeros, scales, g_idx, groupsize, out, K, N, (hipStream_t)stream);
+}
+
 extern "C" int q4_permute_rows(const int32_t* qweight, const int32_t* perm, int32_t* out, int K, int N, void* stream) {
     if (!qweight || !perm || !out) return Q4_ERR_NULL_POINTER;
     if (K < 8 || N < 1 || (K % 8) != 0) return Q4_ERR_BAD_SHAPE;

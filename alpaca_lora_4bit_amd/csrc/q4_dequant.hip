@@ -76,7 +76,100 @@ __global__ __launch_bounds__(256) void permute_rows_kernel(const uint32_t* __res
     out[tid] = word;
 }
 
+// v1 layout: one fp16 scale and one fp16 zero per column, W = rn16(rn16(s*q) - zero)
+// (src/alpaca_lora_4bit/quant_cuda/quant_cuda_kernel.cu:1076-1097).  Same thread mapping as dequant_kernel.
+__global__ __launch_bounds__(256) void dequant_v1_kernel(const uint32_t* __restrict__ qweight,
+                                                         const half_t* __restrict__ scales,
+                                                         const half_t* __restrict__ zeros,
+                                                         half_t* __restrict__ out, int K, int N) {
+    const int ncol8 = N >> 3;
+    const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (tid >= (long)(K >> 3) * ncol8) return;
+    const int kw = (int)(tid / ncol8);
+    const int n0 = (int)(tid - (long)kw * ncol8) << 3;
+    const uint4_t* wp = reinterpret_cast<const uint4_t*>(qweight + (size_t)kw * N + n0);
+    const uint4_t wa = wp[0], wb = wp[1];
+    const uint32_t w[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+    const uint4_t sv = *reinterpret_cast<const uint4_t*>(scales + n0);
+    const uint4_t zv = *reinterpret_cast<const uint4_t*>(zeros + n0);
+    const uint32_t sraw[4] = {sv.x, sv.y, sv.z, sv.w}, zraw[4] = {zv.x, zv.y, zv.z, zv.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        uint32_t o[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const uint32_t codes = ((w[2 * p] >> (4 * e)) & 0xFu) | (((w[2 * p + 1] >> (4 * e)) & 0xFu) << 16);
+            o[p] = as_u32(dequant_pair(codes_to_half2(codes), as_half2(sraw[p]), as_half2(zraw[p])));
+        }
+        *reinterpret_cast<uint4_t*>(out + (size_t)((kw << 3) + e) * N + n0) = uint4_t{o[0], o[1], o[2], o[3]};
+    }
+}
+
+// 2-bit v2 layout: sixteen codes per word along K, sixteen zero codes per word along N, zero point = code + 1,
+// W = rn16(rn16(s*q) - rn16(s*(z+1)))  (quant_cuda_kernel.cu:1185-1211).  One thread = one packed word-row
+// (16 rows) x 8 columns.
+__global__ __launch_bounds__(256) void dequant2_kernel(const uint32_t* __restrict__ qweight,
+                                                       const uint32_t* __restrict__ qzeros,
+                                                       const half_t* __restrict__ scales,
+                                                       const int32_t* __restrict__ g_idx, int groupsize,
+                                                       half_t* __restrict__ out, int K, int N) {
+    const int ncol8 = N >> 3;
+    const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (tid >= (long)(K >> 4) * ncol8) return;
+    const int kw = (int)(tid / ncol8);
+    const int nb = (int)(tid - (long)kw * ncol8);
+    const int n0 = nb << 3;
+    const uint4_t* wp = reinterpret_cast<const uint4_t*>(qweight + (size_t)kw * N + n0);
+    const uint4_t wa = wp[0], wb = wp[1];
+    const uint32_t w[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+    int gprev = -1;
+    half2_t s2[4], zero2[4];
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        const int k = (kw << 4) + e;
+        const int g = g_idx ? g_idx[k] : k / groupsize;
+        if (g != gprev) {
+            gprev = g;
+            const uint4_t sv = *reinterpret_cast<const uint4_t*>(scales + (size_t)g * N + n0);
+            // 8 adjacent columns are half of one packed zero word (16 codes of 2 bits)
+            const uint32_t zw = qzeros[(size_t)g * (N >> 4) + (n0 >> 4)] >> ((n0 & 8) * 2);
+            const uint32_t sraw[4] = {sv.x, sv.y, sv.z, sv.w};
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                s2[p] = as_half2(sraw[p]);
+                zero2[p] = zero_term(s2[p], (zw >> (4 * p)) & 0x3u, (zw >> (4 * p + 2)) & 0x3u);
+            }
+        }
+        uint32_t o[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const uint32_t codes = ((w[2 * p] >> (2 * e)) & 0x3u) | (((w[2 * p + 1] >> (2 * e)) & 0x3u) << 16);
+            o[p] = as_u32(dequant_pair(codes_to_half2(codes), s2[p], zero2[p]));
+        }
+        *reinterpret_cast<uint4_t*>(out + (size_t)k * N + n0) = uint4_t{o[0], o[1], o[2], o[3]};
+    }
+}
+
 }  // namespace q4
+
+extern "C" int q4_launch_dequant_v1(const int32_t* qweight, const void* scales, const void* zeros, void* out,
+                                    int K, int N, hipStream_t stream) {
+    const long total = (long)(K / 8) * (N / 8);
+    hipLaunchKernelGGL(q4::dequant_v1_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                       reinterpret_cast<const uint32_t*>(qweight), reinterpret_cast<const q4::half_t*>(scales),
+                       reinterpret_cast<const q4::half_t*>(zeros), reinterpret_cast<q4::half_t*>(out), K, N);
+    return hipGetLastError() == hipSuccess ? 0 : -4;
+}
+
+extern "C" int q4_launch_dequant2(const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                                  const int32_t* g_idx, int groupsize, void* out, int K, int N, hipStream_t stream) {
+    const long total = (long)(K / 16) * (N / 8);
+    hipLaunchKernelGGL(q4::dequant2_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                       reinterpret_cast<const uint32_t*>(qweight), reinterpret_cast<const uint32_t*>(qzeros),
+                       reinterpret_cast<const q4::half_t*>(scales), g_idx, groupsize,
+                       reinterpret_cast<q4::half_t*>(out), K, N);
+    return hipGetLastError() == hipSuccess ? 0 : -4;
+}
 
 extern "C" int q4_launch_permute_rows(const int32_t* qweight, const int32_t* perm, int32_t* out, int K, int N,
                                       hipStream_t stream) {

@@ -92,21 +92,52 @@ def _matmul4bit_v2_recons(x, qweight, scales, zeros, g_idx, transpose=False, gro
                                  out_shape=lead + (qweight.shape[0] * 8,))
 
 
-def _v1_unsupported(*args, **kwargs):
-    raise NotImplementedError('the v1 (per-column fp zeros) and 2-bit layouts are not built for gfx950; '
-                              'only 4-bit v2 checkpoints (int32 qzeros) are supported')
+def _dense_matmul(x, w, transpose):
+    # the dense buffer is fp16; activations follow it (the reference multiplies in the buffer's dtype)
+    xh = x if x.dtype == torch.float16 else x.half()
+    return torch.matmul(xh, w.t() if transpose else w)
 
 
-_matmul4bit_v1 = _v1_unsupported
-_matmul4bit_v1_recons = _v1_unsupported
-_matmul2bit_v2_recons = _v1_unsupported
-v2_to_v1 = _v1_unsupported
+def _matmul4bit_v1_recons(x, qweight, scales, zeros, transpose=False):
+    """v1 layers (one fp scale / zero per column): dense dequant on the GPU, then a library GEMM
+    (matmul_utils_4bit.py:98-111).  The fused kernels of this package cover the v2 layout only."""
+    if not transpose:
+        assert qweight.shape[0] * 8 == x.shape[-1]
+    else:
+        assert qweight.shape[1] == x.shape[-1]
+    return _dense_matmul(x, quant_hip.dequant_v1(qweight, scales, zeros), transpose)
+
+
+def _matmul4bit_v1(x, qweight, scales, zeros):
+    """matmul_utils_4bit.py:36-56: same result through the dense path (no dedicated v1 GEMV here)."""
+    assert qweight.shape[0] * 8 == x.shape[-1]
+    return _matmul4bit_v1_recons(x, qweight, scales, zeros).to(x.dtype)
+
+
+def _matmul2bit_v2_recons(x, qweight, scales, zeros, g_idx, transpose=False):
+    """2-bit v2 layers: dense dequant + library GEMM (matmul_utils_4bit.py:130-143)."""
+    if not transpose:
+        assert qweight.shape[0] * 16 == x.shape[-1]
+    else:
+        assert qweight.shape[1] == x.shape[-1]
+    return _dense_matmul(x, quant_hip.dequant2(qweight, zeros, _half_scales(scales), g_idx), transpose)
+
+
+def v2_to_v1(scales, zeros):
+    """Zero points of a single-group v2 layer as v1 fp zeros: scales * (z + 1)
+    (matmul_utils_4bit.py:173-186, which builds the same numbers through vecquant4recons_v1)."""
+    assert zeros.shape[0] == 1
+    N = scales.shape[-1]
+    shifts = (torch.arange(N, device=zeros.device) % 8) * 4
+    z = (zeros.reshape(-1)[torch.arange(N, device=zeros.device) // 8] >> shifts) & 0xF
+    return z.to(torch.float16) * scales + scales
 
 
 def matmul4bit(x, qweight, scales, zeros, g_idx=None, groupsize=None):
     """No-grad dispatcher, matmul_utils_4bit.py:146-170."""
     if zeros.dtype != torch.int32:
-        return _v1_unsupported()
+        # v1 layout (matmul_utils_4bit.py:148-156)
+        return _matmul4bit_v1_recons(x.half(), qweight, scales.half(), zeros.half())
     gs = _groupsize_of(qweight, scales, groupsize)
     rows = int(np.prod(x.shape[:-1]))
     thd = min(int(auto_switch_thd), quant_hip.MAX_GEMV_ROWS)

@@ -221,6 +221,60 @@ def dequant(qweight, qzeros, scales, g_idx=None, groupsize=None, out=None):
     return out
 
 
+def dequant_v1(qweight, scales, zeros, out=None):
+    """W fp16 [K, N] of a v1 layer (per-column fp16 scale and zero), bit-exact with vecquant4recons_v1
+    (quant_cuda_kernel.cu:1076-1097)."""
+    _require(qweight.is_cuda and qweight.dtype == torch.int32 and qweight.dim() == 2 and qweight.is_contiguous(),
+             "qweight must be a contiguous int32 [K/8, N] CUDA tensor")
+    dev = qweight.device
+    K, N = qweight.shape[0] * 8, qweight.shape[1]
+    s1 = scales.reshape(-1)
+    z1 = zeros.reshape(-1)
+    _require(s1.numel() == N and z1.numel() == N and s1.device == dev and z1.device == dev,
+             "v1 scales and zeros hold one value per column")
+    s1 = s1 if s1.dtype == torch.float16 else s1.half()
+    z1 = z1 if z1.dtype == torch.float16 else z1.half()
+    s1, z1 = s1.contiguous(), z1.contiguous()
+    _require(N % 64 == 0, "N must be a multiple of 64")
+    if out is None:
+        out = torch.empty((K, N), dtype=torch.float16, device=dev)
+    _require(out.dtype == torch.float16 and tuple(out.shape) == (K, N) and out.is_contiguous() and out.device == dev,
+             "out must be a contiguous float16 [K, N] tensor on the same device")
+    with torch.cuda.device(dev):
+        rc = _lib.lib().q4_dequant_v1_f16(qweight.data_ptr(), s1.data_ptr(), z1.data_ptr(), out.data_ptr(), K, N,
+                                          _stream(dev))
+    _lib.check(rc, "q4_dequant_v1_f16")
+    return out
+
+
+def dequant2(qweight, qzeros, scales, g_idx=None, groupsize=None, out=None):
+    """W fp16 [K, N] of a 2-bit v2 layer (qweight [K/16, N], qzeros [G, N/16]), bit-exact with
+    vecquant2recons_v2 (quant_cuda_kernel.cu:1185-1211)."""
+    for name, tns, dt in (("qweight", qweight, torch.int32), ("qzeros", qzeros, torch.int32), ("scales", scales, torch.float16)):
+        _require(tns.is_cuda and tns.dtype == dt and tns.dim() == 2 and tns.is_contiguous(),
+                 f"{name} must be a contiguous 2-D {dt} CUDA tensor")
+    dev = qweight.device
+    K, N = qweight.shape[0] * 16, qweight.shape[1]
+    G = scales.shape[0]
+    _require(N % 64 == 0 and tuple(scales.shape) == (G, N) and tuple(qzeros.shape) == (G, N // 16)
+             and qzeros.device == dev and scales.device == dev, "2-bit layer shapes do not match")
+    gp, gs = 0, int(groupsize or -(-K // G))
+    if g_idx is not None:
+        _require(g_idx.dtype == torch.int32 and g_idx.numel() == K and g_idx.device == dev and g_idx.is_contiguous(),
+                 "g_idx must be a contiguous int32 [K] tensor on the same device")
+        if classify_g_idx(g_idx, gs, G) != "seq" or gs % 16 != 0:
+            gp = g_idx.data_ptr()
+    if out is None:
+        out = torch.empty((K, N), dtype=torch.float16, device=dev)
+    _require(out.dtype == torch.float16 and tuple(out.shape) == (K, N) and out.is_contiguous() and out.device == dev,
+             "out must be a contiguous float16 [K, N] tensor on the same device")
+    with torch.cuda.device(dev):
+        rc = _lib.lib().q4_dequant2_f16(qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), gp, gs,
+                                        out.data_ptr(), K, N, G, _stream(dev))
+    _lib.check(rc, "q4_dequant2_f16")
+    return out
+
+
 def gemv(x, qweight, qzeros, scales, g_idx=None, groupsize=None, out=None, accumulate=False, out_shape=None):
     """y fp16 [M, N] = x [M, K] @ W for M <= 16 (decode).  `out_shape` (same number of elements)
     lets the result be allocated with the caller's leading dimensions instead of being a view."""
@@ -386,6 +440,24 @@ def _scales_half(scales):
     return scales if scales.dtype == torch.float16 else scales.half()
 
 
+def vecquant4recons_v1(mat, res, scales, zeros):
+    """quant_cuda.vecquant4recons_v1(mat, res, scales, zeros) -> None; res[K,N] = W of a v1 layer
+    (quant_cuda.cpp:129-135)."""
+    if res.dtype == torch.float16 and res.is_contiguous():
+        dequant_v1(mat, scales, zeros, out=res)
+    else:
+        res.copy_(dequant_v1(mat, scales, zeros))
+
+
+def vecquant2recons_v2(mat, res, scales, zeros, g_idx):
+    """quant_cuda.vecquant2recons_v2(mat, res, scales, zeros, g_idx) -> None (quant_cuda.cpp:156-161)."""
+    gs = _infer_groupsize(mat.shape[0] * 16, scales.shape[0])
+    if res.dtype == torch.float16 and res.is_contiguous():
+        dequant2(mat, zeros, _scales_half(scales), g_idx, gs, out=res)
+    else:
+        res.copy_(dequant2(mat, zeros, _scales_half(scales), g_idx, gs))
+
+
 def vecquant4recons_v2(mat, res, scales, zeros, g_idx):
     """quant_cuda.vecquant4recons_v2(mat, res, scales, zeros, g_idx) -> None; res[K,N] = W.
     (quant_cuda.cpp:143-148).  fp16 `res` is written in place; other dtypes via one cast."""
@@ -427,12 +499,12 @@ def vecquant4matmul_old_faster(vec, mat, mul, scales, zeros, groupsize, vec_heig
 
 def _unsupported(name):
     def fn(*args, **kwargs):
-        raise NotImplementedError(f"{name}: only the 4-bit v2 (grouped, int32 qzeros) layout is built for gfx950")
+        raise NotImplementedError(f"{name}: not built for gfx950 (4-bit v2 runs fused; v1 and 2-bit v2 run through "
+                                  "vecquant4recons_v1 / vecquant2recons_v2 + a dense GEMM)")
     fn.__name__ = name
     return fn
 
 
 for _n in ("vecquant2matmul", "vecquant3matmul", "vecquant8matmul", "vecquant2matmul_faster", "vecquant3matmul_faster",
-           "vecquant4matmul_v1_faster", "vecquant4recons_v1", "vecquant2recons_v2", "vecquant4matmul_seq_v2",
-           "vecquant4matmul_g"):
+           "vecquant4matmul_v1_faster", "vecquant4matmul_seq_v2", "vecquant4matmul_g"):
     globals()[_n] = _unsupported(_n)

@@ -49,6 +49,18 @@ int q4_dequant_f16(const int32_t *qweight, const int32_t *qzeros, const void *sc
                    const int32_t *g_idx, int groupsize, void *out,
                    int K, int N, int G, void *stream);
 
+/* Dense dequantization of the older "v1" layout: one fp16 scale and one fp16 zero per column
+ * (scales, zeros: [N]),  W[k,n] = rn16( rn16(s[n]*q) - zero[n] ).
+ * Replaces quant_cuda.vecquant4recons_v1 (quant_cuda/quant_cuda.cpp:131-135, kernel quant_cuda_kernel.cu:1076-1097). */
+int q4_dequant_v1_f16(const int32_t *qweight, const void *scales, const void *zeros, void *out,
+                      int K, int N, void *stream);
+
+/* Dense dequantization of 2-bit v2 layers: qweight int32 [K/16, N] (sixteen codes per word along K),
+ * qzeros int32 [G, N/16], scales fp16 [G, N], W = rn16( rn16(s*q) - rn16(s*(z+1)) ).  K % 16 == 0.
+ * Replaces quant_cuda.vecquant2recons_v2 (quant_cuda/quant_cuda.cpp:150-161, kernel quant_cuda_kernel.cu:1185-1211). */
+int q4_dequant2_f16(const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                    const int32_t *g_idx, int groupsize, void *out, int K, int N, int G, void *stream);
+
 /* Row permutation of packed weights: out int32 [K/8, N] holds in row p the 4-bit codes of row perm[p]
  * of qweight (perm int32 [K], a permutation of 0..K-1, not checked).  No counterpart in the reference:
  * it is the one-time repack that lets an act-order layer (rows assigned to groups through g_idx,

@@ -20,6 +20,9 @@ Parity status of each function (what pins it is in tests/test_oracle_*.py):
   gemv_v2_fp32                              pinned  (same brute force; fp32 form)
   lora_forward / lora_backward              pinned  (finite differences in float64, and torch
                                                      autograd through dense nn.Linear in tests)
+  dequant_v1 / dequant2_v2                  pinned  (exact Fraction arithmetic with the independent
+                                                     round-to-nearest-even of tests/golden/make_fixtures.py,
+                                                     pure-Python index loops for the 2-bit packing)
   peft 0.6 LoraLayer internals              parity unpinned (peft is not importable here; only the
                                                      arithmetic in models.py:58-66 is restated)
 """
@@ -112,6 +115,58 @@ def dequant_v2(qweight, qzeros, scales, g_idx) -> np.ndarray:
     zero = s_rows * zp1                               # rn16(s*(z+1))
     prod = s_rows * q.astype(np.float16)              # rn16(s*q)
     return prod - zero                                # rn16(prod - zero)
+
+
+def dequant_v1(qweight, scales, zeros) -> np.ndarray:
+    """Dense fp16 W of a v1 layer as VecQuant4ReconsV1Kernel<Half> produces it
+    (quant_cuda_kernel.cu:1076-1097): scale, zero per column; result = scale * Half(q) - zero,
+    i.e. W = rn16( rn16(s*q) - zero ).  Parity pinned by exact-rational arithmetic in tests/test_oracle.py."""
+    s = np.asarray(scales).reshape(-1)
+    z = np.asarray(zeros).reshape(-1)
+    assert s.dtype == np.float16 and z.dtype == np.float16
+    q = unpack_qweight(qweight).astype(np.float16)
+    return (s[None, :] * q) - z[None, :]
+
+
+def pack_qweight2(codes: np.ndarray) -> np.ndarray:
+    """codes uint8 [K, N] in 0..3 -> int32 [K/16, N]: row k in bits 2*(k%16).. of word [k/16, n]
+    (index arithmetic of quant_cuda_kernel.cu:1206-1208)."""
+    K, N = codes.shape
+    c = codes.astype(np.uint32).reshape(K // 16, 16, N)
+    w = np.zeros((K // 16, N), dtype=np.uint32)
+    for e in range(16):
+        w |= c[:, e, :] << np.uint32(2 * e)
+    return w.view(np.int32)
+
+
+def pack_qzeros2(zcodes: np.ndarray) -> np.ndarray:
+    """zero codes uint8 [G, N] in 0..3 -> int32 [G, N/16]: column n in bits 2*(n%16).. of word [g, n/16]
+    (quant_cuda_kernel.cu:1201-1203)."""
+    G, N = zcodes.shape
+    c = zcodes.astype(np.uint32).reshape(G, N // 16, 16)
+    w = np.zeros((G, N // 16), dtype=np.uint32)
+    for e in range(16):
+        w |= c[:, :, e] << np.uint32(2 * e)
+    return w.view(np.int32)
+
+
+def dequant2_v2(qweight, qzeros, scales, g_idx) -> np.ndarray:
+    """Dense fp16 W of a 2-bit v2 layer as VecQuant2ReconsV2Kernel<Half> produces it
+    (quant_cuda_kernel.cu:1185-1211): the 4-bit formula with 2-bit fields,
+    W = rn16( rn16(s*q) - rn16(s*(z+1)) )."""
+    scales = np.asarray(scales)
+    assert scales.dtype == np.float16
+    wq = np.asarray(qweight).view(np.uint32)
+    zq = np.asarray(qzeros).view(np.uint32)
+    K, N = wq.shape[0] * 16, wq.shape[1]
+    k = np.arange(K)
+    q = ((wq[k // 16, :] >> ((k % 16) * 2).astype(np.uint32)[:, None]) & 3).astype(np.float16)      # [K, N]
+    n = np.arange(N)
+    z = ((zq[:, n // 16] >> ((n % 16) * 2).astype(np.uint32)[None, :]) & 3).astype(np.int32)         # [G, N]
+    g = np.asarray(g_idx).astype(np.int64)
+    s_rows = scales[g]
+    zero = s_rows * (z + 1).astype(np.float16)[g]
+    return s_rows * q - zero
 
 
 def dequant_v2_single_rounding(qweight, qzeros, scales, g_idx) -> np.ndarray:

@@ -60,6 +60,11 @@ def test_error_codes_and_validation_need_no_gpu():
     assert L.q4_gemm_workspace_bytes(1, 2048, 4096, 4096) == 0            # enough tiles: no split
     assert L.q4_gemm_workspace_bytes(1, 64, 4096, 4096) == 8 * 64 * 4096 * 4    # 32 tiles -> 8 splits of fp32 partials
     assert L.q4_gemm_workspace_bytes(0, 64, 4096, 11008) == 8 * 64 * 4096 * 4
+    # older layouts (dense dequantization only)
+    assert L.q4_dequant_v1_f16(fake, fake, None, fake, 256, 128, None) == -1
+    assert L.q4_dequant_v1_f16(fake, fake, fake, fake, 250, 128, None) == -2
+    assert L.q4_dequant2_f16(fake, fake, fake, None, 128, fake, 264, 128, 3, None) == -2     # K % 16
+    assert L.q4_dequant2_f16(fake, fake, fake, None, 128, odd, 256, 128, 2, None) == -5
     # adapter helpers
     assert L.q4_lora_down_f16(fake, None, 4096, 1, 1, fake, 64, 4096, 8, None) == -1
     assert L.q4_lora_down_f16(fake, fake, 4096, 1, 1, fake, 64, 4100, 8, None) == -2        # C % 32
@@ -131,9 +136,9 @@ def test_unsupported_bitwidth_and_layouts_raise_like_the_reference():
     m = Autograd4bitQuantLinear(256, 128, groupsize=128, bits=3)
     with pytest.raises(ValueError, match="Unsupported bitwidth"):
         m(torch.zeros(1, 256))
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(ValueError, match="CUDA"):      # fp zeros = v1 layout: dispatched, then rejected as CPU tensors
         mm4b.matmul4bit(torch.zeros(1, 256), torch.zeros(32, 128, dtype=torch.int32), torch.zeros(128, 1),
-                        torch.zeros(128, 1))          # fp zeros = v1 layout
+                        torch.zeros(128, 1))
     with pytest.raises(AssertionError):                # K mismatch, matmul_utils_4bit.py:71
         mm4b._matmul4bit_v2(torch.zeros(1, 128), torch.zeros(32, 128, dtype=torch.int32), torch.zeros(2, 128),
                             torch.zeros(2, 16, dtype=torch.int32), torch.zeros(256, dtype=torch.int32))
@@ -160,7 +165,9 @@ def test_quant_cuda_mirror_exports_the_pybind_names():
                  "vecquant4matmul_seq_v2", "vecquant4matmul_g"):
         assert callable(getattr(quant_hip, name)), name
     with pytest.raises(NotImplementedError):
-        quant_hip.vecquant2recons_v2()
+        quant_hip.vecquant2matmul()
+    assert list(inspect.signature(quant_hip.vecquant4recons_v1).parameters) == ["mat", "res", "scales", "zeros"]
+    assert list(inspect.signature(quant_hip.vecquant2recons_v2).parameters) == ["mat", "res", "scales", "zeros", "g_idx"]
     assert list(inspect.signature(quant_hip.vecquant4recons_v2).parameters) == ["mat", "res", "scales", "zeros", "g_idx"]
     assert list(inspect.signature(quant_hip.vecquant4matmul_old_faster).parameters) == \
         ["vec", "mat", "mul", "scales", "zeros", "groupsize", "vec_height"]

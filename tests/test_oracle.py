@@ -243,3 +243,61 @@ def test_synthetic_generators_follow_the_config_distributions():
     assert (counts == 128).all() and not np.array_equal(lay["g_idx"], np.arange(1024) // 128)
     A, B = o.make_lora(4096, 4096, 8, seed=1)
     assert A.shape == (8, 4096) and B.shape == (4096, 8) and np.abs(A).max() <= 1 / 64 and 0.015 < B.std() < 0.025
+
+
+# --------------------------------------------------------------------------- older layouts (v1, 2-bit)
+def _load_generator():
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(os.path.dirname(__file__), "golden", "make_fixtures.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def test_dequant_v1_against_exact_rational_arithmetic(oracle):
+    """W = rn16(rn16(s*q) - zero) per element (quant_cuda_kernel.cu:1094), checked with Fractions and the
+    generator's own round-to-nearest-even."""
+    gen = _load_generator()
+    rng = np.random.default_rng(5)
+    K, N = 16, 64
+    codes = rng.integers(0, 16, size=(K, N), dtype=np.uint8)
+    scales = rng.uniform(0.004, 0.03, size=N).astype(np.float16)
+    zeros = (scales.astype(np.float32) * rng.integers(1, 17, size=N)).astype(np.float16)
+    W = oracle.dequant_v1(oracle.pack_qweight(codes), scales, zeros)
+    sb, zb, wb = scales.view(np.uint16), zeros.view(np.uint16), W.view(np.uint16)
+    for k in range(K):
+        for n in range(N):
+            s = gen.half_bits_to_fraction(int(sb[n]))
+            prod = gen.half_bits_to_fraction(gen.rn16(s * int(codes[k, n])))
+            expect = gen.rn16(prod - gen.half_bits_to_fraction(int(zb[n])))
+            assert int(wb[k, n]) == expect or (expect & 0x7FFF) == 0 and (int(wb[k, n]) & 0x7FFF) == 0
+
+
+def test_dequant2_against_loops_and_exact_arithmetic(oracle):
+    """2-bit packing by pure-Python index arithmetic of the kernel (quant_cuda_kernel.cu:1196-1210) and the
+    three-rounding value by Fractions."""
+    gen = _load_generator()
+    rng = np.random.default_rng(6)
+    K, N, gs = 64, 64, 32
+    G = K // gs
+    codes = rng.integers(0, 4, size=(K, N), dtype=np.uint8)
+    zc = rng.integers(0, 4, size=(G, N), dtype=np.uint8)
+    scales = rng.uniform(0.01, 0.2, size=(G, N)).astype(np.float16)
+    g_idx = rng.permutation(K).astype(np.int32) % G                     # scattered groups
+    qw, qz = oracle.pack_qweight2(codes), oracle.pack_qzeros2(zc)
+    assert qw.shape == (K // 16, N) and qz.shape == (G, N // 16)
+    W = oracle.dequant2_v2(qw, qz, scales, g_idx)
+    sb, wb = scales.view(np.uint16), W.view(np.uint16)
+    for k in range(0, K, 3):
+        for n in range(0, N, 5):
+            word = gen.as_unsigned(int(qw[k // 16, n]))
+            q = (word >> (k % 16 * 2)) & 0x3
+            assert q == codes[k, n]
+            g = int(g_idx[k])
+            z = ((gen.as_unsigned(int(qz[g, n // 16])) >> ((n % 16) * 2)) & 0x3) + 1
+            assert z == zc[g, n] + 1
+            s = gen.half_bits_to_fraction(int(sb[g, n]))
+            zero = gen.half_bits_to_fraction(gen.rn16(s * z))
+            prod = gen.half_bits_to_fraction(gen.rn16(s * q))
+            expect = gen.rn16(prod - zero)
+            assert int(wb[k, n]) == expect or (expect & 0x7FFF) == 0 and (int(wb[k, n]) & 0x7FFF) == 0
