@@ -596,6 +596,19 @@ static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
 
 }  // namespace q4
 
+extern "C" int q4_launch_splitk_reduce(const float* part, void* out, long total, int splits, hipStream_t stream) {
+    hipLaunchKernelGGL(q4::gemm_splitk_reduce_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream,
+                       part, reinterpret_cast<q4::half_t*>(out), total, splits);
+    return hipGetLastError() == hipSuccess ? 0 : -4;
+}
+
+extern "C" {
+int q4_skinny_applicable(int M, int K, int N, int groupsize, int has_gidx);
+size_t q4_skinny_workspace(int M, int K, int N);
+int q4_launch_skinny(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales, int groupsize,
+                     const void* bias, void* y, int M, int K, int N, void* workspace, hipStream_t stream);
+}
+
 extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros,
                               const void* scales, const int32_t* g_idx, int groupsize, const void* bias,
                               const void* la, const void* lb, int lb_sr, int lb_sc, int lb_is_f32, float lb_scale, int R,
@@ -620,6 +633,10 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     a.phase_step = env_phase < 0 ? 0 : env_phase;
     const int nout = fwd ? N : K;
     const bool gidx = g_idx != nullptr;
+    // 17..32 rows, forward, no adapter: the weight-streaming kernel (one pass over the packed weights)
+    if (fwd && a.R == 0 && q4_skinny_applicable(M, K, N, groupsize, gidx) && workspace &&
+        workspace_bytes >= q4_skinny_workspace(M, K, N))
+        return q4_launch_skinny(act, qweight, qzeros, scales, groupsize, bias, out, M, K, N, workspace, stream);
     // tile configuration: 256-row tiles once they still give every CU a workgroup; split-K for few tiles
     const GemmPlan p = plan_gemm(M, fwd ? K : N, nout, workspace ? workspace_bytes : 0);
     a.part = reinterpret_cast<float*>(workspace);
@@ -634,5 +651,10 @@ extern "C" size_t q4_gemm_plan_workspace(int fwd, int M, int K, int N) {
     using namespace q4;
     const int nout = fwd ? N : K;
     const GemmPlan p = plan_gemm(M, fwd ? K : N, nout, ~(size_t)0);
-    return p.splits > 1 ? (size_t)p.splits * (size_t)M * (size_t)nout * sizeof(float) : 0;
+    size_t need = p.splits > 1 ? (size_t)p.splits * (size_t)M * (size_t)nout * sizeof(float) : 0;
+    if (fwd && M > 16 && M <= 32) {               // the skinny kernel's partial rows (it may or may not apply)
+        const size_t sk = q4_skinny_workspace(M, K, N);
+        if (sk > need) need = sk;
+    }
+    return need;
 }

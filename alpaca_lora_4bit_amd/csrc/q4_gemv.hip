@@ -192,6 +192,119 @@ __global__ __launch_bounds__(NSTEP >= 16 ? 512 : 1024) void gemv_seq_kernel(Gemv
     gemv_finish(a, yacc, n0, wave, nwaves, kk, c);
 }
 
+// ------------------------------------------------------------------ 17 <= M <= 32 (sequential groups)
+// The same streaming scheme for two 16-row blocks of activations (every strip re-reads the activations of
+// its chunk, M*K*2 bytes per strip in total, so beyond 32 rows the tiled GEMM with split-K is faster): the packed weights of a chunk
+// are loaded once and multiplied with every block (the B operands are rebuilt from the words, five ALU
+// ops each).  With M rows per strip the cross-workgroup sum would need M*64 atomics per workgroup, so the
+// workgroups of a strip leave fp32 partial rows in a scratch buffer [gridDim.y][M][N] instead and a
+// second kernel adds them in order (bit-reproducible); the bias rides with split 0.
+// Chunks of 128 rows inside one quantization group only (NSTEP = 4, groupsize % 128 == 0).
+struct SkinnyArgs {
+    const half_t* x;
+    const uint32_t* qweight;
+    const uint32_t* qzeros;
+    const half_t* scales;
+    const half_t* bias;       // [N] or null
+    int groupsize;
+    half_t* y;                // written directly when gridDim.y == 1
+    float* part;              // [gridDim.y][M][N]
+    int M, K, N;
+};
+
+template <int RB>
+__global__ __launch_bounds__(512) void skinny_seq_kernel(SkinnyArgs a) {
+    constexpr int NSTEP = 4;
+    __shared__ float red[8 * 16 * 64];             // [wavefront][row of the block][column of the strip]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nwaves = blockDim.x >> 6;
+    const int kk = lane >> 4, c = lane & 15;
+    const int n0 = blockIdx.x * kColsPerWave;
+    const int k0 = (blockIdx.y * nwaves + wave) * (32 * NSTEP);
+    const bool active = k0 < a.K;                  // wave-uniform
+    const int col = n0 + 4 * c;
+
+    uint2_t sv = {0u, 0u};
+    uint32_t zv = 0;
+    uint4_t wv[NSTEP], xv[RB][NSTEP];
+    if (active) {
+        const int g = k0 / a.groupsize;
+        sv = *reinterpret_cast<const uint2_t*>(a.scales + (size_t)g * a.N + col);
+        zv = a.qzeros[(size_t)g * (a.N >> 3) + (col >> 3)];
+        const uint32_t* wp = a.qweight + (size_t)((k0 >> 3) + kk) * a.N + col;
+#pragma unroll
+        for (int t = 0; t < NSTEP; ++t) wv[t] = *reinterpret_cast<const uint4_t*>(wp + (size_t)(4 * t) * a.N);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            // rows >= M hold a copy of row M-1: they only reach rows of the product that are never stored
+            const half_t* xp = a.x + (size_t)min(16 * rb + c, a.M - 1) * a.K + k0 + 8 * kk;
+#pragma unroll
+            for (int t = 0; t < NSTEP; ++t) xv[rb][t] = *reinterpret_cast<const uint4_t*>(xp + 32 * t);
+        }
+        __builtin_amdgcn_sched_barrier(0);        // one burst of loads, nothing sunk below the arithmetic
+    }
+    const half8_t offs = make_half8(0x64006400u, 0x54005400u, 0x64006400u, 0x54005400u);
+    const half8_t ones = make_half8(0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u);
+    const uint32_t zw = zv >> ((c & 1) * 16);
+    const half2_t s01 = as_half2(sv.x), s23 = as_half2(sv.y);
+    const float sf[4] = {(float)s01[0], (float)s01[1], (float)s23[0], (float)s23[1]};
+    const int S = gridDim.y;
+
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        float4_t yacc[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) yacc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+        if (active) {
+            float4_t acc[4], acco = {0.f, 0.f, 0.f, 0.f}, accx = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int t = 0; t < NSTEP; ++t) {
+                const half8_t av = make_half8(__builtin_amdgcn_perm(xv[rb][t].z, xv[rb][t].x, 0x05040100u),
+                                              __builtin_amdgcn_perm(xv[rb][t].z, xv[rb][t].x, 0x07060302u),
+                                              __builtin_amdgcn_perm(xv[rb][t].w, xv[rb][t].y, 0x05040100u),
+                                              __builtin_amdgcn_perm(xv[rb][t].w, xv[rb][t].y, 0x07060302u));
+                const uint32_t w[4] = {wv[t].x, wv[t].y, wv[t].z, wv[t].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t hi = w[j] >> 8;
+                    const half8_t bv = make_half8((w[j] & 0x000F000Fu) | 0x64006400u, (w[j] & 0x00F000F0u) | 0x54005400u,
+                                                  (hi & 0x000F000Fu) | 0x64006400u, (hi & 0x00F000F0u) | 0x54005400u);
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, acc[j], 0, 0, 0);
+                }
+                acco = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, offs, acco, 0, 0, 0);
+                accx = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, ones, accx, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float zf = (float)(((zw >> (4 * j)) & 0xFu) + 1u);
+                    yacc[j][r] = sf[j] * ((acc[j][r] - acco[r]) - zf * accx[r]);
+                }
+        }
+        // sum over the wavefronts of the workgroup; row 4*kk + r of the block, columns 4c .. 4c+3
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            *reinterpret_cast<float4_t*>(red + ((wave * 16 + 4 * kk + r) << 6) + 4 * c) =
+                float4_t{yacc[0][r], yacc[1][r], yacc[2][r], yacc[3][r]};
+        __syncthreads();
+        for (int e = threadIdx.x; e < 16 * 64; e += blockDim.x) {
+            const int m = 16 * rb + (e >> 6), cc = n0 + (e & 63);
+            if (m < a.M) {
+                float v = 0.f;
+                for (int w = 0; w < nwaves; ++w) v += red[(w << 10) + e];
+                if (a.bias && blockIdx.y == 0) v += (float)a.bias[cc];
+                if (S == 1) a.y[(size_t)m * a.N + cc] = (half_t)v;
+                else a.part[((size_t)blockIdx.y * a.M + m) * a.N + cc] = v;
+            }
+        }
+        __syncthreads();                           // red is reused by the next row block
+    }
+}
+
 // ------------------------------------------------------------------ act-order (per-row groups)
 template <int NSTEP>
 __global__ __launch_bounds__(512) void gemv_gidx_kernel(GemvArgs a) {
@@ -363,4 +476,45 @@ extern "C" int q4_launch_gemv(const void* x, const int32_t* qweight, const int32
         }
     }
     return hipGetLastError() == hipSuccess ? 0 : -4;
+}
+
+
+extern "C" int q4_launch_splitk_reduce(const float* part, void* out, long total, int splits, hipStream_t stream);
+
+// Shapes the skinny kernel takes: 17..32 rows, sequential groups that are multiples of 128 rows.
+extern "C" int q4_skinny_applicable(int M, int K, int N, int groupsize, int has_gidx) {
+    return M > 16 && M <= 32 && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 64 == 0;
+}
+
+static int skinny_splits(int K) {
+    const int chunks = K / 128;
+    return (chunks + 7) / 8;                      // 8 wavefronts per workgroup, one chunk each
+}
+
+extern "C" size_t q4_skinny_workspace(int M, int K, int N) {
+    const int S = skinny_splits(K);
+    return S > 1 ? (size_t)S * (size_t)M * (size_t)N * sizeof(float) : 0;
+}
+
+extern "C" int q4_launch_skinny(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                                int groupsize, const void* bias, void* y, int M, int K, int N,
+                                void* workspace, hipStream_t stream) {
+    using namespace q4;
+    SkinnyArgs a;
+    a.x = reinterpret_cast<const half_t*>(x);
+    a.qweight = reinterpret_cast<const uint32_t*>(qweight);
+    a.qzeros = reinterpret_cast<const uint32_t*>(qzeros);
+    a.scales = reinterpret_cast<const half_t*>(scales);
+    a.bias = reinterpret_cast<const half_t*>(bias);
+    a.groupsize = groupsize;
+    a.y = reinterpret_cast<half_t*>(y);
+    a.part = reinterpret_cast<float*>(workspace);
+    a.M = M; a.K = K; a.N = N;
+    const int S = skinny_splits(K);
+    const int chunks = K / 128;
+    const dim3 grid(N / kColsPerWave, S), block(64 * (chunks < 8 ? chunks : 8));
+    hipLaunchKernelGGL(skinny_seq_kernel<2>, grid, block, 0, stream, a);
+    if (hipGetLastError() != hipSuccess) return -4;
+    if (S > 1) return q4_launch_splitk_reduce(a.part, y, (long)M * N, S, stream);
+    return 0;
 }

@@ -130,3 +130,24 @@ def test_split_k_is_reproducible_and_matches_unsplit(oracle):
     ref = ref + bias.float().cpu().numpy()
     err = np.abs(y1.float().cpu().numpy() - ref).max()
     assert err <= 1e-2 * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("M", [17, 32, 33, 48, 64])
+@pytest.mark.parametrize("K,N,gs,act", [(4096, 1024, 128, False), (1408, 256, 128, False), (512, 384, 128, True),
+                                        (11008, 256, 128, False)])
+def test_gemm_forward_17_to_64_rows(oracle, M, K, N, gs, act):
+    """17..32 rows take the weight-streaming kernel (both row blocks share one pass over the packed weights;
+    partial rows of the K splits are added by a second kernel), 33..64 the tiled kernel with split-K; with bias."""
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    layer = oracle.make_layer(K, N, gs, act_order=act, seed=K + N + M)
+    t = to_cuda_layer(layer)
+    x = oracle.make_activations(M, K, seed=M + 11)
+    bias = (np.random.default_rng(M).standard_normal(N) * 0.5).astype(np.float16)
+    ref = oracle.matmul_recons(x, layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"]) + bias.astype(np.float32)
+    y = quant_hip.gemm_fwd(torch.from_numpy(x).cuda(), t["qweight"], t["qzeros"], t["scales"], t["g_idx"], gs,
+                           bias=torch.from_numpy(bias).cuda())
+    y2 = quant_hip.gemm_fwd(torch.from_numpy(x).cuda(), t["qweight"], t["qzeros"], t["scales"], t["g_idx"], gs,
+                            bias=torch.from_numpy(bias).cuda())
+    assert y.shape == (M, N) and torch.equal(y, y2)
+    assert np.abs(y.float().cpu().numpy() - ref).max() <= 1e-2 * np.abs(ref).max()
