@@ -18,8 +18,8 @@ import sys
 
 __version__ = "0.1.0"
 
-_ALIASED = ("autograd_4bit", "matmul_utils_4bit", "quant_hip", "models", "amp_wrapper", "monkeypatch",
-            "monkeypatch.peft_tuners_lora_monkey_patch")
+_ALIASED = ("autograd_4bit", "matmul_utils_4bit", "quant_hip", "models", "amp_wrapper", "model_attn_mlp_patch",
+            "loaders", "monkeypatch", "monkeypatch.peft_tuners_lora_monkey_patch")
 
 
 def install_as_alpaca_lora_4bit(name: str = "alpaca_lora_4bit") -> None:
