@@ -652,7 +652,7 @@ extern "C" size_t q4_gemm_plan_workspace(int fwd, int M, int K, int N) {
     const int nout = fwd ? N : K;
     const GemmPlan p = plan_gemm(M, fwd ? K : N, nout, ~(size_t)0);
     size_t need = p.splits > 1 ? (size_t)p.splits * (size_t)M * (size_t)nout * sizeof(float) : 0;
-    if (fwd && M > 16 && M <= 32) {               // the skinny kernel's partial rows (it may or may not apply)
+    if (fwd && M > 16 && M <= 64) {               // the skinny kernel's partial rows (it may or may not apply)
         const size_t sk = q4_skinny_workspace(M, K, N);
         if (sk > need) need = sk;
     }

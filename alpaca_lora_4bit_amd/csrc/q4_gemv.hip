@@ -192,14 +192,20 @@ __global__ __launch_bounds__(NSTEP >= 16 ? 512 : 1024) void gemv_seq_kernel(Gemv
     gemv_finish(a, yacc, n0, wave, nwaves, kk, c);
 }
 
-// ------------------------------------------------------------------ 17 <= M <= 32 (sequential groups)
-// The same streaming scheme for two 16-row blocks of activations (every strip re-reads the activations of
-// its chunk, M*K*2 bytes per strip in total, so beyond 32 rows the tiled GEMM with split-K is faster): the packed weights of a chunk
-// are loaded once and multiplied with every block (the B operands are rebuilt from the words, five ALU
-// ops each).  With M rows per strip the cross-workgroup sum would need M*64 atomics per workgroup, so the
-// workgroups of a strip leave fp32 partial rows in a scratch buffer [gridDim.y][M][N] instead and a
-// second kernel adds them in order (bit-reproducible); the bias rides with split 0.
-// Chunks of 128 rows inside one quantization group only (NSTEP = 4, groupsize % 128 == 0).
+// ------------------------------------------------------------------ 17 <= M <= 64 (sequential groups)
+// The same streaming scheme for RB blocks of 16 activation rows.  A wavefront owns one chunk of 128
+// reduction rows: it loads that chunk of every activation row once, keeps it as MFMA A operands in
+// registers (together with the two offset products, which do not depend on the weights) and walks over
+// `strips_per_wg` neighbouring 64-column strips, prefetching the packed weights of the next strip while it
+// multiplies the current one - so the activations are read once per strips_per_wg strips, not once per
+// strip.  The B operands are rebuilt from the words (five ALU ops each) once per strip and used for every
+// row block.  The eight wavefronts of a workgroup (eight chunks) are summed through LDS; with M rows per
+// strip the cross-workgroup sum would need M*64 atomics per workgroup, so the workgroups of a strip
+// leave fp32 partial rows in a scratch buffer [gridDim.y][M][N] instead and a second kernel adds them in
+// order (bit-reproducible); the bias rides with split 0.
+// Chunks of 128 rows inside one quantization group only (groupsize % 128 == 0).  No branches around the
+// loads: a wavefront past the end of K, and the prefetch after the last strip, fetch from an offset
+// beyond every buffer, which returns zeros without traffic.
 struct SkinnyArgs {
     const half_t* x;
     const uint32_t* qweight;
@@ -210,98 +216,179 @@ struct SkinnyArgs {
     half_t* y;                // written directly when gridDim.y == 1
     float* part;              // [gridDim.y][M][N]
     int M, K, N;
+    int strips_per_wg;
 };
 
 template <int RB>
-__global__ __launch_bounds__(512) void skinny_seq_kernel(SkinnyArgs a) {
-    constexpr int NSTEP = 4;
-    __shared__ float red[8 * 16 * 64];             // [wavefront][row of the block][column of the strip]
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(RB <= 2 ? 4 : 2)))
+void skinny_seq_kernel(SkinnyArgs a) {
+    constexpr int NSTEP = 4, NW = 8;
+    constexpr int kFar = 0x70000000;
+    // [row block][wavefront][row][column of the strip]; before the first strip, the activation tiles
+    __shared__ __attribute__((aligned(16))) float red[RB][NW][16 * 64];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int nwaves = blockDim.x >> 6;
     const int kk = lane >> 4, c = lane & 15;
-    const int n0 = blockIdx.x * kColsPerWave;
-    const int k0 = (blockIdx.y * nwaves + wave) * (32 * NSTEP);
-    const bool active = k0 < a.K;                  // wave-uniform
-    const int col = n0 + 4 * c;
-
-    uint2_t sv = {0u, 0u};
-    uint32_t zv = 0;
-    uint4_t wv[NSTEP], xv[RB][NSTEP];
-    if (active) {
-        const int g = k0 / a.groupsize;
-        sv = *reinterpret_cast<const uint2_t*>(a.scales + (size_t)g * a.N + col);
-        zv = a.qzeros[(size_t)g * (a.N >> 3) + (col >> 3)];
-        const uint32_t* wp = a.qweight + (size_t)((k0 >> 3) + kk) * a.N + col;
-#pragma unroll
-        for (int t = 0; t < NSTEP; ++t) wv[t] = *reinterpret_cast<const uint4_t*>(wp + (size_t)(4 * t) * a.N);
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-            // rows >= M hold a copy of row M-1: they only reach rows of the product that are never stored
-            const half_t* xp = a.x + (size_t)min(16 * rb + c, a.M - 1) * a.K + k0 + 8 * kk;
-#pragma unroll
-            for (int t = 0; t < NSTEP; ++t) xv[rb][t] = *reinterpret_cast<const uint4_t*>(xp + 32 * t);
-        }
-        __builtin_amdgcn_sched_barrier(0);        // one burst of loads, nothing sunk below the arithmetic
-    }
-    const half8_t offs = make_half8(0x64006400u, 0x54005400u, 0x64006400u, 0x54005400u);
-    const half8_t ones = make_half8(0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u);
-    const uint32_t zw = zv >> ((c & 1) * 16);
-    const half2_t s01 = as_half2(sv.x), s23 = as_half2(sv.y);
-    const float sf[4] = {(float)s01[0], (float)s01[1], (float)s23[0], (float)s23[1]};
+    const int strip0 = blockIdx.x * a.strips_per_wg;
+    const int nl = min(a.strips_per_wg, (a.N >> 6) - strip0);
+    const int k0 = (blockIdx.y * NW + wave) * (32 * NSTEP);
+    const int dead = k0 < a.K ? 0 : kFar;          // wave-uniform
+    const int G = a.K / a.groupsize, g = dead ? 0 : k0 / a.groupsize;
     const int S = gridDim.y;
 
+    const rsrc_t rw = make_rsrc(a.qweight, (unsigned)((size_t)(a.K >> 3) * a.N * 4));
+    const rsrc_t rs = make_rsrc(a.scales, (unsigned)((size_t)G * a.N * 2));
+    const rsrc_t rz = make_rsrc(a.qzeros, (unsigned)((size_t)G * (a.N >> 3) * 4));
+    const rsrc_t rx = make_rsrc(a.x, (unsigned)((size_t)a.M * a.K * 2));
+    // the bias rides with split 0; an empty buffer reads as zeros
+    const rsrc_t rb_bias = make_rsrc(a.bias, a.bias && blockIdx.y == 0 ? (unsigned)a.N * 2 : 0u);
+    const int vw = dead ? 0 : (((k0 >> 3) + kk) * a.N + 4 * c) * 4;
+    const int vs = (g * a.N + 4 * c) * 2;
+    const int vz = (g * (a.N >> 3) + (c >> 1)) * 4;
+    const int wstep = 16 * a.N;                    // bytes between the words of two steps (4 packed rows)
+
+    // weights of the first strip, then the activations of the chunk
+    uint4_t wv[NSTEP];
+    uint2_t sv = buf_load64(rs, vs, dead + strip0 * 128);
+    uint32_t zv = buf_load32(rz, vz, dead + strip0 * 32);
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-        float4_t yacc[4];
+    for (int t = 0; t < NSTEP; ++t) wv[t] = buf_load128(rw, vw, dead + strip0 * 256 + t * wstep);
+    // Activations: a lane of the MFMA A operand wants 16 bytes of row c, so a direct load would touch 16
+    // rows (16 cache lines) per quarter wavefront and the vector cache would spend its time on tag lookups.
+    // Load row-contiguous instead (a quarter wavefront = 256 contiguous bytes of one row) and turn the tile
+    // through this wavefront's own 4 KB of LDS per row block: 16 rows x 16 units of 16 bytes, unit q of
+    // row r stored at q ^ r, which keeps both the row-wise writes and the column-wise reads conflict-free.
+    half8_t av[RB][NSTEP];
+    {
+        uint4_t xv[RB][NSTEP];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) yacc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
-        if (active) {
-            float4_t acc[4], acco = {0.f, 0.f, 0.f, 0.f}, accx = {0.f, 0.f, 0.f, 0.f};
+        for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+            for (int i = 0; i < NSTEP; ++i) {
+                // rows >= M hold a copy of row M-1: they only reach rows of the product that are never stored
+                const int vx = (min(16 * rb + 4 * i + kk, a.M - 1) * a.K + 8 * c) * 2;
+                xv[rb][i] = buf_load128(rx, vx, dead + k0 * 2);
+            }
+        __builtin_amdgcn_sched_barrier(0);        // one burst of loads, nothing sunk below the arithmetic
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            uint4_t* stage = reinterpret_cast<uint4_t*>(&red[rb][wave][0]);
+#pragma unroll
+            for (int i = 0; i < NSTEP; ++i) stage[(4 * i + kk) * 16 + (c ^ (4 * i + kk))] = xv[rb][i];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // A operands in the order the nibble split below produces: (e0,e4)(e1,e5)(e2,e6)(e3,e7)
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const uint4_t* stage = reinterpret_cast<const uint4_t*>(&red[rb][wave][0]);
 #pragma unroll
             for (int t = 0; t < NSTEP; ++t) {
-                const half8_t av = make_half8(__builtin_amdgcn_perm(xv[rb][t].z, xv[rb][t].x, 0x05040100u),
-                                              __builtin_amdgcn_perm(xv[rb][t].z, xv[rb][t].x, 0x07060302u),
-                                              __builtin_amdgcn_perm(xv[rb][t].w, xv[rb][t].y, 0x05040100u),
-                                              __builtin_amdgcn_perm(xv[rb][t].w, xv[rb][t].y, 0x07060302u));
-                const uint32_t w[4] = {wv[t].x, wv[t].y, wv[t].z, wv[t].w};
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint32_t hi = w[j] >> 8;
-                    const half8_t bv = make_half8((w[j] & 0x000F000Fu) | 0x64006400u, (w[j] & 0x00F000F0u) | 0x54005400u,
-                                                  (hi & 0x000F000Fu) | 0x64006400u, (hi & 0x00F000F0u) | 0x54005400u);
-                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, acc[j], 0, 0, 0);
-                }
-                acco = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, offs, acco, 0, 0, 0);
-                accx = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, ones, accx, 0, 0, 0);
+                const uint4_t u = stage[c * 16 + ((4 * t + kk) ^ c)];
+                av[rb][t] = make_half8(__builtin_amdgcn_perm(u.z, u.x, 0x05040100u), __builtin_amdgcn_perm(u.z, u.x, 0x07060302u),
+                                       __builtin_amdgcn_perm(u.w, u.y, 0x05040100u), __builtin_amdgcn_perm(u.w, u.y, 0x07060302u));
             }
+        }
+    }
+    // sum x*offset and sum x of the chunk: the same for every strip
+    const half8_t offs = make_half8(0x64006400u, 0x54005400u, 0x64006400u, 0x54005400u);
+    const half8_t ones = make_half8(0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u);
+    float4_t acco[RB], accx[RB];
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
+    for (int rb = 0; rb < RB; ++rb) {
+        acco[rb] = float4_t{0.f, 0.f, 0.f, 0.f};
+        accx[rb] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < NSTEP; ++t) {
+            acco[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[rb][t], offs, acco[rb], 0, 0, 0);
+            accx[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[rb][t], ones, accx[rb], 0, 0, 0);
+        }
+    }
+
+    for (int l = 0; l < nl; ++l) {
+        const int n0 = (strip0 + l) << 6;
+        const int next = (dead || l + 1 >= nl) ? kFar : 0;    // uniform
+        // bias of the two columns this thread finishes, ahead of the prefetch so that waiting for it
+        // leaves the prefetch in flight
+        const uint32_t bias2 = buf_load32(rb_bias, (2 * (int)threadIdx.x & 63) * 2, n0 * 2);
+        uint4_t wn[NSTEP];
+        const uint2_t sn = buf_load64(rs, vs, next + (strip0 + l + 1) * 128);
+        const uint32_t zn = buf_load32(rz, vz, next + (strip0 + l + 1) * 32);
+#pragma unroll
+        for (int t = 0; t < NSTEP; ++t) wn[t] = buf_load128(rw, vw, next + (strip0 + l + 1) * 256 + t * wstep);
+        __builtin_amdgcn_sched_barrier(0);
+
+        float4_t acc[RB][4];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[rb][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < NSTEP; ++t) {
+            const uint32_t w[4] = {wv[t].x, wv[t].y, wv[t].z, wv[t].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                // a code in mantissa bits 0..3 of fp16 1024.0 reads 1024 + q, in bits 4..7 of fp16 64.0 it reads 64 + q
+                const uint32_t hi = w[j] >> 8;
+                const half8_t bv = make_half8((w[j] & 0x000F000Fu) | 0x64006400u, (w[j] & 0x00F000F0u) | 0x54005400u,
+                                              (hi & 0x000F000Fu) | 0x64006400u, (hi & 0x00F000F0u) | 0x54005400u);
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb)
+                    acc[rb][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[rb][t], bv, acc[rb][j], 0, 0, 0);
+            }
+        }
+        const uint32_t zw = zv >> ((c & 1) * 16);
+        const half2_t s01 = as_half2(sv.x), s23 = as_half2(sv.y);
+        const float sf[4] = {(float)s01[0], (float)s01[1], (float)s23[0], (float)s23[1]};
+        // y = s * ((sum x*(off+q) - sum x*off) - (z+1) * sum x); row 4*kk + r of the block, columns 4c .. 4c+3
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float4_t v;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const float zf = (float)(((zw >> (4 * j)) & 0xFu) + 1u);
-                    yacc[j][r] = sf[j] * ((acc[j][r] - acco[r]) - zf * accx[r]);
+                    v[j] = sf[j] * ((acc[rb][j][r] - acco[rb][r]) - zf * accx[rb][r]);
                 }
-        }
-        // sum over the wavefronts of the workgroup; row 4*kk + r of the block, columns 4c .. 4c+3
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-            *reinterpret_cast<float4_t*>(red + ((wave * 16 + 4 * kk + r) << 6) + 4 * c) =
-                float4_t{yacc[0][r], yacc[1][r], yacc[2][r], yacc[3][r]};
+                *reinterpret_cast<float4_t*>(&red[rb][wave][((4 * kk + r) << 6) + 4 * c]) = v;
+            }
         __syncthreads();
-        for (int e = threadIdx.x; e < 16 * 64; e += blockDim.x) {
-            const int m = 16 * rb + (e >> 6), cc = n0 + (e & 63);
-            if (m < a.M) {
-                float v = 0.f;
-                for (int w = 0; w < nwaves; ++w) v += red[(w << 10) + e];
-                if (a.bias && blockIdx.y == 0) v += (float)a.bias[cc];
-                if (S == 1) a.y[(size_t)m * a.N + cc] = (half_t)v;
-                else a.part[((size_t)blockIdx.y * a.M + m) * a.N + cc] = v;
+        // sum over the wavefronts: thread t finishes row t/32 of every block, columns 2*(t%32) and the next
+        {
+            const int e = 2 * threadIdx.x;
+            const int row = e >> 6, cc = n0 + (e & 63);
+            const half2_t b2 = as_half2(bias2);
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) {
+                    const float* rp = &red[rb][w][e];
+                    v0 += rp[0];
+                    v1 += rp[1];
+                }
+                const int m = 16 * rb + row;
+                if (m < a.M) {
+                    v0 += (float)b2[0];
+                    v1 += (float)b2[1];
+                    if (S == 1) {
+                        const half2_t h = {(half_t)v0, (half_t)v1};
+                        *reinterpret_cast<half2_t*>(a.y + (size_t)m * a.N + cc) = h;
+                    } else {
+                        float* pp = a.part + ((size_t)blockIdx.y * a.M + m) * a.N + cc;
+                        pp[0] = v0;
+                        pp[1] = v1;
+                    }
+                }
             }
         }
-        __syncthreads();                           // red is reused by the next row block
+        __syncthreads();                           // red is rewritten for the next strip
+#pragma unroll
+        for (int t = 0; t < NSTEP; ++t) wv[t] = wn[t];
+        sv = sn;
+        zv = zn;
     }
 }
 
@@ -481,9 +568,10 @@ extern "C" int q4_launch_gemv(const void* x, const int32_t* qweight, const int32
 
 extern "C" int q4_launch_splitk_reduce(const float* part, void* out, long total, int splits, hipStream_t stream);
 
-// Shapes the skinny kernel takes: 17..32 rows, sequential groups that are multiples of 128 rows.
+// Shapes the skinny kernel takes: 17..64 rows, sequential groups that are multiples of 128 rows.
 extern "C" int q4_skinny_applicable(int M, int K, int N, int groupsize, int has_gidx) {
-    return M > 16 && M <= 32 && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 64 == 0;
+    static const int max_rows = getenv("Q4_SKINNY_MAX_ROWS") ? atoi(getenv("Q4_SKINNY_MAX_ROWS")) : 64;
+    return M > 16 && M <= max_rows && M <= 64 && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 64 == 0;
 }
 
 static int skinny_splits(int K) {
@@ -511,9 +599,18 @@ extern "C" int q4_launch_skinny(const void* x, const int32_t* qweight, const int
     a.part = reinterpret_cast<float*>(workspace);
     a.M = M; a.K = K; a.N = N;
     const int S = skinny_splits(K);
-    const int chunks = K / 128;
-    const dim3 grid(N / kColsPerWave, S), block(64 * (chunks < 8 ? chunks : 8));
-    hipLaunchKernelGGL(skinny_seq_kernel<2>, grid, block, 0, stream, a);
+    const int strips = N / kColsPerWave;
+    // neighbouring strips per workgroup: enough for the whole grid to be resident at once (two workgroups
+    // per compute unit fit with two row blocks, one with more), at most 4
+    static const int force_l = getenv("Q4_SKINNY_STRIPS") ? atoi(getenv("Q4_SKINNY_STRIPS")) : 0;
+    const int slots = M <= 32 ? 512 : 256;
+    int L = force_l > 0 ? force_l : (strips * S + slots - 1) / slots;
+    L = L < 1 ? 1 : (L > 4 ? 4 : L);
+    a.strips_per_wg = L;
+    const dim3 grid((strips + L - 1) / L, S), block(512);    // wavefronts past the end of K read zeros
+    if (M <= 32) hipLaunchKernelGGL(skinny_seq_kernel<2>, grid, block, 0, stream, a);
+    else if (M <= 48) hipLaunchKernelGGL(skinny_seq_kernel<3>, grid, block, 0, stream, a);
+    else hipLaunchKernelGGL(skinny_seq_kernel<4>, grid, block, 0, stream, a);
     if (hipGetLastError() != hipSuccess) return -4;
     if (S > 1) return q4_launch_splitk_reduce(a.part, y, (long)M * N, S, stream);
     return 0;

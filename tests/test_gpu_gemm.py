@@ -136,8 +136,8 @@ def test_split_k_is_reproducible_and_matches_unsplit(oracle):
 @pytest.mark.parametrize("K,N,gs,act", [(4096, 1024, 128, False), (1408, 256, 128, False), (512, 384, 128, True),
                                         (11008, 256, 128, False)])
 def test_gemm_forward_17_to_64_rows(oracle, M, K, N, gs, act):
-    """17..32 rows take the weight-streaming kernel (both row blocks share one pass over the packed weights;
-    partial rows of the K splits are added by a second kernel), 33..64 the tiled kernel with split-K; with bias."""
+    """17..64 rows without act-order take the weight-streaming kernel (all row blocks share one pass over the packed
+    weights; partial rows of the K splits are added by a second kernel), act-order the tiled kernel; with bias."""
     import torch
     from alpaca_lora_4bit_amd import quant_hip
     layer = oracle.make_layer(K, N, gs, act_order=act, seed=K + N + M)
@@ -149,5 +149,23 @@ def test_gemm_forward_17_to_64_rows(oracle, M, K, N, gs, act):
                            bias=torch.from_numpy(bias).cuda())
     y2 = quant_hip.gemm_fwd(torch.from_numpy(x).cuda(), t["qweight"], t["qzeros"], t["scales"], t["g_idx"], gs,
                             bias=torch.from_numpy(bias).cuda())
+    assert y.shape == (M, N) and torch.equal(y, y2)
+    assert np.abs(y.float().cpu().numpy() - ref).max() <= 1e-2 * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("M", [20, 40, 64])
+@pytest.mark.parametrize("K,N", [(4096, 11008), (4096, 16512), (2048, 24704)])
+def test_gemm_forward_streaming_kernel_several_strips_per_workgroup(oracle, M, K, N):
+    """Wide outputs: a workgroup of the streaming kernel walks over 2 or 3 neighbouring 64-column strips with the
+    activations held in registers; 16512 and 24704 columns (258 and 386 strips, 4 and 3 per workgroup) leave the
+    last workgroup two strips."""
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    layer = oracle.make_layer(K, N, 128, seed=K + N + M)
+    t = to_cuda_layer(layer)
+    x = oracle.make_activations(M, K, seed=M + 5)
+    ref = oracle.matmul_recons(x, layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
+    y = quant_hip.gemm_fwd(torch.from_numpy(x).cuda(), t["qweight"], t["qzeros"], t["scales"], None, 128)
+    y2 = quant_hip.gemm_fwd(torch.from_numpy(x).cuda(), t["qweight"], t["qzeros"], t["scales"], None, 128)
     assert y.shape == (M, N) and torch.equal(y, y2)
     assert np.abs(y.float().cpu().numpy() - ref).max() <= 1e-2 * np.abs(ref).max()
