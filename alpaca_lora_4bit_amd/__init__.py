@@ -6,6 +6,8 @@ Sub-modules keep the reference's names so its callers read unchanged:
     quant_hip            tensor-level mirror of the reference's quant_cuda extension module
     models               Linear4bitLt, GPTQLoraModel
     monkeypatch.peft_tuners_lora_monkey_patch   replace_peft_model_with_int4_lora_model
+    arg_parser, Finetune4bConfig, train_data, gradient_checkpointing   what the finetune script imports
+    finetune, inference  the reference's two top-level scripts as runnable modules (python -m ...)
 
 `install_as_alpaca_lora_4bit()` registers these modules under the reference's package name so
 that `from alpaca_lora_4bit import autograd_4bit` in an unmodified caller resolves here.
@@ -19,7 +21,8 @@ import sys
 __version__ = "0.1.0"
 
 _ALIASED = ("autograd_4bit", "matmul_utils_4bit", "quant_hip", "models", "amp_wrapper", "model_attn_mlp_patch",
-            "loaders", "monkeypatch", "monkeypatch.peft_tuners_lora_monkey_patch")
+            "loaders", "arg_parser", "Finetune4bConfig", "train_data", "gradient_checkpointing", "monkeypatch",
+            "monkeypatch.peft_tuners_lora_monkey_patch")
 
 
 def install_as_alpaca_lora_4bit(name: str = "alpaca_lora_4bit") -> None:

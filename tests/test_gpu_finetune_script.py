@@ -1,0 +1,71 @@
+"""The finetune and inference flows end to end on the GPU (the reference's finetune.py / inference.py as modules):
+command line -> packed-model loader -> LoRA injection -> dataset reader -> transformers.Trainer under fp16 autocast
+-> adapter files -> generation with the adapter applied.  Model: the synthetic 2-block LLaMA of tiny_llama.py."""
+import json
+import os
+import random
+
+import pytest
+import torch
+
+from tiny_llama import GROUPSIZE, build
+
+pytestmark = pytest.mark.gpu
+
+WORDS = ["alpha", "beta", "gamma", "delta", "lora", "quant", "weight", "matrix", "token", "layer", "the", "of"]
+
+
+def _corpus(path, lines=48):
+    rnd = random.Random(1)
+    with open(path, "w") as fh:
+        for _ in range(lines):
+            # a strongly repetitive pattern: a few steps of LoRA training must lower its loss
+            start = rnd.randrange(len(WORDS))
+            fh.write(" ".join(WORDS[(start + j) % len(WORDS)] for j in range(10)) + "\n")
+
+
+@pytest.mark.parametrize("grad_chckpt", [False, True])
+def test_finetune_module_trains_and_saves_an_adapter(tmp_path, oracle, grad_chckpt):
+    from safetensors.torch import load_file
+    from alpaca_lora_4bit_amd import finetune
+    ckpt = str(tmp_path / "ckpt")
+    build(ckpt, oracle, seed=5, with_tokenizer=True)
+    data = str(tmp_path / "data.txt")
+    _corpus(data)
+    out = str(tmp_path / "lora_out")
+    argv = [data, "--ds_type", "txt", "--llama_q4_config_dir", ckpt, "--llama_q4_model",
+            os.path.join(ckpt, "model.safetensors"), "--groupsize", str(GROUPSIZE), "--lora_out_dir", out,
+            "--mbatch_size", "4", "--batch_size", "8", "--epochs", "3", "--lr", "5e-3", "--cutoff_len", "24",
+            "--warmup_steps", "1", "--logging_steps", "1", "--val_set_size", "0", "--lora_dropout", "0.0"]
+    if grad_chckpt:
+        argv += ["--grad_chckpt", "--grad_chckpt_ratio", "0.5"]
+    model, tokenizer, trainer = finetune.main(argv)
+
+    losses = [h["loss"] for h in trainer.state.log_history if "loss" in h]
+    assert len(losses) >= 6 and all(l == l for l in losses)                 # 48 rows / 8 per step * 3 epochs; no NaN
+    # only rank-8 adapters on q_proj / v_proj of a random model train: the loss falls slowly but steadily
+    assert sum(losses[-3:]) / 3 < sum(losses[:3]) / 3 - 0.1, losses
+    lora = [m for m in model.modules() if "Linear4bitLt" in str(type(m))]
+    assert len(lora) == 4                                                   # q_proj, v_proj of two blocks
+    assert all(float(m.lora_B["default"].weight.detach().abs().max()) > 0 for m in lora)      # B starts at zero
+    assert all(m.qweight.dtype == torch.int32 and m.scales.dtype == torch.float16 for m in lora)
+    if grad_chckpt:
+        assert [hasattr(l, "old_forward_for_cp") for l in model.model.layers] == [True, False]   # int(2 * 0.5) = 1 block
+
+    saved = load_file(os.path.join(out, "adapter_model.safetensors"))
+    assert len(saved) == 8 and all(k.startswith("base_model.model.model.layers.") for k in saved)
+    name = "model.layers.1.self_attn.v_proj"
+    live = dict(model.named_modules())[name]
+    assert torch.equal(saved[f"base_model.model.{name}.lora_B.weight"], live.lora_B["default"].weight.detach().cpu())
+    cfg = json.load(open(os.path.join(out, "adapter_config.json")))
+    assert cfg["r"] == 8 and cfg["lora_alpha"] == 16 and cfg["target_modules"] == ["q_proj", "v_proj"]
+
+    if not grad_chckpt:
+        # generation through the inference flow, with and without the adapter
+        from alpaca_lora_4bit_amd import inference
+        base_args = [ckpt, os.path.join(ckpt, "model.safetensors"), "--groupsize", str(GROUPSIZE), "--prompt",
+                     "alpha beta gamma", "--max_new_tokens", "6", "--greedy"]
+        text_lora, _ = inference.main(base_args + ["--lora", out])
+        text_base, _ = inference.main(base_args)
+        assert isinstance(text_lora, str) and text_lora.startswith("alpha beta gamma")
+        assert text_base.startswith("alpha beta gamma")
