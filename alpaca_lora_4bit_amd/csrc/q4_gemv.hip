@@ -58,6 +58,67 @@ __device__ __forceinline__ half8_t make_half8(uint32_t a, uint32_t b, uint32_t c
     return __builtin_bit_cast(half8_t, v);
 }
 
+// Finishes EB outputs per thread (e0, e0 + blockDim.x, ...): all LDS reads of the batch are issued before
+// the first sum needs them and all atomics of the batch are in flight before the first reply is looked at,
+// so a thread pays one LDS latency and one atomic round trip per batch, not per term.
+template <int EB>
+__device__ __forceinline__ void gemv_finish_batch(const GemvArgs& a, const float* red, int e0, int total, int n0,
+                                                  int nwaves) {
+    const int M = a.M, S = gridDim.y;
+    float v[EB];
+#pragma unroll
+    for (int i = 0; i < EB; ++i) {
+        const int e = min(e0 + i * (int)blockDim.x, total - 1);
+        float t = 0.f;
+        int w = 0;
+        for (; w + 8 <= nwaves; w += 8) {
+            float p[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) p[u] = red[(((w + u) * M) << 6) + e];
+            t += ((p[0] + p[1]) + (p[2] + p[3])) + ((p[4] + p[5]) + (p[6] + p[7]));
+        }
+        for (; w < nwaves; ++w) t += red[((w * M) << 6) + e];
+        v[i] = t;
+    }
+    if (S == 1) {
+#pragma unroll
+        for (int i = 0; i < EB; ++i) {
+            const int e = e0 + i * blockDim.x;
+            if (e < total) {
+                half_t* yp = a.y + (size_t)(e >> 6) * a.N + n0 + (e & 63);
+                float out = v[i];
+                if (a.accumulate) out += (float)*yp;
+                *yp = (half_t)out;
+            }
+        }
+        return;
+    }
+    unsigned long long old[EB], add[EB];
+#pragma unroll
+    for (int i = 0; i < EB; ++i) {
+        const int e = e0 + i * blockDim.x;
+        const float c = fminf(fmaxf(v[i], -kClamp), kClamp);
+        const long long fx = __float2ll_rn(c * (float)(1 << kFracBits));
+        add[i] = (1ull << 56) + (unsigned long long)(fx + kBias);
+        old[i] = 0;
+        if (e < total)
+            old[i] = __hip_atomic_fetch_add(a.acc64 + (size_t)(e >> 6) * a.N + n0 + (e & 63), add[i],
+                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int i = 0; i < EB; ++i) {
+        const int e = e0 + i * blockDim.x;
+        if (e < total && (old[i] >> 56) == (unsigned long long)(S - 1)) {      // last of the S workgroups of the strip
+            const size_t at = (size_t)(e >> 6) * a.N + n0 + (e & 63);
+            const long long tot = (long long)((old[i] + add[i]) & ((1ull << 56) - 1)) - (long long)S * kBias;
+            float out = (float)((double)tot * (1.0 / (double)(1 << kFracBits)));
+            if (a.accumulate) out += (float)a.y[at];
+            a.y[at] = (half_t)out;
+            __hip_atomic_store(a.acc64 + at, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
 // yacc[j][r] of this lane belongs to row 4*kk + r, column n0 + 4c + j.
 __device__ __forceinline__ void gemv_finish(const GemvArgs& a, const float4_t yacc[4], int n0, int wave, int nwaves,
                                             int kk, int c) {
@@ -71,29 +132,11 @@ __device__ __forceinline__ void gemv_finish(const GemvArgs& a, const float4_t ya
                 float4_t{yacc[0][r], yacc[1][r], yacc[2][r], yacc[3][r]};
     }
     __syncthreads();
-    for (int e = threadIdx.x; e < M * 64; e += blockDim.x) {
-        float v = 0.f;
-        for (int w = 0; w < nwaves; ++w) v += red[((w * M) << 6) + e];
-        const int m = e >> 6, col = n0 + (e & 63);
-        half_t* yp = a.y + (size_t)m * a.N + col;
-        const int S = gridDim.y;
-        if (S == 1) {
-            if (a.accumulate) v += (float)*yp;
-            *yp = (half_t)v;
-        } else {
-            v = fminf(fmaxf(v, -kClamp), kClamp);
-            const long long fx = __float2ll_rn(v * (float)(1 << kFracBits));
-            const unsigned long long add = (1ull << 56) + (unsigned long long)(fx + kBias);
-            unsigned long long* ap = a.acc64 + (size_t)m * a.N + col;
-            const unsigned long long old = __hip_atomic_fetch_add(ap, add, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if ((old >> 56) == (unsigned long long)(S - 1)) {
-                const long long tot = (long long)((old + add) & ((1ull << 56) - 1)) - (long long)S * kBias;
-                float out = (float)((double)tot * (1.0 / (double)(1 << kFracBits)));
-                if (a.accumulate) out += (float)*yp;
-                *yp = (half_t)out;
-                __hip_atomic_store(ap, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
+    const int total = M * 64;
+    if (total <= (int)blockDim.x) {              // at most one output per thread (uniform)
+        if ((int)threadIdx.x < total) gemv_finish_batch<1>(a, red, threadIdx.x, total, n0, nwaves);
+    } else {
+        for (int e0 = threadIdx.x; e0 < total; e0 += 2 * blockDim.x) gemv_finish_batch<2>(a, red, e0, total, n0, nwaves);
     }
 }
 
