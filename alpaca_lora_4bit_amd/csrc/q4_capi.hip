@@ -97,6 +97,7 @@ extern "C" int q4_gemv_f16(const void* x, const int32_t* qweight, const int32_t*
     if (rc != Q4_OK) return rc;
     if (!x || !y) return Q4_ERR_NULL_POINTER;
     if (M < 1 || M > 16 || K > 32 * 255 * 8 * 16) return Q4_ERR_BAD_SHAPE;
+    if ((long long)(K / 8) * N * 4 >= 0x70000000ll) return Q4_ERR_BAD_SHAPE;      /* 32-bit buffer offsets */
     if (misaligned(x) || misaligned(y)) return Q4_ERR_MISALIGNED;
     if (!workspace || workspace_bytes < q4_gemv_workspace_bytes(M, K, N)) return Q4_ERR_WORKSPACE;
     if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;

@@ -72,6 +72,11 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* p, unsigned bytes) {
 __device__ __forceinline__ uint4_t buf_load128(rsrc_t r, int voff, int soff) {
     return __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
 }
+// Same with the non-temporal cache policy, for data that is read once (packed weights in the streaming kernels).
+constexpr int kAuxNonTemporal = 2;
+__device__ __forceinline__ uint4_t buf_load128_stream(rsrc_t r, int voff, int soff) {
+    return __builtin_bit_cast(uint4_t, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, kAuxNonTemporal));
+}
 __device__ __forceinline__ uint2_t buf_load64(rsrc_t r, int voff, int soff) {
     return __builtin_bit_cast(uint2_t, __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0));
 }

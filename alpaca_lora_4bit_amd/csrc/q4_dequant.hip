@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void dequant_kernel(
             o[p] = as_u32(dequant_pair(codes_to_half2(codes), s2[p], zero2[p]));
         }
         uint4_t ov = {o[0], o[1], o[2], o[3]};
-        *reinterpret_cast<uint4_t*>(out + (size_t)k * N + n0) = ov;
+        __builtin_nontemporal_store(ov, reinterpret_cast<uint4_t*>(out + (size_t)k * N + n0));   // written once, not re-read here
     }
 }
 

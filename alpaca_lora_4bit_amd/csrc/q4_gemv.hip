@@ -172,11 +172,14 @@ __global__ __launch_bounds__(NSTEP >= 16 ? 512 : 1024) void gemv_seq_kernel(Gemv
             zv[i] = a.qzeros[(size_t)(g0 + i) * ncol8 + (col >> 3)];
         }
         uint4_t wv[NSTEP], xv[NSTEP];
-        const uint32_t* wp = a.qweight + (size_t)((k0 >> 3) + kk) * a.N + col;
+        // the packed words are read exactly once per product: streaming loads, so they do not displace the
+        // activations and scales that every strip shares from the caches
+        const rsrc_t rw = make_rsrc(a.qweight, (unsigned)((size_t)(a.K >> 3) * a.N * 4));
+        const int vw = (((k0 >> 3) + kk) * a.N + col) * 4;
         const half_t* xp = a.x + (size_t)min(c, a.M - 1) * a.K + k0 + 8 * kk;
 #pragma unroll
         for (int t = 0; t < NSTEP; ++t) {
-            wv[t] = *reinterpret_cast<const uint4_t*>(wp + (size_t)(4 * t) * a.N);
+            wv[t] = buf_load128_stream(rw, vw, 16 * t * a.N);
             xv[t] = *reinterpret_cast<const uint4_t*>(xp + 32 * t);
         }
         // Rows >= M of the A operand hold a copy of row M-1: harmless, a row of A only reaches the
@@ -464,7 +467,7 @@ __global__ __launch_bounds__(512) void gemv_gidx_kernel(GemvArgs a) {
         }
 #pragma unroll
         for (int t = 0; t < NSTEP; ++t) {
-            wv[t] = *reinterpret_cast<const uint4_t*>(wp + (size_t)(4 * t) * a.N);
+            wv[t] = __builtin_nontemporal_load(reinterpret_cast<const uint4_t*>(wp + (size_t)(4 * t) * a.N));
             xv[t] = *reinterpret_cast<const uint4_t*>(xp + 32 * t);
         }
         __builtin_amdgcn_sched_barrier(0);
