@@ -10,6 +10,7 @@
 // W is read in place with strides and in its own dtype (fp32 or fp16): no cast or transpose
 // kernels around the adapter.
 #include "q4_common.hpp"
+#include <stdlib.h>
 
 namespace q4 {
 
@@ -43,7 +44,8 @@ constexpr int kDownWaves = 16;
 template <int RB, int WL, bool F32, int RQ>   // RQ: ceil(R/4) for kCols / kRowsT, else unused
 __global__ __launch_bounds__(64 * kDownWaves) void lora_down_kernel(const half_t* __restrict__ in,
                                                                     const void* __restrict__ w, int w_sr, int w_sc,
-                                                                    half_t* __restrict__ out, int M, int C, int R) {
+                                                                    half_t* __restrict__ out, int M, int C, int R,
+                                                                    int rows) {
     constexpr int NW = kDownWaves;
     constexpr int UN = WL == kAny ? (RB == 1 ? 4 : RB == 2 ? 2 : 1) : (RB == 1 ? 8 : 4);   // steps whose loads are issued together
     constexpr int ES = F32 ? 4 : 2;
@@ -54,10 +56,10 @@ __global__ __launch_bounds__(64 * kDownWaves) void lora_down_kernel(const half_t
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int kk = lane >> 4, c = lane & 15;
-    const int m0 = blockIdx.x * 16;
+    const int m0 = blockIdx.x * rows;                           // rows = 16, 8 or 4: operand rows past it read as zero
     const int steps = C / 32;                                   // C is a multiple of 32
     const int s_begin = (steps * wave) / NW, s_end = (steps * (wave + 1)) / NW;
-    const rsrc_t rs_in = make_rsrc(in + (size_t)m0 * C, (unsigned)min(16, M - m0) * (unsigned)C * 2u);
+    const rsrc_t rs_in = make_rsrc(in + (size_t)m0 * C, (unsigned)min(rows, M - m0) * (unsigned)C * 2u);
     const rsrc_t rs_w = make_rsrc(w, ((unsigned)(R - 1) * (unsigned)w_sr + (unsigned)(C - 1) * (unsigned)w_sc + 1u) * ES);
     const int voff_in = (c * C + 8 * kk) * 2;
     float4_t acc[RB];
@@ -207,7 +209,7 @@ __global__ __launch_bounds__(64 * kDownWaves) void lora_down_kernel(const half_t
 #pragma unroll
         for (int wv = 0; wv < NW; ++wv) v += red[wv][b][i];
         const int m = m0 + (i >> 4), j = 16 * b + (i & 15);
-        if (m < M && j < R) out[(size_t)m * R + j] = (half_t)v;
+        if ((i >> 4) < rows && m < M && j < R) out[(size_t)m * R + j] = (half_t)v;
     }
 }
 
@@ -389,8 +391,14 @@ inline GradPlan plan_grad(int M, int C, int R) {
 template <int RB, int WL, bool F32, int RQ>
 static void launch_down_kernel(const q4::half_t* ip, const void* w, int w_sr, int w_sc, q4::half_t* op,
                                int M, int C, int R, hipStream_t stream) {
-    hipLaunchKernelGGL((q4::lora_down_kernel<RB, WL, F32, RQ>), dim3((M + 15) / 16), dim3(64 * q4::kDownWaves), 0, stream,
-                       ip, w, w_sr, w_sc, op, M, C, R);
+    // rows of `in` per workgroup: 16 fill the MFMA operand, but with few rows that leaves compute units idle and
+    // the kernel is bound by the latency of its single burst of loads, so smaller blocks spread it out
+    static const int force_rows = getenv("Q4_LORA_DOWN_ROWS") ? atoi(getenv("Q4_LORA_DOWN_ROWS")) : 0;
+    int rows = 16;
+    while (rows > 4 && (M + rows - 1) / rows < 256) rows >>= 1;
+    if (force_rows == 4 || force_rows == 8 || force_rows == 16) rows = force_rows;
+    hipLaunchKernelGGL((q4::lora_down_kernel<RB, WL, F32, RQ>), dim3((M + rows - 1) / rows), dim3(64 * q4::kDownWaves), 0,
+                       stream, ip, w, w_sr, w_sc, op, M, C, R, rows);
 }
 
 template <int WL, bool F32>
