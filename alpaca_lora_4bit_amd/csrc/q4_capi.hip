@@ -7,11 +7,12 @@
 extern "C" {
 int q4_launch_dequant(const int32_t*, const int32_t*, const void*, const int32_t*, int, void*, int, int, hipStream_t);
 int q4_launch_permute_rows(const int32_t*, const int32_t*, int32_t*, int, int, hipStream_t);
-int q4_launch_gemv(const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, void*, int,
-                   int, int, int, int, void*, hipStream_t);
+int q4_launch_gemv(const void*, const int32_t*, const int32_t*, const void*, const int32_t*, const int32_t*, int, void*,
+                   int, int, int, int, int, void*, hipStream_t);
 int q4_launch_gemm(int, const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, const void*,
                    const void*, const void*, int, int, int, float, int, void*, int, int, int, int, void*, size_t, hipStream_t);
 size_t q4_gemm_plan_workspace(int, int, int, int);
+int q4_gemv_sorted_applicable(int, int);
 int q4_launch_lora_down(const void*, const void*, int, int, int, void*, int, int, int, hipStream_t);
 int q4_launch_lora_grad(const void*, const void*, float*, int, int, float, int, int, int, void*, hipStream_t);
 size_t q4_lora_grad_workspace(int, int, int);
@@ -34,7 +35,7 @@ int check_layer(const void* qweight, const void* qzeros, const void* scales, con
 }
 }  // namespace
 
-extern "C" int q4_abi_version(void) { return 4; }
+extern "C" int q4_abi_version(void) { return 5; }
 
 extern "C" const char* q4_error_string(int code) {
     switch (code) {
@@ -90,19 +91,36 @@ extern "C" int q4_permute_rows(const int32_t* qweight, const int32_t* perm, int3
     return q4_launch_permute_rows(qweight, perm, out, K, N, (hipStream_t)stream);
 }
 
-extern "C" int q4_gemv_f16(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
-                           const int32_t* g_idx, int groupsize, void* y, int accumulate,
-                           int M, int K, int N, int G, void* workspace, size_t workspace_bytes, void* stream) {
+static int gemv_common(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                       const int32_t* g_idx, const int32_t* perm, int groupsize, void* y, int accumulate,
+                       int M, int max_rows, int K, int N, int G, void* workspace, size_t workspace_bytes, void* stream) {
     int rc = check_layer(qweight, qzeros, scales, g_idx, groupsize, K, N, G);
     if (rc != Q4_OK) return rc;
     if (!x || !y) return Q4_ERR_NULL_POINTER;
-    if (M < 1 || M > 16 || K > 32 * 255 * 8 * 16) return Q4_ERR_BAD_SHAPE;
+    if (M < 1 || M > max_rows || K > 32 * 255 * 8 * 16) return Q4_ERR_BAD_SHAPE;
     if ((long long)(K / 8) * N * 4 >= 0x70000000ll) return Q4_ERR_BAD_SHAPE;      /* 32-bit buffer offsets */
     if (misaligned(x) || misaligned(y)) return Q4_ERR_MISALIGNED;
     if (!workspace || workspace_bytes < q4_gemv_workspace_bytes(M, K, N)) return Q4_ERR_WORKSPACE;
     if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
-    return q4_launch_gemv(x, qweight, qzeros, scales, g_idx, groupsize, y, accumulate, M, K, N, G, workspace,
+    return q4_launch_gemv(x, qweight, qzeros, scales, g_idx, perm, groupsize, y, accumulate, M, K, N, G, workspace,
                           (hipStream_t)stream);
+}
+
+extern "C" int q4_gemv_f16(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                           const int32_t* g_idx, int groupsize, void* y, int accumulate,
+                           int M, int K, int N, int G, void* workspace, size_t workspace_bytes, void* stream) {
+    return gemv_common(x, qweight, qzeros, scales, g_idx, nullptr, groupsize, y, accumulate, M, 16, K, N, G, workspace,
+                       workspace_bytes, stream);
+}
+
+extern "C" int q4_gemv_sorted_f16(const void* x, const int32_t* qweight_sorted, const int32_t* qzeros, const void* scales,
+                                  const int32_t* perm, int groupsize, void* y, int accumulate,
+                                  int M, int K, int N, int G, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!perm) return Q4_ERR_NULL_POINTER;
+    if (reinterpret_cast<uintptr_t>(perm) & 3u) return Q4_ERR_MISALIGNED;
+    if (M >= 1 && !q4_gemv_sorted_applicable(M, K)) return Q4_ERR_BAD_SHAPE;
+    return gemv_common(x, qweight_sorted, qzeros, scales, nullptr, perm, groupsize, y, accumulate, M, 4, K, N, G, workspace,
+                       workspace_bytes, stream);
 }
 
 static int gemm_common(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros, const void* scales,

@@ -51,6 +51,7 @@ struct GemvArgs {
     int accumulate;
     int M, K, N, G;
     unsigned long long* acc64;   // [M, N], zero between calls
+    const int32_t* perm;         // gemv_seq_perm_kernel only: original index of every (sorted) reduction row
 };
 
 __device__ __forceinline__ half8_t make_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
@@ -144,49 +145,58 @@ __device__ __forceinline__ void gemv_finish(const GemvArgs& a, const float4_t ya
 // GSTEPS = steps of 32 rows per quantization group (1, 2, 4, 8; NSTEP % GSTEPS == 0), or
 // 0 when a whole chunk lies inside one group (groupsize % (32*NSTEP) == 0).
 template <int NSTEP, int GSTEPS>
-__global__ __launch_bounds__(NSTEP >= 16 ? 512 : 1024) void gemv_seq_kernel(GemvArgs a) {
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int nwaves = blockDim.x >> 6;
-    const int kk = lane >> 4, c = lane & 15;
-    const int n0 = blockIdx.x * kColsPerWave;
-    const int k0 = (blockIdx.y * nwaves + wave) * (32 * NSTEP);
-    constexpr int NG = GSTEPS == 0 ? 1 : NSTEP / GSTEPS;
-    constexpr int GS = GSTEPS == 0 ? NSTEP : GSTEPS;
+struct SeqChunk {
+    static constexpr int NG = GSTEPS == 0 ? 1 : NSTEP / GSTEPS;
+    static constexpr int GS = GSTEPS == 0 ? NSTEP : GSTEPS;
+    uint2_t sv[NG];
+    uint32_t zv[NG];
+    uint4_t wv[NSTEP], xv[NSTEP];
 
-    float4_t yacc[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) yacc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
-
-    if (k0 < a.K) {                               // wave-uniform; K % (32*NSTEP) == 0 (checked on the host)
+    // scale / zero of every group of the chunk first: they are consumed last but must not sit behind the
+    // weights in the in-order return queue.  The packed words are read exactly once per product: streaming
+    // loads, so they do not displace the activations and scales that every strip shares from the caches.
+    __device__ __forceinline__ void load_weights(const GemvArgs& a, int k0, int col, int kk) {
         const int ncol8 = a.N >> 3;
-        const int col = n0 + 4 * c;
-        // scale / zero of every group of the chunk first: they are consumed last but must not
-        // sit behind the weights in the in-order return queue
         const int g0 = k0 / a.groupsize;
-        uint2_t sv[NG];
-        uint32_t zv[NG];
 #pragma unroll
         for (int i = 0; i < NG; ++i) {
             sv[i] = *reinterpret_cast<const uint2_t*>(a.scales + (size_t)(g0 + i) * a.N + col);
             zv[i] = a.qzeros[(size_t)(g0 + i) * ncol8 + (col >> 3)];
         }
-        uint4_t wv[NSTEP], xv[NSTEP];
-        // the packed words are read exactly once per product: streaming loads, so they do not displace the
-        // activations and scales that every strip shares from the caches
         const rsrc_t rw = make_rsrc(a.qweight, (unsigned)((size_t)(a.K >> 3) * a.N * 4));
         const int vw = (((k0 >> 3) + kk) * a.N + col) * 4;
-        const half_t* xp = a.x + (size_t)min(c, a.M - 1) * a.K + k0 + 8 * kk;
 #pragma unroll
-        for (int t = 0; t < NSTEP; ++t) {
-            wv[t] = buf_load128_stream(rw, vw, 16 * t * a.N);
-            xv[t] = *reinterpret_cast<const uint4_t*>(xp + 32 * t);
-        }
-        // Rows >= M of the A operand hold a copy of row M-1: harmless, a row of A only reaches the
-        // same row of the product, and rows >= M of the product are never stored.
-        // Keep the burst a burst: the scheduler must not sink loads below the arithmetic.
-        __builtin_amdgcn_sched_barrier(0);
+        for (int t = 0; t < NSTEP; ++t) wv[t] = buf_load128_stream(rw, vw, 16 * t * a.N);
+    }
 
+    // The same without a branch around it: a wavefront past the end of K (wave-uniform `live` false) fetches
+    // from an offset beyond every buffer, which returns zeros without traffic.
+    __device__ __forceinline__ void load_weights_branch_free(const GemvArgs& a, int k0, int col, int kk, bool live) {
+        constexpr int kFar = 0x70000000;
+        const int ncol8 = a.N >> 3;
+        const int g0 = live ? k0 / a.groupsize : 0;
+        const int off = live ? 0 : kFar;
+        const rsrc_t rs = make_rsrc(a.scales, (unsigned)((size_t)a.G * a.N * 2));
+        const rsrc_t rz = make_rsrc(a.qzeros, (unsigned)((size_t)a.G * ncol8 * 4));
+#pragma unroll
+        for (int i = 0; i < NG; ++i) {
+            sv[i] = buf_load64(rs, ((g0 + i) * a.N + col) * 2, off);
+            zv[i] = buf_load32(rz, ((g0 + i) * ncol8 + (col >> 3)) * 4, off);
+        }
+        const rsrc_t rw = make_rsrc(a.qweight, (unsigned)((size_t)(a.K >> 3) * a.N * 4));
+        const int vw = live ? (((k0 >> 3) + kk) * a.N + col) * 4 : 0;
+#pragma unroll
+        for (int t = 0; t < NSTEP; ++t) wv[t] = buf_load128_stream(rw, vw, off + 16 * t * a.N);
+    }
+
+    // Rows >= M of the A operand hold a copy of row M-1: harmless, a row of A only reaches the same row of
+    // the product, and rows >= M of the product are never stored.
+    __device__ __forceinline__ void load_x(const half_t* row_chunk) {
+#pragma unroll
+        for (int t = 0; t < NSTEP; ++t) xv[t] = *reinterpret_cast<const uint4_t*>(row_chunk + 32 * t);
+    }
+
+    __device__ __forceinline__ void multiply(const GemvArgs& a, float4_t yacc[4], int c) const {
         // B operands of the two extra MFMAs: per-position offsets (1024 | 64) and all ones
         const half8_t offs = make_half8(0x64006400u, 0x54005400u, 0x64006400u, 0x54005400u);
         const half8_t ones = make_half8(0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u);
@@ -234,6 +244,102 @@ __global__ __launch_bounds__(NSTEP >= 16 ? 512 : 1024) void gemv_seq_kernel(Gemv
                 }
             }
         }
+    }
+};
+
+template <int NSTEP, int GSTEPS>
+__global__ __launch_bounds__(NSTEP >= 16 ? 512 : 1024) void gemv_seq_kernel(GemvArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nwaves = blockDim.x >> 6;
+    const int kk = lane >> 4, c = lane & 15;
+    const int n0 = blockIdx.x * kColsPerWave;
+    const int k0 = (blockIdx.y * nwaves + wave) * (32 * NSTEP);
+
+    float4_t yacc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) yacc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    if (k0 < a.K) {                               // wave-uniform; K % (32*NSTEP) == 0 (checked on the host)
+        SeqChunk<NSTEP, GSTEPS> ch;
+        ch.load_weights(a, k0, n0 + 4 * c, kk);
+        ch.load_x(a.x + (size_t)min(c, a.M - 1) * a.K + k0 + 8 * kk);
+        // Keep the burst a burst: the scheduler must not sink loads below the arithmetic.
+        __builtin_amdgcn_sched_barrier(0);
+        ch.multiply(a, yacc, c);
+    }
+    gemv_finish(a, yacc, n0, wave, nwaves, kk, c);
+}
+
+// The same for an act-order layer whose packed rows were sorted by group (q4_permute_rows): row p of the
+// sorted matrix is row perm[p] of the original, so the product needs x[:, perm[p]].  Gathering from global
+// memory would cost one scattered request per element in every strip's workgroups; instead the workgroup copies
+// the whole activation rows into LDS with coalesced loads (M*K*2 bytes, small for M <= 4), gathers the
+// entries of its K range from there into the operand tile and continues as the kernel above.  The
+// permutation entries are requested first and the weights right after, so everything is in flight together.
+// LDS: reduction buffer [nwaves][M][64] fp32, operand tile [M][span] fp16, activation rows [M][K] fp16.
+template <int NSTEP, int GSTEPS>
+__global__ __launch_bounds__(1024) void gemv_seq_perm_kernel(GemvArgs a) {
+    extern __shared__ float red[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nwaves = blockDim.x >> 6;
+    const int kk = lane >> 4, c = lane & 15;
+    const int n0 = blockIdx.x * kColsPerWave;
+    const int span = nwaves * 32 * NSTEP;          // reduction rows of this workgroup
+    const int kbase = blockIdx.y * span;
+    const int k0 = kbase + wave * (32 * NSTEP);
+    const bool active = k0 < a.K;                  // wave-uniform
+    half_t* xs = reinterpret_cast<half_t*>(red + ((nwaves * a.M) << 6));     // [M][span]
+    half_t* xfull = xs + a.M * span;                                          // [M][K]
+
+    float4_t yacc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) yacc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    // No branch sits between the loads below (out-of-range pieces come back as zeros), so the compiler's wait
+    // before the first use of the early ones does not include the weights.
+    constexpr int PT = 2;                          // reduction rows per thread: span <= 2 * blockDim.x
+    constexpr int XT = 8;                          // 16-byte pieces of x per thread: M*K*2 <= 64 KB with 512 threads
+    const rsrc_t rp = make_rsrc(a.perm, (unsigned)a.K * 4u);
+    const rsrc_t rx = make_rsrc(a.x, (unsigned)(a.M * a.K) * 2u);
+    int src[PT];
+#pragma unroll
+    for (int u = 0; u < PT; ++u) src[u] = (int)buf_load32(rp, (kbase + (int)threadIdx.x + u * (int)blockDim.x) * 4, 0);
+    uint4_t xc[XT];
+#pragma unroll
+    for (int u = 0; u < XT; ++u) xc[u] = buf_load128(rx, ((int)threadIdx.x + u * (int)blockDim.x) * 16, 0);
+    SeqChunk<NSTEP, GSTEPS> ch;
+    ch.load_weights_branch_free(a, k0, n0 + 4 * c, kk, active);
+    __builtin_amdgcn_sched_barrier(0);
+    const int n16 = (a.M * a.K) >> 3;              // K % 32 == 0
+#pragma unroll
+    for (int u = 0; u < XT; ++u) {
+        const int i = threadIdx.x + u * blockDim.x;
+        if (i < n16) reinterpret_cast<uint4_t*>(xfull)[i] = xc[u];
+    }
+    __syncthreads();
+    {
+        half_t got[PT][4];                         // all LDS reads first, then the writes: one LDS latency, not 2*M
+#pragma unroll
+        for (int u = 0; u < PT; ++u)
+#pragma unroll
+            for (int m = 0; m < 4; ++m) got[u][m] = xfull[min(m, a.M - 1) * a.K + src[u]];
+#pragma unroll
+        for (int u = 0; u < PT; ++u) {
+            const int i = threadIdx.x + u * blockDim.x;
+            if (i < span && kbase + i < a.K) {
+#pragma unroll
+                for (int m = 0; m < 4; ++m)
+                    if (m < a.M) xs[m * span + i] = got[u][m];
+            }
+        }
+    }
+    __syncthreads();
+    if (active) {
+        ch.load_x(xs + min(c, a.M - 1) * span + (k0 - kbase) + 8 * kk);
+        __builtin_amdgcn_sched_barrier(0);
+        ch.multiply(a, yacc, c);
     }
     gemv_finish(a, yacc, n0, wave, nwaves, kk, c);
 }
@@ -572,8 +678,25 @@ static void launch_seq(const q4::GemvPlan& p, dim3 grid, dim3 block, size_t lds,
     }
 }
 
+// Shapes q4_gemv_sorted_f16 takes: up to 4 rows whose activations (plus 4 KB per row of staging) fit in 64 KB of LDS.
+extern "C" int q4_gemv_sorted_applicable(int M, int K) {
+    return M >= 1 && M <= 4 && K >= 1024 && (size_t)M * ((size_t)K * 2 + 4096) <= 65536;   // K >= 1024: 8 wavefronts
+}
+
+template <int NSTEP>
+static void launch_seq_perm(const q4::GemvPlan& p, dim3 grid, dim3 block, size_t lds, hipStream_t stream, const q4::GemvArgs& a) {
+    using namespace q4;
+    switch (p.gsteps) {
+        case 0: hipLaunchKernelGGL((gemv_seq_perm_kernel<NSTEP, 0>), grid, block, lds, stream, a); break;
+        case 1: if constexpr (NSTEP > 1) hipLaunchKernelGGL((gemv_seq_perm_kernel<NSTEP, 1>), grid, block, lds, stream, a); break;
+        case 2: if constexpr (NSTEP > 2) hipLaunchKernelGGL((gemv_seq_perm_kernel<NSTEP, 2>), grid, block, lds, stream, a); break;
+    }
+}
+
+// `perm` != null: the packed rows are sorted by group and x is gathered through perm inside the kernel
+// (sequential groups only, M <= 4).
 extern "C" int q4_launch_gemv(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
-                              const int32_t* g_idx, int groupsize, void* y, int accumulate,
+                              const int32_t* g_idx, const int32_t* perm, int groupsize, void* y, int accumulate,
                               int M, int K, int N, int G, void* workspace, hipStream_t stream) {
     using namespace q4;
     GemvArgs a;
@@ -587,13 +710,23 @@ extern "C" int q4_launch_gemv(const void* x, const int32_t* qweight, const int32
     a.accumulate = accumulate;
     a.M = M; a.K = K; a.N = N; a.G = G;
     a.acc64 = reinterpret_cast<unsigned long long*>(workspace);
+    a.perm = perm;
 
     const bool seq = (g_idx == nullptr);
     const GemvPlan p = plan_gemv(K, N, groupsize, seq, 4);
     const dim3 grid(N / kColsPerWave, p.splits);
     const dim3 block(64 * p.waves);
     const size_t lds = (size_t)p.waves * M * 64 * sizeof(float);
-    if (seq) {
+    if (perm) {
+        // + the operand tile and the activation rows; q4_gemv_sorted_applicable() keeps this within 64 KB
+        const size_t lds_x = lds + (size_t)M * p.waves * 32 * p.nstep * sizeof(half_t) + (size_t)M * K * sizeof(half_t);
+        if (!seq || M > 4 || lds_x > 65536 || (size_t)M * K / 8 > (size_t)8 * block.x) return -2;
+        switch (p.nstep) {
+            case 4: launch_seq_perm<4>(p, grid, block, lds_x, stream, a); break;
+            case 2: launch_seq_perm<2>(p, grid, block, lds_x, stream, a); break;
+            default: launch_seq_perm<1>(p, grid, block, lds_x, stream, a); break;
+        }
+    } else if (seq) {
         switch (p.nstep) {
             case 16: launch_seq<16>(p, grid, block, lds, stream, a); break;
             case 8: launch_seq<8>(p, grid, block, lds, stream, a); break;

@@ -22,6 +22,7 @@ from ._lib import Q4Error  # noqa: F401  (re-exported)
 _lib.lib()  # fail at import time, loudly, if the HIP library is missing
 
 MAX_GEMV_ROWS = 16
+MAX_GEMV_SORTED_ROWS = 3          # q4_gemv_sorted_f16 (x gathered inside the kernel) wins up to 3 rows, ties at 4
 _workspaces = {}
 _scratch_bufs = {}
 
@@ -287,15 +288,25 @@ def gemv(x, qweight, qzeros, scales, g_idx=None, groupsize=None, out=None, accum
         out = torch.empty(_out_shape(out_shape, M, N), dtype=torch.float16, device=dev)
     _require(out.dtype == torch.float16 and out.numel() == M * N and out.shape[-1] == N and out.is_contiguous()
              and out.device == dev, "out must be a contiguous float16 [..., N] tensor with M rows on the same device")
+    L = _lib.lib()
+    nbytes = L.q4_gemv_workspace_bytes(M, K, N)
     plan = _actorder_plan(qweight, scales, g_idx, groupsize, G)
+    if plan is not None and M <= MAX_GEMV_SORTED_ROWS and K >= 1024 and M * (2 * K + 4096) <= 65536:     # rows fit in LDS
+        # sorted copy of the packed rows; the kernel gathers x through the permutation itself
+        perm, _, qweight, gs_sorted = plan
+        with torch.cuda.device(dev):
+            ws = _workspace(dev, nbytes)
+            rc = L.q4_gemv_sorted_f16(x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
+                                      perm.data_ptr(), gs_sorted, out.data_ptr(), int(bool(accumulate)), M, K, N, G,
+                                      ws.data_ptr(), ws.numel(), _stream(dev))
+        _lib.check(rc, "q4_gemv_sorted_f16")
+        return out
     if plan is not None:
         perm, _, qweight, gs_sorted = plan
         x2 = x2.index_select(1, perm)
         gp, gs = 0, gs_sorted
     else:
         gp, gs = _gidx_arg(g_idx, groupsize, G)
-    L = _lib.lib()
-    nbytes = L.q4_gemv_workspace_bytes(M, K, N)
     with torch.cuda.device(dev):
         ws = _workspace(dev, nbytes)
         rc = L.q4_gemv_f16(x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), gp, gs,

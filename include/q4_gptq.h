@@ -84,6 +84,18 @@ int q4_gemv_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, co
                 int M, int K, int N, int G,
                 void *workspace, size_t workspace_bytes, void *stream);
 
+/* The same product for an act-order layer whose packed rows were sorted by group with q4_permute_rows
+ * (1 <= M <= 4, K >= 1024 and M * (2*K + 4096) <= 65536 bytes, i.e. the activation rows fit in LDS:
+ * K <= 30720 at M=1, K <= 6144 at M=4): `qweight_sorted` is that sorted copy, `perm` [K] int32 the permutation it was made with
+ * (perm[p] = original index of sorted row p), `groupsize` = K / G.  x is the ORIGINAL activation matrix: the
+ * kernel gathers x[:, perm[p]] itself (through LDS) while its weight loads are in flight, which replaces the separate gather
+ * the caller would otherwise run before q4_gemv_f16.  The values are those of the reference's act-order
+ * product (quant_cuda_kernel.cu:443-536 with per-row g_idx).  Workspace as for q4_gemv_f16. */
+int q4_gemv_sorted_f16(const void *x, const int32_t *qweight_sorted, const int32_t *qzeros, const void *scales,
+                       const int32_t *perm, int groupsize, void *y, int accumulate,
+                       int M, int K, int N, int G,
+                       void *workspace, size_t workspace_bytes, void *stream);
+
 /* Forward GEMM, any M >= 1:
  *   y fp16 [M, N] = x fp16 [M, K] @ W  (+ bias fp16 [N])  (+ lora_scale * xa fp16 [M, R] @ Bm [R, N])
  * with fp32 accumulation on MFMA; W tiles are dequantized in LDS and never written to HBM.

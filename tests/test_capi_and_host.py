@@ -51,6 +51,11 @@ def test_error_codes_and_validation_need_no_gpu():
     assert L.q4_gemv_f16(fake, fake, fake, fake, None, 128, fake, 0, 17, 256, 128, 2, fake, 1 << 20, None) == -2
     assert L.q4_gemv_f16(fake, fake, fake, fake, None, 128, fake, 0, 1, 256, 128, 2, None, 0, None) == -3
     assert L.q4_gemv_f16(fake, fake, fake, fake, None, 128, fake, 0, 1, 256, 128, 2, fake, 8, None) == -3
+    assert L.q4_gemv_sorted_f16(fake, fake, fake, fake, None, 128, fake, 0, 1, 256, 128, 2, fake, 1 << 20, None) == -1   # no perm
+    assert L.q4_gemv_sorted_f16(fake, fake, fake, fake, fake, 128, fake, 0, 5, 256, 128, 2, fake, 1 << 20, None) == -2   # M > 4
+    assert L.q4_gemv_sorted_f16(fake, fake, fake, fake, fake, 128, fake, 0, 4, 2048, 128, 16, None, 0, None) == -3
+    assert L.q4_gemv_sorted_f16(fake, fake, fake, fake, fake, 128, fake, 0, 1, 512, 128, 4, fake, 1 << 20, None) == -2   # K < 1024
+    assert L.q4_gemv_sorted_f16(fake, fake, fake, fake, fake, 128, fake, 0, 4, 8192, 128, 64, fake, 1 << 20, None) == -2  # rows do not fit in LDS
     assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, None, None, 0, 0, 0, 1.0, 0, fake, 64, 192, 128, 2, None, 0, None) == -2
     assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, None, 1, 8, 0, 1.0, 8, fake, 64, 256, 128, 2, None, 0, None) == -1
     assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, fake, 1, 12, 0, 1.0, 12, fake, 64, 256, 128, 2, None, 0, None) == -2

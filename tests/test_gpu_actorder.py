@@ -55,7 +55,8 @@ def test_sorted_layer_plan(oracle):
     assert quant_hip.sorted_layer(t["qweight"], g2, 8) is None
 
 
-@pytest.mark.parametrize("K,N,M", [(5120, 13824, 1), (5120, 13824, 16), (512, 256, 5)])
+@pytest.mark.parametrize("K,N,M", [(5120, 13824, 1), (5120, 13824, 16), (512, 256, 5), (5120, 13824, 4), (512, 256, 2),
+                                   (1408, 256, 3), (256, 128, 1)])
 def test_actorder_gemv(oracle, repack, K, N, M):
     import torch
     from alpaca_lora_4bit_amd import quant_hip
@@ -65,6 +66,34 @@ def test_actorder_gemv(oracle, repack, K, N, M):
     ref = oracle.matmul_recons(x, layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
     y = quant_hip.gemv(torch.from_numpy(x).cuda(), t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 128)
     assert rel_err(y.cpu().numpy(), ref) <= TOL
+
+
+def test_sorted_gemv_gathers_activations_in_the_kernel(oracle):
+    """Up to 4 rows: q4_gemv_sorted_f16 takes the original x and the permutation and gives the bits of the
+    sequential kernel run on x gathered beforehand; it also accumulates into y and leaves the workspace zero."""
+    import torch
+    from alpaca_lora_4bit_amd import _lib, quant_hip
+    K, N = 1408, 384                                      # 11 chunks of 128: the second workgroup of a strip is partly idle
+    layer = oracle.make_layer(K, N, 128, act_order=True, seed=9)
+    t = to_cuda_layer(layer)
+    perm, _, qsorted, gs = quant_hip.sorted_layer(t["qweight"], t["g_idx"], K // 128)
+    L = _lib.lib()
+    for M in (1, 3, 4):
+        x = torch.from_numpy(oracle.make_activations(M, K, seed=M)).cuda()
+        want = quant_hip.gemv(x.index_select(1, perm.long()).contiguous(), qsorted, t["qzeros"], t["scales"], None, gs)
+        got = quant_hip.gemv(x, t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 128)
+        assert torch.equal(got, want)
+        base = torch.randn(M, N, device="cuda").half()
+        acc = base.clone()
+        quant_hip.gemv(x, t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 128, out=acc, accumulate=True)
+        assert torch.allclose(acc.float(), base.float() + want.float(), rtol=0, atol=2e-3 * float(want.abs().max()))
+    ws = torch.zeros(L.q4_gemv_workspace_bytes(4, K, N), dtype=torch.uint8, device="cuda")
+    y = torch.empty(4, N, dtype=torch.float16, device="cuda")
+    x = torch.from_numpy(oracle.make_activations(4, K, seed=3)).cuda()
+    rc = L.q4_gemv_sorted_f16(x.data_ptr(), qsorted.data_ptr(), t["qzeros"].data_ptr(), t["scales"].data_ptr(),
+                              perm.data_ptr(), gs, y.data_ptr(), 0, 4, K, N, K // 128, ws.data_ptr(), ws.numel(), None)
+    torch.cuda.synchronize()
+    assert rc == 0 and int(ws.count_nonzero()) == 0
 
 
 @pytest.mark.parametrize("K,N,M", [(5120, 13824, 512), (512, 384, 40)])
