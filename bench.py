@@ -138,6 +138,27 @@ def bench_single_gemv(K, N, M, act_order, reps, copies, seed=3):
     return dict(us=per * 1e6, gbs=b / per / 1e9, frac_hbm=b / per / 1e9 / HBM_PEAK_GBS, bytes=b, copies=copies)
 
 
+def bench_dequant(K, N, act_order, reps, copies=6, seed=9):
+    """Dense dequantization (the reference's vecquant4recons_v2): bytes = packed layer read + fp16 matrix written."""
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    lays = [make_layer_gpu(K, N, 128, gen, act_order) for _ in range(copies)]
+    outs = [torch.empty((K, N), dtype=torch.float16, device="cuda") for _ in range(copies)]
+
+    inner = 4                                # 24 launches per graph replay: the replay cost is amortised
+
+    def step():
+        for _ in range(inner):
+            for l, o in zip(lays, outs):
+                quant_hip.dequant(l["qweight"], l["qzeros"], l["scales"], l["g_idx"], 128, out=o)
+    _, ev = time_graph(step, reps, 2)
+    per = ev / (reps * copies * inner)
+    G = lays[0]["G"]
+    b = K * N // 2 + G * N // 2 + 2 * G * N + 4 * K + 2 * K * N
+    return dict(us=per * 1e6, gbs=b / per / 1e9, frac_hbm=b / per / 1e9 / HBM_PEAK_GBS, bytes=b, copies=copies)
+
+
 def bench_lora_step(reps, seed=5):
     """Config 2: Linear4bitLt 4096->4096, r=8, alpha=16, 2048 tokens: forward + backward
     (dx, dA, dB).  138.24 GFLOP of algorithmic work per step."""
@@ -360,6 +381,8 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--llama7b-step-only", action="store_true",
                     help="run only the config-4 full-model LoRA training step (32-layer LLaMA-7B shapes, random init)")
+    ap.add_argument("--dequant-only", action="store_true",
+                    help="run only the dense dequantization of a 4096x11008 layer (short run for profiling)")
     ap.add_argument("--lora-step-only", action="store_true",
                     help="run only the config-2 LoRA layer step (forward + backward, M=2048) and print its figures: "
                          "a short run for profiling the GEMM and adapter kernels")
@@ -377,6 +400,10 @@ def main():
     if args.llama7b_step_only:
         r = bench_llama7b_lora_train_step(max(args.steps, 2))
         print(json.dumps({"workload": "config4_llama7b_lora_train_step_b4_s256", **{k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()}}))
+        return
+    if args.dequant_only:
+        r = bench_dequant(4096, 11008, False, max(args.steps, 5))
+        print(json.dumps({"workload": "dense_dequant_K4096_N11008", **{k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()}}))
         return
     if args.lora_step_only:
         r = bench_lora_step(max(args.steps, 5))
@@ -429,6 +456,10 @@ def main():
         c3g = bench_single_gemv(5120, 13824, 1, True, 10, 12)
         extra["config3_actorder_K5120_N13824_M1_gather_kernel"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in c3g.items()}
         quant_hip.actorder_repack = True
+        for (K, N, act, name) in ((4096, 11008, False, "dense_dequant_K4096_N11008"),
+                                  (5120, 13824, True, "dense_dequant_actorder_K5120_N13824")):
+            dq = bench_dequant(K, N, act, 10)
+            extra[name] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in dq.items()}
         lo = bench_lora_step(20)
         extra["config2_lora_fwd_bwd_M2048"] = {k: round(v, 4) for k, v in lo.items()}
         gm = bench_gemm_only(2048, 4096, 4096, False, 20)
