@@ -13,6 +13,7 @@ int q4_launch_gemm(int, const void*, const int32_t*, const int32_t*, const void*
                    const void*, const void*, int, int, int, float, int, void*, int, int, int, int, void*, size_t, hipStream_t);
 size_t q4_gemm_plan_workspace(int, int, int, int);
 int q4_gemv_sorted_applicable(int, int);
+int q4_launch_gemv_v1(const void*, const int32_t*, const void*, const void*, void*, int, int, int, int, void*, hipStream_t);
 int q4_launch_lora_down(const void*, const void*, int, int, int, void*, int, int, int, hipStream_t);
 int q4_launch_lora_grad(const void*, const void*, float*, int, int, float, int, int, int, void*, hipStream_t);
 size_t q4_lora_grad_workspace(int, int, int);
@@ -35,7 +36,7 @@ int check_layer(const void* qweight, const void* qzeros, const void* scales, con
 }
 }  // namespace
 
-extern "C" int q4_abi_version(void) { return 5; }
+extern "C" int q4_abi_version(void) { return 6; }
 
 extern "C" const char* q4_error_string(int code) {
     switch (code) {
@@ -121,6 +122,19 @@ extern "C" int q4_gemv_sorted_f16(const void* x, const int32_t* qweight_sorted, 
     if (M >= 1 && !q4_gemv_sorted_applicable(M, K)) return Q4_ERR_BAD_SHAPE;
     return gemv_common(x, qweight_sorted, qzeros, scales, nullptr, perm, groupsize, y, accumulate, M, 4, K, N, G, workspace,
                        workspace_bytes, stream);
+}
+
+extern "C" int q4_gemv_v1_f16(const void* x, const int32_t* qweight, const void* scales, const void* zeros, void* y,
+                              int accumulate, int M, int K, int N, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!x || !qweight || !scales || !zeros || !y) return Q4_ERR_NULL_POINTER;
+    if (M < 1 || M > 16 || K < 64 || N < 64 || (K % 32) != 0 || (N % 64) != 0 || K > 32 * 255 * 8 * 16) return Q4_ERR_BAD_SHAPE;
+    if ((long long)(K / 8) * N * 4 >= 0x70000000ll) return Q4_ERR_BAD_SHAPE;      /* 32-bit buffer offsets */
+    if (misaligned(x) || misaligned(qweight) || misaligned(y) || (reinterpret_cast<uintptr_t>(scales) & 7u) ||
+        (reinterpret_cast<uintptr_t>(zeros) & 7u))
+        return Q4_ERR_MISALIGNED;
+    if (!workspace || workspace_bytes < q4_gemv_workspace_bytes(M, K, N)) return Q4_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
+    return q4_launch_gemv_v1(x, qweight, scales, zeros, y, accumulate, M, K, N, workspace, (hipStream_t)stream);
 }
 
 static int gemm_common(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros, const void* scales,

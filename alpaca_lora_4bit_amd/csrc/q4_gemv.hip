@@ -52,6 +52,7 @@ struct GemvArgs {
     int M, K, N, G;
     unsigned long long* acc64;   // [M, N], zero between calls
     const int32_t* perm;         // gemv_seq_perm_kernel only: original index of every (sorted) reduction row
+    const half_t* v1_zeros;      // v1 layout only: fp16 zero value per column
 };
 
 __device__ __forceinline__ half8_t make_half8(uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
@@ -144,24 +145,33 @@ __device__ __forceinline__ void gemv_finish(const GemvArgs& a, const float4_t ya
 // ------------------------------------------------------------------ sequential groups
 // GSTEPS = steps of 32 rows per quantization group (1, 2, 4, 8; NSTEP % GSTEPS == 0), or
 // 0 when a whole chunk lies inside one group (groupsize % (32*NSTEP) == 0).
-template <int NSTEP, int GSTEPS>
+// V1: the older layout with one fp16 scale and one fp16 zero VALUE per column (no groups, no zero codes):
+// W = s*q - zero (quant_cuda_kernel.cu:1076-1097), so y = s * sum(x*q) - zero * sum(x).
+template <int NSTEP, int GSTEPS, bool V1 = false>
 struct SeqChunk {
     static constexpr int NG = GSTEPS == 0 ? 1 : NSTEP / GSTEPS;
     static constexpr int GS = GSTEPS == 0 ? NSTEP : GSTEPS;
+    static_assert(!V1 || GSTEPS == 0, "the v1 layout has a single group");
     uint2_t sv[NG];
     uint32_t zv[NG];
+    uint2_t zh;                                   // V1: four fp16 zeros
     uint4_t wv[NSTEP], xv[NSTEP];
 
     // scale / zero of every group of the chunk first: they are consumed last but must not sit behind the
     // weights in the in-order return queue.  The packed words are read exactly once per product: streaming
     // loads, so they do not displace the activations and scales that every strip shares from the caches.
     __device__ __forceinline__ void load_weights(const GemvArgs& a, int k0, int col, int kk) {
-        const int ncol8 = a.N >> 3;
-        const int g0 = k0 / a.groupsize;
+        if constexpr (V1) {
+            sv[0] = *reinterpret_cast<const uint2_t*>(a.scales + col);
+            zh = *reinterpret_cast<const uint2_t*>(a.v1_zeros + col);
+        } else {
+            const int ncol8 = a.N >> 3;
+            const int g0 = k0 / a.groupsize;
 #pragma unroll
-        for (int i = 0; i < NG; ++i) {
-            sv[i] = *reinterpret_cast<const uint2_t*>(a.scales + (size_t)(g0 + i) * a.N + col);
-            zv[i] = a.qzeros[(size_t)(g0 + i) * ncol8 + (col >> 3)];
+            for (int i = 0; i < NG; ++i) {
+                sv[i] = *reinterpret_cast<const uint2_t*>(a.scales + (size_t)(g0 + i) * a.N + col);
+                zv[i] = a.qzeros[(size_t)(g0 + i) * ncol8 + (col >> 3)];
+            }
         }
         const rsrc_t rw = make_rsrc(a.qweight, (unsigned)((size_t)(a.K >> 3) * a.N * 4));
         const int vw = (((k0 >> 3) + kk) * a.N + col) * 4;
@@ -229,17 +239,30 @@ struct SeqChunk {
                 accx = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, ones, accx, 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);      // consume the loads in the order they return
             }
-            // group epilogue: y += s * ((sum x*(off+q) - sum x*off) - (z+1) * sum x)
-            const uint32_t zw = zv[gi] >> ((c & 1) * 16);
             const half2_t s01 = as_half2(sv[gi].x), s23 = as_half2(sv[gi].y);
             const float sf[4] = {(float)s01[0], (float)s01[1], (float)s23[0], (float)s23[1]};
+            if constexpr (V1) {
+                // y += s * (sum x*(off+q) - sum x*off) - zero * sum x
+                const half2_t z01 = as_half2(zh.x), z23 = as_half2(zh.y);
+                const float zf[4] = {(float)z01[0], (float)z01[1], (float)z23[0], (float)z23[1]};
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                if (r < a.M) {                          // uniform: with M <= 3 the other accumulator rows are unused
+                for (int r = 0; r < 4; ++r) {
+                    if (r < a.M) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const float zf = (float)(((zw >> (4 * j)) & 0xFu) + 1u);
-                        yacc[j][r] += sf[j] * ((acc[j][r] - acco[r]) - zf * accx[r]);
+                        for (int j = 0; j < 4; ++j) yacc[j][r] += sf[j] * (acc[j][r] - acco[r]) - zf[j] * accx[r];
+                    }
+                }
+            } else {
+                // group epilogue: y += s * ((sum x*(off+q) - sum x*off) - (z+1) * sum x)
+                const uint32_t zw = zv[gi] >> ((c & 1) * 16);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (r < a.M) {                      // uniform: with M <= 3 the other accumulator rows are unused
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const float zf = (float)(((zw >> (4 * j)) & 0xFu) + 1u);
+                            yacc[j][r] += sf[j] * ((acc[j][r] - acco[r]) - zf * accx[r]);
+                        }
                     }
                 }
             }
@@ -247,7 +270,7 @@ struct SeqChunk {
     }
 };
 
-template <int NSTEP, int GSTEPS>
+template <int NSTEP, int GSTEPS, bool V1 = false>
 __global__ __launch_bounds__(NSTEP >= 16 ? 512 : 1024) void gemv_seq_kernel(GemvArgs a) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -261,7 +284,7 @@ __global__ __launch_bounds__(NSTEP >= 16 ? 512 : 1024) void gemv_seq_kernel(Gemv
     for (int j = 0; j < 4; ++j) yacc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
 
     if (k0 < a.K) {                               // wave-uniform; K % (32*NSTEP) == 0 (checked on the host)
-        SeqChunk<NSTEP, GSTEPS> ch;
+        SeqChunk<NSTEP, GSTEPS, V1> ch;
         ch.load_weights(a, k0, n0 + 4 * c, kk);
         ch.load_x(a.x + (size_t)min(c, a.M - 1) * a.K + k0 + 8 * kk);
         // Keep the burst a burst: the scheduler must not sink loads below the arithmetic.
@@ -711,6 +734,7 @@ extern "C" int q4_launch_gemv(const void* x, const int32_t* qweight, const int32
     a.M = M; a.K = K; a.N = N; a.G = G;
     a.acc64 = reinterpret_cast<unsigned long long*>(workspace);
     a.perm = perm;
+    a.v1_zeros = nullptr;
 
     const bool seq = (g_idx == nullptr);
     const GemvPlan p = plan_gemv(K, N, groupsize, seq, 4);
@@ -744,6 +768,34 @@ extern "C" int q4_launch_gemv(const void* x, const int32_t* qweight, const int32
     return hipGetLastError() == hipSuccess ? 0 : -4;
 }
 
+
+// v1 layout: scales and zeros are fp16 [N]; one group spanning K.
+extern "C" int q4_launch_gemv_v1(const void* x, const int32_t* qweight, const void* scales, const void* zeros, void* y,
+                                 int accumulate, int M, int K, int N, void* workspace, hipStream_t stream) {
+    using namespace q4;
+    GemvArgs a;
+    a.x = reinterpret_cast<const half_t*>(x);
+    a.qweight = reinterpret_cast<const uint32_t*>(qweight);
+    a.qzeros = nullptr;
+    a.scales = reinterpret_cast<const half_t*>(scales);
+    a.g_idx = nullptr;
+    a.groupsize = K;
+    a.y = reinterpret_cast<half_t*>(y);
+    a.accumulate = accumulate;
+    a.M = M; a.K = K; a.N = N; a.G = 1;
+    a.acc64 = reinterpret_cast<unsigned long long*>(workspace);
+    a.perm = nullptr;
+    a.v1_zeros = reinterpret_cast<const half_t*>(zeros);
+    const GemvPlan p = plan_gemv(K, N, K, true, 4);
+    const dim3 grid(N / kColsPerWave, p.splits), block(64 * p.waves);
+    const size_t lds = (size_t)p.waves * M * 64 * sizeof(float);
+    switch (p.nstep) {                                       // one group: gsteps is always 0
+        case 4: hipLaunchKernelGGL((gemv_seq_kernel<4, 0, true>), grid, block, lds, stream, a); break;
+        case 2: hipLaunchKernelGGL((gemv_seq_kernel<2, 0, true>), grid, block, lds, stream, a); break;
+        default: hipLaunchKernelGGL((gemv_seq_kernel<1, 0, true>), grid, block, lds, stream, a); break;
+    }
+    return hipGetLastError() == hipSuccess ? 0 : -4;
+}
 
 extern "C" int q4_launch_splitk_reduce(const float* part, void* out, long total, int splits, hipStream_t stream);
 

@@ -109,9 +109,13 @@ def _matmul4bit_v1_recons(x, qweight, scales, zeros, transpose=False):
 
 
 def _matmul4bit_v1(x, qweight, scales, zeros):
-    """matmul_utils_4bit.py:36-56: same result through the dense path (no dedicated v1 GEMV here)."""
+    """x @ W of a v1 layer for a handful of rows (matmul_utils_4bit.py:36-56); more rows than the GEMV takes go
+    through the dense path."""
     assert qweight.shape[0] * 8 == x.shape[-1]
-    return _matmul4bit_v1_recons(x, qweight, scales, zeros).to(x.dtype)
+    if int(np.prod(x.shape[:-1])) > quant_hip.MAX_GEMV_ROWS:
+        return _matmul4bit_v1_recons(x, qweight, scales, zeros).to(x.dtype)
+    outshape = x.shape[:-1] + (qweight.shape[1],)
+    return quant_hip.gemv_v1(x, qweight, scales, zeros, out_shape=outshape).to(x.dtype)
 
 
 def _matmul2bit_v2_recons(x, qweight, scales, zeros, g_idx, transpose=False):
@@ -136,7 +140,11 @@ def v2_to_v1(scales, zeros):
 def matmul4bit(x, qweight, scales, zeros, g_idx=None, groupsize=None):
     """No-grad dispatcher, matmul_utils_4bit.py:146-170."""
     if zeros.dtype != torch.int32:
-        # v1 layout (matmul_utils_4bit.py:148-156)
+        # v1 layout (matmul_utils_4bit.py:148-156): decode sizes take the GEMV, the rest dense dequant + GEMM
+        rows = int(np.prod(x.shape[:-1]))
+        thd = min(int(auto_switch_thd), quant_hip.MAX_GEMV_ROWS) if (use_new and auto_switch) else quant_hip.MAX_GEMV_ROWS
+        if 1 <= rows <= thd:
+            return _matmul4bit_v1(x, qweight, scales, zeros)
         return _matmul4bit_v1_recons(x.half(), qweight, scales.half(), zeros.half())
     gs = _groupsize_of(qweight, scales, groupsize)
     rows = int(np.prod(x.shape[:-1]))

@@ -248,6 +248,36 @@ def dequant_v1(qweight, scales, zeros, out=None):
     return out
 
 
+def gemv_v1(x, qweight, scales, zeros, out=None, accumulate=False, out_shape=None):
+    """y fp16 [M, N] = x [M, K] @ W for a v1 layer (per-column fp16 scale and zero), M <= 16: the decode product
+    of vecquant4matmul_v1_faster (quant_cuda_kernel.cu:1244-1302) with fp32 accumulation."""
+    _require(qweight.is_cuda and qweight.dtype == torch.int32 and qweight.dim() == 2 and qweight.is_contiguous(),
+             "qweight must be a contiguous int32 [K/8, N] CUDA tensor")
+    dev = qweight.device
+    K, N = qweight.shape[0] * 8, qweight.shape[1]
+    s1, z1 = scales.reshape(-1), zeros.reshape(-1)
+    _require(s1.numel() == N and z1.numel() == N and s1.device == dev and z1.device == dev,
+             "v1 scales and zeros hold one value per column")
+    s1 = (s1 if s1.dtype == torch.float16 else s1.half()).contiguous()
+    z1 = (z1 if z1.dtype == torch.float16 else z1.half()).contiguous()
+    _require(K % 32 == 0 and N % 64 == 0, "K must be a multiple of 32 and N of 64")
+    x2 = _flat_half(x, K, dev, "x")
+    M = x2.shape[0]
+    _require(1 <= M <= MAX_GEMV_ROWS, f"gemv handles 1..{MAX_GEMV_ROWS} rows, got {M}")
+    if out is None:
+        _require(not accumulate, "accumulate needs an output tensor")
+        out = torch.empty(_out_shape(out_shape, M, N), dtype=torch.float16, device=dev)
+    _require(out.dtype == torch.float16 and out.numel() == M * N and out.shape[-1] == N and out.is_contiguous()
+             and out.device == dev, "out must be a contiguous float16 [..., N] tensor with M rows on the same device")
+    L = _lib.lib()
+    with torch.cuda.device(dev):
+        ws = _workspace(dev, L.q4_gemv_workspace_bytes(M, K, N))
+        rc = L.q4_gemv_v1_f16(x2.data_ptr(), qweight.data_ptr(), s1.data_ptr(), z1.data_ptr(), out.data_ptr(),
+                              int(bool(accumulate)), M, K, N, ws.data_ptr(), ws.numel(), _stream(dev))
+    _lib.check(rc, "q4_gemv_v1_f16")
+    return out
+
+
 def dequant2(qweight, qzeros, scales, g_idx=None, groupsize=None, out=None):
     """W fp16 [K, N] of a 2-bit v2 layer (qweight [K/16, N], qzeros [G, N/16]), bit-exact with
     vecquant2recons_v2 (quant_cuda_kernel.cu:1185-1211)."""
@@ -508,14 +538,20 @@ def vecquant4matmul_old_faster(vec, mat, mul, scales, zeros, groupsize, vec_heig
     _matmul_into(vec, mat, mul, scales, zeros, None, groupsize)
 
 
+def vecquant4matmul_v1_faster(vec, mat, mul, scales, zeros):
+    """quant_cuda.vecquant4matmul_v1_faster (quant_cuda.cpp:163-175): mul += vec @ W for a v1 layer."""
+    mul.add_(gemv_v1(vec, mat, scales, zeros).to(mul.dtype))
+
+
 def _unsupported(name):
     def fn(*args, **kwargs):
         raise NotImplementedError(f"{name}: not built for gfx950 (4-bit v2 runs fused; v1 and 2-bit v2 run through "
-                                  "vecquant4recons_v1 / vecquant2recons_v2 + a dense GEMM)")
+                                  "vecquant4recons_v1 / vecquant2recons_v2 + a dense GEMM, v1 decode through "
+                                  "vecquant4matmul_v1_faster)")
     fn.__name__ = name
     return fn
 
 
 for _n in ("vecquant2matmul", "vecquant3matmul", "vecquant8matmul", "vecquant2matmul_faster", "vecquant3matmul_faster",
-           "vecquant4matmul_v1_faster", "vecquant4matmul_seq_v2", "vecquant4matmul_g"):
+           "vecquant4matmul_seq_v2", "vecquant4matmul_g"):
     globals()[_n] = _unsupported(_n)

@@ -91,6 +91,15 @@ int q4_gemv_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, co
  * kernel gathers x[:, perm[p]] itself (through LDS) while its weight loads are in flight, which replaces the separate gather
  * the caller would otherwise run before q4_gemv_f16.  The values are those of the reference's act-order
  * product (quant_cuda_kernel.cu:443-536 with per-row g_idx).  Workspace as for q4_gemv_f16. */
+/* The same product for the v1 layout (one fp16 scale and one fp16 zero value per column, W = s*q - zero):
+ *   y fp16 [M, N] = x fp16 [M, K] @ W,  1 <= M <= 16.
+ * Replaces quant_cuda.vecquant4matmul_v1_faster (quant_cuda/quant_cuda.cpp:163-175; kernel
+ * quant_cuda_kernel.cu:1244-1302, launcher :1304-1335) as called from matmul_utils_4bit.py:36-56.  `scales`, `zeros` fp16 [N],
+ * 8-byte aligned.  Workspace as for q4_gemv_f16. */
+int q4_gemv_v1_f16(const void *x, const int32_t *qweight, const void *scales, const void *zeros, void *y,
+                   int accumulate, int M, int K, int N,
+                   void *workspace, size_t workspace_bytes, void *stream);
+
 int q4_gemv_sorted_f16(const void *x, const int32_t *qweight_sorted, const int32_t *qzeros, const void *scales,
                        const int32_t *perm, int groupsize, void *y, int accumulate,
                        int M, int K, int N, int G,

@@ -67,6 +67,11 @@ def test_error_codes_and_validation_need_no_gpu():
     assert L.q4_gemm_workspace_bytes(0, 64, 4096, 11008) == 8 * 64 * 4096 * 4
     # older layouts (dense dequantization only)
     assert L.q4_dequant_v1_f16(fake, fake, None, fake, 256, 128, None) == -1
+    assert L.q4_gemv_v1_f16(fake, fake, fake, None, fake, 0, 1, 256, 128, fake, 1 << 20, None) == -1
+    assert L.q4_gemv_v1_f16(fake, fake, fake, fake, fake, 0, 17, 256, 128, fake, 1 << 20, None) == -2
+    assert L.q4_gemv_v1_f16(fake, fake, fake, fake, fake, 0, 1, 250, 128, fake, 1 << 20, None) == -2
+    assert L.q4_gemv_v1_f16(fake, fake, fake, fake, fake, 0, 1, 256, 128, None, 0, None) == -3
+    assert L.q4_gemv_v1_f16(fake, fake, fake, ctypes.c_void_p(0x1004), fake, 0, 1, 256, 128, fake, 1 << 20, None) == -5
     assert L.q4_dequant_v1_f16(fake, fake, fake, fake, 250, 128, None) == -2
     assert L.q4_dequant2_f16(fake, fake, fake, None, 128, fake, 264, 128, 3, None) == -2     # K % 16
     assert L.q4_dequant2_f16(fake, fake, fake, None, 128, odd, 256, 128, 2, None) == -5
@@ -171,6 +176,7 @@ def test_quant_cuda_mirror_exports_the_pybind_names():
         assert callable(getattr(quant_hip, name)), name
     with pytest.raises(NotImplementedError):
         quant_hip.vecquant2matmul()
+    assert list(inspect.signature(quant_hip.vecquant4matmul_v1_faster).parameters) == ["vec", "mat", "mul", "scales", "zeros"]
     assert list(inspect.signature(quant_hip.vecquant4recons_v1).parameters) == ["mat", "res", "scales", "zeros"]
     assert list(inspect.signature(quant_hip.vecquant2recons_v2).parameters) == ["mat", "res", "scales", "zeros", "g_idx"]
     assert list(inspect.signature(quant_hip.vecquant4recons_v2).parameters) == ["mat", "res", "scales", "zeros", "g_idx"]

@@ -40,6 +40,31 @@ def test_dequant_v1_bit_exact(oracle, K, N):
     assert torch.equal(res, got)
 
 
+@pytest.mark.parametrize("K,N", [(4096, 4096), (512, 256), (1408, 192), (64, 64)])
+@pytest.mark.parametrize("M", [1, 5, 16])
+def test_gemv_v1(oracle, K, N, M):
+    """Decode product of a v1 layer (the reference's vecquant4matmul_v1_faster): within 1e-2 of the fp32 product
+    with the bit-exact dense W; accumulates into y on request; the pybind-style wrapper adds into `mul`."""
+    from alpaca_lora_4bit_amd import quant_hip
+    qw, s, z = _v1_layer(oracle, K, N, K + N + M)
+    t = lambda a: torch.from_numpy(a).cuda()
+    W = oracle.dequant_v1(qw, s, z).astype(np.float32)
+    x = oracle.make_activations(M, K, seed=M)
+    ref = x.astype(np.float32) @ W
+    y = quant_hip.gemv_v1(t(x), t(qw), t(s), t(z))
+    assert y.shape == (M, N) and y.dtype == torch.float16
+    assert np.abs(y.float().cpu().numpy() - ref).max() <= 1e-2 * np.abs(ref).max()
+    assert np.abs(y.float().cpu().numpy() - ref).max() <= 2e-3 * np.abs(ref).max()
+    assert torch.equal(quant_hip.gemv_v1(t(x), t(qw), t(s), t(z)), y)              # reproducible
+    base = torch.randn(M, N, device="cuda").half()
+    acc = base.clone()
+    quant_hip.gemv_v1(t(x), t(qw), t(s), t(z), out=acc, accumulate=True)
+    assert torch.allclose(acc.float(), base.float() + y.float(), rtol=0, atol=2e-3 * float(np.abs(ref).max()) + 2e-3)
+    mul = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    quant_hip.vecquant4matmul_v1_faster(t(x), t(qw), mul, t(s), t(z))
+    assert torch.equal(mul, y)
+
+
 @pytest.mark.parametrize("K,N,gs,act", [(256, 128, 128, False), (4096, 1024, 128, False), (512, 192, 64, True),
                                         (272, 64, 16, True)])
 def test_dequant2_bit_exact(oracle, K, N, gs, act):
@@ -70,9 +95,12 @@ def test_v1_module_forward_backward(oracle, rows):
     ref_y, ref_dx = x.astype(np.float32) @ W, dy.astype(np.float32) @ W.T
     assert np.abs(y.detach().float().cpu().numpy() - ref_y).max() <= 1e-2 * np.abs(ref_y).max()
     assert np.abs(xd.grad.float().cpu().numpy() - ref_dx).max() <= 1e-2 * np.abs(ref_dx).max()
-    with torch.no_grad():                                   # the no-grad dispatcher takes the same route
+    with torch.no_grad():                                   # no-grad dispatcher: the v1 GEMV for a few rows, else the same route
         y2 = m(torch.from_numpy(x).cuda())
-    assert torch.equal(y2, y.detach())
+    if rows > 8:
+        assert torch.equal(y2, y.detach())
+    else:
+        assert np.abs(y2.float().cpu().numpy() - ref_y).max() <= 1e-2 * np.abs(ref_y).max()
 
 
 def test_2bit_module_forward_backward(oracle):
