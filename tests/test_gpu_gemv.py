@@ -103,3 +103,36 @@ def test_gemv_accumulate_flag(oracle):
     quant_hip.gemv(torch.from_numpy(x).cuda(), t["qweight"], t["qzeros"], t["scales"], None, 128, out=base,
                    accumulate=True)
     assert rel_err(base.cpu().numpy(), ref + 1.5) <= TOL
+
+
+def test_two_streams_and_two_threads_use_separate_workspaces(oracle):
+    """The split-K accumulators (GEMV) and partial-sum scratch (GEMM) are cached per stream: products launched
+    concurrently on two streams, from two Python threads, give the bits of the same products run one by one."""
+    import threading
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    layers = [to_cuda_layer(oracle.make_layer(4096, 2048, 128, seed=50 + i)) for i in range(2)]
+    xs = [torch.from_numpy(oracle.make_activations(m, 4096, seed=60 + i)).cuda() for i, m in enumerate((1, 16))]
+    xg = [torch.from_numpy(oracle.make_activations(40, 4096, seed=70 + i)).cuda() for i in range(2)]
+    want = [quant_hip.gemv(x, t["qweight"], t["qzeros"], t["scales"], None, 128) for x, t in zip(xs, layers)]
+    want_g = [quant_hip.gemm_fwd(x, t["qweight"], t["qzeros"], t["scales"], None, 128) for x, t in zip(xg, layers)]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    got = [[None] * 30, [None] * 30]
+    got_g = [[None] * 30, [None] * 30]
+
+    def work(i):
+        with torch.cuda.stream(streams[i]):
+            for r in range(30):
+                got[i][r] = quant_hip.gemv(xs[i], layers[i]["qweight"], layers[i]["qzeros"], layers[i]["scales"], None, 128)
+                got_g[i][r] = quant_hip.gemm_fwd(xg[i], layers[i]["qweight"], layers[i]["qzeros"], layers[i]["scales"],
+                                                 None, 128)
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    torch.cuda.synchronize()
+    for i in range(2):
+        assert all(torch.equal(y, want[i]) for y in got[i])
+        assert all(torch.equal(y, want_g[i]) for y in got_g[i])
