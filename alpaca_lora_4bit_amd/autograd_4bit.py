@@ -135,6 +135,24 @@ def matmul4bit_with_backend(x, qweight, scales, qzeros, g_idx, bits, maxq, group
     raise ValueError('Backend not supported.')
 
 
+def _is_all_zero(bias):
+    """True when `bias` holds only zeros, which is what checkpoints without biases leave in the buffer
+    (autograd_4bit.py:186): the in-place add of the reference's forward (:207-208) is then skipped.  The verdict
+    is kept on the tensor object with its in-place version counter; the first call per tensor synchronises."""
+    key = (bias._version, bias.data_ptr())
+    cached = getattr(bias, "_q4_zero", None)
+    if cached is not None and cached[0] == key:
+        return cached[1]
+    if torch.cuda.is_available() and bias.is_cuda and torch.cuda.is_current_stream_capturing():
+        return False                  # no synchronising reduction inside a graph capture: keep the add
+    verdict = not bool(bias.any())
+    try:
+        bias._q4_zero = (key, verdict)
+    except AttributeError:
+        pass
+    return verdict
+
+
 class Autograd4bitQuantLinear(nn.Module):
     """GPTQ 4-bit linear layer; buffers as registered at autograd_4bit.py:166-189."""
 
@@ -172,7 +190,7 @@ class Autograd4bitQuantLinear(nn.Module):
             out = AutogradMatmul2bit.apply(x, self.qweight, self.scales, self.qzeros, self.g_idx, self.bits, self.maxq)
         else:
             raise ValueError('Unsupported bitwidth.')
-        if not self.disable_bias:
+        if not self.disable_bias and not _is_all_zero(self.bias):
             out += self.bias
         return out
 

@@ -49,6 +49,11 @@ def get_buffer(shape_of_qweight, dtype=torch.float16, device='cuda', bits=4):
     return buf
 
 
+def _rows(x):
+    """Number of rows of x seen as a matrix [rows, K] (np.prod(x.shape[:-1]) of the reference)."""
+    return x.numel() // x.shape[-1] if x.shape[-1] else 0
+
+
 def _groupsize_of(qweight, scales, groupsize):
     if groupsize is not None and groupsize > 0:
         return int(groupsize)
@@ -112,7 +117,7 @@ def _matmul4bit_v1(x, qweight, scales, zeros):
     """x @ W of a v1 layer for a handful of rows (matmul_utils_4bit.py:36-56); more rows than the GEMV takes go
     through the dense path."""
     assert qweight.shape[0] * 8 == x.shape[-1]
-    if int(np.prod(x.shape[:-1])) > quant_hip.MAX_GEMV_ROWS:
+    if _rows(x) > quant_hip.MAX_GEMV_ROWS:
         return _matmul4bit_v1_recons(x, qweight, scales, zeros).to(x.dtype)
     outshape = x.shape[:-1] + (qweight.shape[1],)
     return quant_hip.gemv_v1(x, qweight, scales, zeros, out_shape=outshape).to(x.dtype)
@@ -141,13 +146,13 @@ def matmul4bit(x, qweight, scales, zeros, g_idx=None, groupsize=None):
     """No-grad dispatcher, matmul_utils_4bit.py:146-170."""
     if zeros.dtype != torch.int32:
         # v1 layout (matmul_utils_4bit.py:148-156): decode sizes take the GEMV, the rest dense dequant + GEMM
-        rows = int(np.prod(x.shape[:-1]))
+        rows = _rows(x)
         thd = min(int(auto_switch_thd), quant_hip.MAX_GEMV_ROWS) if (use_new and auto_switch) else quant_hip.MAX_GEMV_ROWS
         if 1 <= rows <= thd:
             return _matmul4bit_v1(x, qweight, scales, zeros)
         return _matmul4bit_v1_recons(x.half(), qweight, scales.half(), zeros.half())
     gs = _groupsize_of(qweight, scales, groupsize)
-    rows = int(np.prod(x.shape[:-1]))
+    rows = _rows(x)
     thd = min(int(auto_switch_thd), quant_hip.MAX_GEMV_ROWS)
     use_gemv = rows <= thd if (use_new and auto_switch) else rows <= quant_hip.MAX_GEMV_ROWS
     if use_gemv and rows >= 1:

@@ -37,8 +37,32 @@ def _ptr(t):
     return 0 if t is None else t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device) -> int:
+    """Handle of torch's current stream on `device` (the raw getter skips building a Stream object per call)."""
+    if _raw_stream is not None:
+        return _raw_stream(device.index if device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _device_ctx(device):
+    """Context that makes `device` current for a launch; free when it already is (the usual case)."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(device)
 
 
 def _require(cond, msg):
@@ -47,6 +71,22 @@ def _require(cond, msg):
 
 
 def _check_layer(qweight, qzeros, scales, g_idx, groupsize):
+    """Validates a layer's tensors against each other; returns (device, K, N, G).  The verdict is kept on the
+    qweight tensor object and reused while the same tensor objects (same storage, same dtypes) come back."""
+    key = (id(qzeros), id(scales), id(g_idx), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), scales.dtype,
+           None if g_idx is None else g_idx.data_ptr(), groupsize if g_idx is None else None)
+    cached = getattr(qweight, "_q4_layer", None)
+    if cached is not None and cached[0] == key:
+        return cached[1]
+    result = _check_layer_uncached(qweight, qzeros, scales, g_idx, groupsize)
+    try:
+        qweight._q4_layer = (key, result)
+    except AttributeError:          # tensor subclasses without a __dict__
+        pass
+    return result
+
+
+def _check_layer_uncached(qweight, qzeros, scales, g_idx, groupsize):
     _require(qweight.is_cuda, "qweight must be on the GPU")
     dev = qweight.device
     _require(qweight.dtype == torch.int32 and qweight.dim() == 2, "qweight must be int32 [K/8, N]")
@@ -128,7 +168,7 @@ def sorted_layer(qweight, g_idx, G):
             inv = torch.empty_like(perm)
             inv[perm.long()] = torch.arange(K, device=perm.device, dtype=torch.int32)
             qs = torch.empty_like(qweight)
-            with torch.cuda.device(qweight.device):
+            with _device_ctx(qweight.device):
                 rc = _lib.lib().q4_permute_rows(qweight.data_ptr(), perm.data_ptr(), qs.data_ptr(), K, N,
                                                 _stream(qweight.device))
             _lib.check(rc, "q4_permute_rows")
@@ -215,7 +255,7 @@ def dequant(qweight, qzeros, scales, g_idx=None, groupsize=None, out=None):
     _require(out.dtype == torch.float16 and tuple(out.shape) == (K, N) and out.is_contiguous() and out.device == dev,
              "out must be a contiguous float16 [K, N] tensor on the same device")
     gp, gs = _gidx_arg(g_idx, groupsize, G, need_multiple=8)
-    with torch.cuda.device(dev):
+    with _device_ctx(dev):
         rc = _lib.lib().q4_dequant_f16(qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), gp, gs,
                                        out.data_ptr(), K, N, G, _stream(dev))
     _lib.check(rc, "q4_dequant_f16")
@@ -241,7 +281,7 @@ def dequant_v1(qweight, scales, zeros, out=None):
         out = torch.empty((K, N), dtype=torch.float16, device=dev)
     _require(out.dtype == torch.float16 and tuple(out.shape) == (K, N) and out.is_contiguous() and out.device == dev,
              "out must be a contiguous float16 [K, N] tensor on the same device")
-    with torch.cuda.device(dev):
+    with _device_ctx(dev):
         rc = _lib.lib().q4_dequant_v1_f16(qweight.data_ptr(), s1.data_ptr(), z1.data_ptr(), out.data_ptr(), K, N,
                                           _stream(dev))
     _lib.check(rc, "q4_dequant_v1_f16")
@@ -270,7 +310,7 @@ def gemv_v1(x, qweight, scales, zeros, out=None, accumulate=False, out_shape=Non
     _require(out.dtype == torch.float16 and out.numel() == M * N and out.shape[-1] == N and out.is_contiguous()
              and out.device == dev, "out must be a contiguous float16 [..., N] tensor with M rows on the same device")
     L = _lib.lib()
-    with torch.cuda.device(dev):
+    with _device_ctx(dev):
         ws = _workspace(dev, L.q4_gemv_workspace_bytes(M, K, N))
         rc = L.q4_gemv_v1_f16(x2.data_ptr(), qweight.data_ptr(), s1.data_ptr(), z1.data_ptr(), out.data_ptr(),
                               int(bool(accumulate)), M, K, N, ws.data_ptr(), ws.numel(), _stream(dev))
@@ -299,7 +339,7 @@ def dequant2(qweight, qzeros, scales, g_idx=None, groupsize=None, out=None):
         out = torch.empty((K, N), dtype=torch.float16, device=dev)
     _require(out.dtype == torch.float16 and tuple(out.shape) == (K, N) and out.is_contiguous() and out.device == dev,
              "out must be a contiguous float16 [K, N] tensor on the same device")
-    with torch.cuda.device(dev):
+    with _device_ctx(dev):
         rc = _lib.lib().q4_dequant2_f16(qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), gp, gs,
                                         out.data_ptr(), K, N, G, _stream(dev))
     _lib.check(rc, "q4_dequant2_f16")
@@ -324,7 +364,7 @@ def gemv(x, qweight, qzeros, scales, g_idx=None, groupsize=None, out=None, accum
     if plan is not None and M <= MAX_GEMV_SORTED_ROWS and K >= 1024 and M * (2 * K + 4096) <= 65536:     # rows fit in LDS
         # sorted copy of the packed rows; the kernel gathers x through the permutation itself
         perm, _, qweight, gs_sorted = plan
-        with torch.cuda.device(dev):
+        with _device_ctx(dev):
             ws = _workspace(dev, nbytes)
             rc = L.q4_gemv_sorted_f16(x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
                                       perm.data_ptr(), gs_sorted, out.data_ptr(), int(bool(accumulate)), M, K, N, G,
@@ -337,7 +377,7 @@ def gemv(x, qweight, qzeros, scales, g_idx=None, groupsize=None, out=None, accum
         gp, gs = 0, gs_sorted
     else:
         gp, gs = _gidx_arg(g_idx, groupsize, G)
-    with torch.cuda.device(dev):
+    with _device_ctx(dev):
         ws = _workspace(dev, nbytes)
         rc = L.q4_gemv_f16(x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), gp, gs,
                            out.data_ptr(), int(bool(accumulate)), M, K, N, G, ws.data_ptr(), ws.numel(), _stream(dev))
@@ -386,7 +426,7 @@ def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, 
         gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
     out = torch.empty(_out_shape(out_shape, M, N), dtype=torch.float16, device=dev)
     L = _lib.lib()
-    with torch.cuda.device(dev):
+    with _device_ctx(dev):
         wp, wn = _gemm_scratch(L, dev, 1, M, K, N)
         rc = L.q4_gemm_fwd_f16(x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
                                gp, gs, _ptr(bias), _ptr(xa), _ptr(lora_bt), sr, sc, f32, float(lora_scale), R,
@@ -412,7 +452,7 @@ def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=Non
     gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
     out = torch.empty(_out_shape(out_shape, M, K), dtype=torch.float16, device=dev)
     L = _lib.lib()
-    with torch.cuda.device(dev):
+    with _device_ctx(dev):
         wp, wn = _gemm_scratch(L, dev, 0, M, K, N)
         rc = L.q4_gemm_bwd_dx_f16(dy2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
                                   gp, gs, _ptr(dyb), _ptr(lora_a), sr, sc, f32, float(lora_scale), R,
@@ -437,7 +477,7 @@ def lora_down(inp, w):
     sr, sc = w.stride()
     _require(sr >= 1 and sc >= 1, "w must have positive strides")
     out = torch.empty((M, R), dtype=torch.float16, device=inp.device)
-    with torch.cuda.device(inp.device):
+    with _device_ctx(inp.device):
         rc = _lib.lib().q4_lora_down_f16(inp.data_ptr(), w.data_ptr(), int(sr), int(sc), f32, out.data_ptr(),
                                          M, C, R, _stream(inp.device))
     _lib.check(rc, "q4_lora_down_f16")
@@ -463,7 +503,7 @@ def lora_grad(p, inp, alpha, transposed=False):
         sr, sc = C, 1
     L = _lib.lib()
     nbytes = L.q4_lora_grad_workspace_bytes(M, C, R)
-    with torch.cuda.device(dev):
+    with _device_ctx(dev):
         ws = _scratch(dev, nbytes)
         rc = L.q4_lora_grad_f32(p.data_ptr(), inp.data_ptr(), out.data_ptr(), sr, sc, float(alpha), M, C, R,
                                 ws.data_ptr(), ws.numel(), _stream(dev))
