@@ -134,8 +134,47 @@ class Linear4bitLt(Autograd4bitQuantLinear, LoraLayer):
             return None
         return name
 
+    def _decode_adapter(self, x):
+        """Name of the single adapter for the short no-grad path (a handful of rows, eval mode), else None."""
+        if torch.is_grad_enabled() or not fuse_lora or not x.is_cuda or self.bits != 4:
+            return None
+        if x.numel() // x.shape[-1] > autograd_4bit.quant_hip.MAX_GEMV_ROWS:
+            return None
+        active = [a for a in self.active_adapters if a in self.lora_A.keys()]
+        if len(active) != 1:
+            return None
+        name = active[0]
+        r = self.lora_A[name].weight.shape[0]
+        drop = self.lora_dropout[name]
+        if r < 1 or r > 64 or self.in_features % 32 or (isinstance(drop, nn.Dropout) and drop.p > 0.0 and self.training):
+            return None
+        return name
+
+    def _half_lora_b(self, name):
+        """fp16 [r, N] copy of lora_B.weight for the rank-r update, rebuilt when the parameter changes."""
+        w = self.lora_B[name].weight
+        key = (w._version, w.data_ptr(), w.dtype)
+        cached = self.__dict__.get("_q4_lora_b16")
+        if cached is None or cached[0] != key:
+            cached = (key, w.detach().t().to(torch.float16).contiguous())
+            self.__dict__["_q4_lora_b16"] = cached
+        return cached[1]
+
     def forward(self, x: torch.Tensor):
         if not self.disable_adapters:
+            name = self._decode_adapter(x)
+            if name is not None:
+                # decode: base product (GEMV), x @ A^T with the adapter read in place, one rank-r update in place:
+                # three launches instead of the seven of the composition below, same values up to fp16 rounding
+                result = Autograd4bitQuantLinear.forward(self, x)
+                xa = autograd_4bit.quant_hip.lora_down(x.reshape(-1, x.shape[-1]).to(torch.float16),
+                                                       self.lora_A[name].weight)
+                out2 = result.view(-1, result.shape[-1])
+                if out2.dtype == torch.float16:
+                    out2.addmm_(xa, self._half_lora_b(name), alpha=float(self.scaling[name]))
+                else:
+                    out2.add_((xa @ self._half_lora_b(name)).to(out2.dtype), alpha=float(self.scaling[name]))
+                return result
             name = self._fusable_adapter(x)
             if name is not None:
                 bias = None

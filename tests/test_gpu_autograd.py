@@ -155,6 +155,48 @@ def test_fused_and_unfused_lora_agree(oracle):
         assert rel_err(a, b) <= TOL
 
 
+@pytest.mark.parametrize("rows", [1, 7, 16])
+@pytest.mark.parametrize("wdtype", ["float32", "float16"])
+def test_lora_layer_decode_path_matches_the_composition(oracle, rows, wdtype):
+    """No-grad forward with a handful of rows: base GEMV + in-place rank-r update (three launches) gives the values
+    of the reference's composition result + lora_B(lora_A(x)) * scaling (models.py:51-69), also after the adapter
+    weights change and with a bias."""
+    import torch
+    from alpaca_lora_4bit_amd import models
+    K, N, r = 512, 384, 8
+    layer = oracle.make_layer(K, N, 128, seed=31)
+    A, B = oracle.make_lora(K, N, r, seed=31)
+    m = models.Linear4bitLt("default", K, N, 128, False, r=r, lora_alpha=16).cuda().eval()
+    _fill(m, layer)
+    dt = getattr(torch, wdtype)
+    m.lora_A["default"].weight.data = torch.from_numpy(A).cuda().to(dt)
+    m.lora_B["default"].weight.data = torch.from_numpy(B).cuda().to(dt)
+    m.bias = torch.from_numpy((np.random.default_rng(5).standard_normal(N) * 0.1).astype(np.float16)).cuda()
+    x = torch.from_numpy(oracle.make_activations(rows, K, seed=rows)).cuda().reshape(1, rows, K)
+    W = oracle.dequant_v2(layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"]).astype(np.float64)
+
+    def reference():
+        a = m.lora_A["default"].weight.detach().double().cpu().numpy()
+        b = m.lora_B["default"].weight.detach().double().cpu().numpy()
+        xd = x.double().cpu().numpy().reshape(rows, K)
+        return xd @ W + m.bias.double().cpu().numpy() + 2.0 * (xd @ a.T) @ b.T
+
+    with torch.no_grad():
+        y = m(x)
+        assert y.shape == (1, rows, N) and y.dtype == torch.float16
+        assert rel_err(y.reshape(rows, N).cpu().numpy(), reference()) <= TOL
+        models.fuse_lora = False
+        try:
+            y_comp = m(x)
+        finally:
+            models.fuse_lora = True
+        assert rel_err(y.cpu().numpy().reshape(rows, N), y_comp.float().cpu().numpy().reshape(rows, N)) <= 2e-3
+        m.lora_B["default"].weight.mul_(3.0)                # in-place change: the cached fp16 copy must follow
+        y2 = m(x)
+        assert rel_err(y2.reshape(rows, N).cpu().numpy(), reference()) <= TOL
+        assert not torch.equal(y2, y)
+
+
 def test_fuse_quant_linears_matches_separate_layers(oracle):
     """gate/up (or q/k/v) concatenated along N: one launch, same numbers."""
     import torch
