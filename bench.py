@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the 4-bit GPTQ dequant-matmul path on one MI355X.
 
-Headline workload (BASELINE.json configs[1]): LLaMA-7B MLP decode GEMVs at M=1 -- gate and up
+Headline workload (configs[1] of the benchmark definition): LLaMA-7B MLP decode GEMVs at M=1 -- gate and up
 4096->11008, down 11008->4096, groupsize 128, no act-order.  One STEP = one token through the
 MLP GEMVs of all 32 decoder layers (96 launches over 2.25 GB of DISTINCT packed weights, so
 nothing is served from the 256 MB Infinity Cache, exactly as in a real decode).  The step is
@@ -229,7 +229,7 @@ def bench_lora_step(reps, seed=5):
 
 
 def bench_llama7b_lora_train_step(reps=4, seed=11, n_layers=32, batch=4, seq=256):
-    """BASELINE configs[4]: random-init 32-layer LLaMA-7B decoder, every q/k/v/o/gate/up/down projection a 4-bit
+    """configs[4] of the benchmark definition: random-init 32-layer LLaMA-7B decoder, every q/k/v/o/gate/up/down projection a 4-bit
     GPTQ layer (groupsize 128), LoRA r=8 alpha=16 on q_proj / v_proj, one forward + backward + AdamW step on
     batch 4 x seq 256 random token ids under fp16 autocast, gradient checkpointing off.  Eager PyTorch around
     the HIP kernels (attention = torch SDPA, lm_head = library GEMM)."""
