@@ -18,7 +18,7 @@ def _run(layer, use_gidx=True):
 
 @pytest.mark.parametrize("K,N,gs,act", [
     (256, 128, 128, False), (256, 128, 128, True), (64, 64, 32, False), (512, 192, 64, True),
-    (4096, 4096, 128, False),          # BASELINE config 0
+    (4096, 4096, 128, False),          # benchmark config 0
     (4096, 11008, 128, False),         # config 1 gate/up
     (11008, 4096, 128, False),         # config 1 down
     (5120, 13824, 128, True),          # config 3 act-order

@@ -60,7 +60,7 @@ def test_gemv_repeatable_and_workspace_left_clean(oracle):
 
 
 def test_gemv_linearity_full_size(oracle):
-    """Size-independent property at a BASELINE shape: (a*x1 + x2) @ W == a*(x1 @ W) + x2 @ W."""
+    """Size-independent property at a full benchmark shape: (a*x1 + x2) @ W == a*(x1 @ W) + x2 @ W."""
     layer = oracle.make_layer(4096, 11008, 128, seed=4)
     x1 = oracle.make_activations(1, 4096, seed=21)
     x2 = oracle.make_activations(1, 4096, seed=22)
