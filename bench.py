@@ -24,8 +24,8 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, GB/s
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
-# HBM bytes per launch of the headline GEMV kernel, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# scaled by a 256 MiB copy (profiles/gemv_seq_mlp_decode_M1_hbm_traffic.md): 23 571 KiB read + 432 KiB written.
+# HBM bytes per launch of the headline GEMV kernel, measured in two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE),
+# each scaled by what the same counter reads for a 256 MiB copy (--calibrate-copy): 23 571 KiB read + 432 KiB written.
 GEMV_TRAFFIC_BYTES = 24578000
 
 
