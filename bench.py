@@ -25,8 +25,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, GB/s
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 # HBM bytes per launch of the headline GEMV kernel, measured in two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE),
-# each scaled by what the same counter reads for a 256 MiB copy (--calibrate-copy): 23 571 KiB read + 432 KiB written.
-GEMV_TRAFFIC_BYTES = 24578000
+# each scaled by what the same counter reads for a 256 MiB copy (--calibrate-copy): 23 587 KiB read + 432 KiB written.
+GEMV_TRAFFIC_BYTES = 24594000
 
 
 def gemv_bytes(M, K, N, G, act_order=False):
@@ -438,7 +438,7 @@ def main():
         "pct_of_hbm_peak": round(100 * head["gbs_wall"] / HBM_PEAK_GBS, 2),
         "roofline": {"bound": "hbm", "achieved": round(head["gbs_kernel"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(head["gbs_kernel"] / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES,
-                     "kernel": "q4::gemv_seq_kernel<4, 0>", "bytes_per_launch": head["bytes_per_launch"],
+                     "kernel": "q4::gemv_seq_kernel<4, 0, false>", "bytes_per_launch": head["bytes_per_launch"],
                      "avg_launch_us": round(head["avg_launch_us"], 3)},
     }
     if not args.no_extra:
