@@ -6,7 +6,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libq4gptq.so")
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _lib = None
 
@@ -29,6 +29,7 @@ SIGNATURES = {
     "q4_lora_down_f16": (_i, [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp]),
     "q4_lora_grad_workspace_bytes": (_sz, [_i, _i, _i]),
     "q4_lora_grad_f32": (_i, [_vp, _vp, _vp, _i, _i, _f, _i, _i, _i, _vp, _sz, _vp]),
+    "q4_lora_grad_pair_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _vp, _sz, _vp]),
 }
 
 

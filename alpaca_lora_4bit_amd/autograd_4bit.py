@@ -322,17 +322,23 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
                                        lora_scale=ctx.scaling,
                                        out_shape=tuple(grad_output.shape[:-1]) + (qweight.shape[0] * 8,))
         r = a.shape[0]
-        if ctx.needs_input_grad[6]:
-            if r in quant_hip.LORA_GRAD_RANKS:
-                da = quant_hip.lora_grad(dyb, x2, ctx.scaling)
-            else:
-                da = torch.mm(dyb.t(), x2).float().mul_(ctx.scaling)
+        need_a, need_b = ctx.needs_input_grad[6], ctx.needs_input_grad[7]
+        if need_a and need_b and r in quant_hip.LORA_GRAD_RANKS:
+            da, db = quant_hip.lora_grad_pair(dyb, x2, xa, dy, ctx.scaling)      # one launch for both gradients
+        else:
+            if need_a:
+                if r in quant_hip.LORA_GRAD_RANKS:
+                    da = quant_hip.lora_grad(dyb, x2, ctx.scaling)
+                else:
+                    da = torch.mm(dyb.t(), x2).float().mul_(ctx.scaling)
+            if need_b:
+                if r in quant_hip.LORA_GRAD_RANKS:
+                    db = quant_hip.lora_grad(xa, dy, ctx.scaling, transposed=True)
+                else:
+                    db = torch.mm(dy.t(), xa).float().mul_(ctx.scaling)
+        if da is not None:
             da = da.to(ctx.ab_dtypes[0])
-        if ctx.needs_input_grad[7]:
-            if r in quant_hip.LORA_GRAD_RANKS:
-                db = quant_hip.lora_grad(xa, dy, ctx.scaling, transposed=True)
-            else:
-                db = torch.mm(dy.t(), xa).float().mul_(ctx.scaling)
+        if db is not None:
             db = db.to(ctx.ab_dtypes[1])
         return dx, None, None, None, None, None, da, db, None, None
 

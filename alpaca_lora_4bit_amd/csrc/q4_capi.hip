@@ -16,6 +16,8 @@ int q4_gemv_sorted_applicable(int, int);
 int q4_launch_gemv_v1(const void*, const int32_t*, const void*, const void*, void*, int, int, int, int, void*, hipStream_t);
 int q4_launch_lora_down(const void*, const void*, int, int, int, void*, int, int, int, hipStream_t);
 int q4_launch_lora_grad(const void*, const void*, float*, int, int, float, int, int, int, void*, hipStream_t);
+int q4_launch_lora_grad_pair(const void*, const void*, float*, int, int, int, const void*, const void*, float*, int, int, int,
+                             float, int, int, void*, hipStream_t);
 size_t q4_lora_grad_workspace(int, int, int);
 }
 
@@ -36,7 +38,7 @@ int check_layer(const void* qweight, const void* qzeros, const void* scales, con
 }
 }  // namespace
 
-extern "C" int q4_abi_version(void) { return 6; }
+extern "C" int q4_abi_version(void) { return 7; }
 
 extern "C" const char* q4_error_string(int code) {
     switch (code) {
@@ -211,4 +213,27 @@ extern "C" int q4_lora_grad_f32(const void* p, const void* in, float* out, int o
         if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
     }
     return q4_launch_lora_grad(p, in, out, o_sr, o_sc, alpha, M, C, R, workspace, (hipStream_t)stream);
+}
+
+extern "C" int q4_lora_grad_pair_f32(const void* p1, const void* in1, float* out1, int o1_sr, int o1_sc, int C1,
+                                     const void* p2, const void* in2, float* out2, int o2_sr, int o2_sc, int C2,
+                                     float alpha, int M, int R, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!p1 || !in1 || !out1 || !p2 || !in2 || !out2) return Q4_ERR_NULL_POINTER;
+    if (M < 1 || (R != 8 && R != 16)) return Q4_ERR_BAD_SHAPE;
+    const int Cs[2] = {C1, C2};
+    const int strides[4] = {o1_sr, o1_sc, o2_sr, o2_sc};
+    for (int i = 0; i < 2; ++i) {
+        if (Cs[i] < 8 || (Cs[i] % 8) != 0 || Cs[i] > (1 << 20) || strides[2 * i] < 1 || strides[2 * i + 1] < 1) return Q4_ERR_BAD_SHAPE;
+        if ((long long)M * Cs[i] * 2 >= 0x70000000ll) return Q4_ERR_BAD_SHAPE;               /* 32-bit buffer offsets */
+    }
+    if (misaligned(p1) || misaligned(in1) || misaligned(p2) || misaligned(in2) ||
+        (reinterpret_cast<uintptr_t>(out1) & 3u) || (reinterpret_cast<uintptr_t>(out2) & 3u))
+        return Q4_ERR_MISALIGNED;
+    const size_t need = q4_lora_grad_workspace(M, C1, R) + q4_lora_grad_workspace(M, C2, R);
+    if (need > 0) {
+        if (!workspace || workspace_bytes < need) return Q4_ERR_WORKSPACE;
+        if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
+    }
+    return q4_launch_lora_grad_pair(p1, in1, out1, o1_sr, o1_sc, C1, p2, in2, out2, o2_sr, o2_sc, C2, alpha, M, R,
+                                    workspace, (hipStream_t)stream);
 }

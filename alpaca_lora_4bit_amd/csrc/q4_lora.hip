@@ -230,12 +230,32 @@ constexpr int kGradWaves = 4;
 template <int ND, int NPP>
 struct RowRegs { uint32_t d[16][ND]; uint32_t plo[NPP], phi[NPP]; };
 
+// One or two gradients per launch (blockIdx.z): the two adapter gradients of a layer share M, R and alpha and are
+// independent, and since a single one is bound by the latency of its burst of loads, running them side by side
+// costs little more than one.  Workgroups beyond a problem's own grid leave at once.
+struct GradProb {
+    const half_t* P;          // [M, R]
+    const half_t* in;         // [M, C]
+    float* out;               // through o_sr, o_sc
+    float* part;              // partial tiles [splits][col_blocks][NACC][64]
+    int o_sr, o_sc, C, col_blocks, splits, rows_per_wg;
+};
+struct GradArgs {
+    GradProb p[2];
+    float alpha;
+    int M;
+};
+
 template <int R>
-__global__ __launch_bounds__(64 * kGradWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void lora_grad_kernel(const half_t* __restrict__ P,
-                                                                    const half_t* __restrict__ in,
-                                                                    float* __restrict__ out, int o_sr, int o_sc,
-                                                                    float alpha, int M, int C, int rows_per_wg,
-                                                                    float* __restrict__ part) {
+__global__ __launch_bounds__(64 * kGradWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void lora_grad_kernel(GradArgs ga) {
+    const GradProb& q = ga.p[blockIdx.z];
+    if ((int)blockIdx.x >= q.col_blocks || (int)blockIdx.y >= q.splits) return;       // uniform over the workgroup
+    const half_t* __restrict__ P = q.P;
+    const half_t* __restrict__ in = q.in;
+    float* __restrict__ out = q.out;
+    float* __restrict__ part = q.part;
+    const int o_sr = q.o_sr, o_sc = q.o_sc, C = q.C, rows_per_wg = q.rows_per_wg, M = ga.M;
+    const float alpha = ga.alpha;
     constexpr int CPT = 64 / R;                  // columns per thread: 8 (R = 8) or 4 (R = 16)
     constexpr int ND = CPT / 2;                  // dwords per thread and row
     constexpr int NPP = 8 * R / 64;              // pairs of P staged per lane and 16-row block
@@ -329,8 +349,8 @@ __global__ __launch_bounds__(64 * kGradWaves) __attribute__((amdgpu_waves_per_eu
 #pragma unroll
         for (int e = 0; e < CPT; ++e) red[wave][j * CPT + e][lane] = acc[j][e];
     __syncthreads();
-    const bool direct = gridDim.y == 1;
-    float* tile = part + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * (NACC * 64);
+    const bool direct = q.splits == 1;
+    float* tile = part + ((size_t)blockIdx.y * q.col_blocks + blockIdx.x) * (NACC * 64);
     for (int o = threadIdx.x; o < NACC * 64; o += 64 * kGradWaves) {
         const int a = o >> 6, ln = o & 63;
         float v = 0.f;
@@ -347,14 +367,17 @@ __global__ __launch_bounds__(64 * kGradWaves) __attribute__((amdgpu_waves_per_eu
 
 // Adds the `splits` partial tiles of every column block in order and writes the scaled result.
 template <int R>
-__global__ __launch_bounds__(256) void lora_grad_reduce_kernel(const float* __restrict__ part, float* __restrict__ out,
-                                                               int o_sr, int o_sc, float alpha, int C,
-                                                               int col_blocks, int splits) {
+__global__ __launch_bounds__(256) void lora_grad_reduce_kernel(GradArgs ga) {
+    const GradProb& q = ga.p[blockIdx.y];
+    const float* __restrict__ part = q.part;
+    float* __restrict__ out = q.out;
+    const int o_sr = q.o_sr, o_sc = q.o_sc, C = q.C, col_blocks = q.col_blocks, splits = q.splits;
+    const float alpha = ga.alpha;
     constexpr int CPT = 64 / R;
     constexpr int NACC = R * CPT;
     const int t = blockIdx.x * 256 + threadIdx.x;         // index into one split's tiles: [column block][a][lane]
     const int total = col_blocks * NACC * 64;
-    if (t >= total) return;
+    if (splits <= 1 || t >= total) return;                // a single split was written directly
     float v = 0.f;
     int s = 0;
     for (; s + 8 <= splits; s += 8) {
@@ -451,23 +474,62 @@ extern "C" size_t q4_lora_grad_workspace(int M, int C, int R) {
     return g.splits == 1 ? 0 : (size_t)g.splits * g.col_blocks * 64 * 64 * sizeof(float);
 }
 
-extern "C" int q4_launch_lora_grad(const void* P, const void* in, float* out, int o_sr, int o_sc, float alpha,
-                                   int M, int C, int R, void* workspace, hipStream_t stream) {
+static q4::GradProb make_grad_prob(const void* P, const void* in, float* out, int o_sr, int o_sc, int M, int C, int R,
+                                   float* part) {
+    const q4::GradPlan g = q4::plan_grad(M, C, R);
+    q4::GradProb q;
+    q.P = reinterpret_cast<const q4::half_t*>(P);
+    q.in = reinterpret_cast<const q4::half_t*>(in);
+    q.out = out;
+    q.part = part;
+    q.o_sr = o_sr; q.o_sc = o_sc; q.C = C;
+    q.col_blocks = g.col_blocks; q.splits = g.splits; q.rows_per_wg = g.rows_per_wg;
+    return q;
+}
+
+static int launch_grad(const q4::GradArgs& ga, int nprob, int R, hipStream_t stream) {
     using namespace q4;
-    const GradPlan g = plan_grad(M, C, R);
-    const dim3 grid(g.col_blocks, g.splits), block(64 * kGradWaves);
-    const half_t* pp = reinterpret_cast<const half_t*>(P);
-    const half_t* ip = reinterpret_cast<const half_t*>(in);
-    float* ws = reinterpret_cast<float*>(workspace);
-    const int rblocks = (g.col_blocks * 64 * 64 + 255) / 256;
+    int gx = 0, gy = 0, rx = 0;
+    bool any_split = false;
+    for (int i = 0; i < nprob; ++i) {
+        gx = ga.p[i].col_blocks > gx ? ga.p[i].col_blocks : gx;
+        gy = ga.p[i].splits > gy ? ga.p[i].splits : gy;
+        const int rb = (ga.p[i].col_blocks * 64 * 64 + 255) / 256;
+        rx = rb > rx ? rb : rx;
+        any_split = any_split || ga.p[i].splits > 1;
+    }
+    const dim3 grid(gx, gy, nprob), block(64 * kGradWaves);
     if (R == 8) {
-        hipLaunchKernelGGL(lora_grad_kernel<8>, grid, block, 0, stream, pp, ip, out, o_sr, o_sc, alpha, M, C, g.rows_per_wg, ws);
-        if (g.splits > 1)
-            hipLaunchKernelGGL(lora_grad_reduce_kernel<8>, dim3(rblocks), dim3(256), 0, stream, ws, out, o_sr, o_sc, alpha, C, g.col_blocks, g.splits);
+        hipLaunchKernelGGL(lora_grad_kernel<8>, grid, block, 0, stream, ga);
+        if (any_split) hipLaunchKernelGGL(lora_grad_reduce_kernel<8>, dim3(rx, nprob), dim3(256), 0, stream, ga);
     } else {
-        hipLaunchKernelGGL(lora_grad_kernel<16>, grid, block, 0, stream, pp, ip, out, o_sr, o_sc, alpha, M, C, g.rows_per_wg, ws);
-        if (g.splits > 1)
-            hipLaunchKernelGGL(lora_grad_reduce_kernel<16>, dim3(rblocks), dim3(256), 0, stream, ws, out, o_sr, o_sc, alpha, C, g.col_blocks, g.splits);
+        hipLaunchKernelGGL(lora_grad_kernel<16>, grid, block, 0, stream, ga);
+        if (any_split) hipLaunchKernelGGL(lora_grad_reduce_kernel<16>, dim3(rx, nprob), dim3(256), 0, stream, ga);
     }
     return hipGetLastError() == hipSuccess ? 0 : -4;
+}
+
+extern "C" int q4_launch_lora_grad(const void* P, const void* in, float* out, int o_sr, int o_sc, float alpha,
+                                   int M, int C, int R, void* workspace, hipStream_t stream) {
+    q4::GradArgs ga;
+    ga.p[0] = make_grad_prob(P, in, out, o_sr, o_sc, M, C, R, reinterpret_cast<float*>(workspace));
+    ga.p[1] = ga.p[0];
+    ga.alpha = alpha;
+    ga.M = M;
+    return launch_grad(ga, 1, R, stream);
+}
+
+// Two gradients with the same M, R and alpha in one launch (plus one launch for both reductions); the workspace
+// holds the partial tiles of the first problem followed by those of the second.
+extern "C" int q4_launch_lora_grad_pair(const void* P1, const void* in1, float* out1, int o1_sr, int o1_sc, int C1,
+                                        const void* P2, const void* in2, float* out2, int o2_sr, int o2_sc, int C2,
+                                        float alpha, int M, int R, void* workspace, hipStream_t stream) {
+    q4::GradArgs ga;
+    float* ws = reinterpret_cast<float*>(workspace);
+    ga.p[0] = make_grad_prob(P1, in1, out1, o1_sr, o1_sc, M, C1, R, ws);
+    ga.p[1] = make_grad_prob(P2, in2, out2, o2_sr, o2_sc, M, C2, R,
+                             ws ? ws + q4_lora_grad_workspace(M, C1, R) / sizeof(float) : nullptr);
+    ga.alpha = alpha;
+    ga.M = M;
+    return launch_grad(ga, 2, R, stream);
 }

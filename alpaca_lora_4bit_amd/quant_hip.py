@@ -511,6 +511,33 @@ def lora_grad(p, inp, alpha, transposed=False):
     return out
 
 
+def lora_grad_pair(p1, inp1, p2, inp2, alpha):
+    """Both adapter gradients of a layer in one launch: returns (alpha * p1^T @ inp1 as [R, C1],
+    alpha * p2^T @ inp2 stored as a contiguous [C2, R] tensor) -- dA from (dyb, x) and dB in lora_B.weight's
+    layout from (xa, dy).  Same requirements as lora_grad; p1 and p2 share their shape."""
+    for p, inp in ((p1, inp1), (p2, inp2)):
+        _require(p.is_cuda and p.dtype == torch.float16 and p.dim() == 2 and p.is_contiguous(),
+                 "p must be a contiguous float16 [M, R] CUDA tensor")
+        _require(inp.dtype == torch.float16 and inp.dim() == 2 and inp.is_contiguous() and inp.device == p.device
+                 and inp.shape[0] == p.shape[0], "inp must be a contiguous float16 [M, C] tensor on the same device")
+    _require(p1.shape == p2.shape and p1.device == p2.device, "the two rank-R operands must share shape and device")
+    M, R = p1.shape
+    C1, C2 = inp1.shape[1], inp2.shape[1]
+    _require(R in LORA_GRAD_RANKS and C1 % 8 == 0 and C2 % 8 == 0 and M >= 1, "lora_grad needs R in (8, 16) and C % 8 == 0")
+    dev = p1.device
+    out1 = torch.empty((R, C1), dtype=torch.float32, device=dev)
+    out2 = torch.empty((C2, R), dtype=torch.float32, device=dev)
+    L = _lib.lib()
+    nbytes = L.q4_lora_grad_workspace_bytes(M, C1, R) + L.q4_lora_grad_workspace_bytes(M, C2, R)
+    with _device_ctx(dev):
+        ws = _scratch(dev, nbytes)
+        rc = L.q4_lora_grad_pair_f32(p1.data_ptr(), inp1.data_ptr(), out1.data_ptr(), C1, 1, C1,
+                                     p2.data_ptr(), inp2.data_ptr(), out2.data_ptr(), 1, R, C2,
+                                     float(alpha), M, R, ws.data_ptr(), ws.numel(), _stream(dev))
+    _lib.check(rc, "q4_lora_grad_pair_f32")
+    return out1, out2
+
+
 # ------------------------------------------------- quant_cuda-compatible entry points
 def _infer_groupsize(K, G):
     return -(-K // G)

@@ -158,6 +158,15 @@ size_t q4_lora_grad_workspace_bytes(int M, int C, int R);
 int q4_lora_grad_f32(const void *p, const void *in, float *out, int o_sr, int o_sc, float alpha,
                      int M, int C, int R, void *workspace, size_t workspace_bytes, void *stream);
 
+/* Both adapter gradients of a layer in one launch (plus one for the two reductions): problem 1 and problem 2 as
+ * for q4_lora_grad_f32, sharing M, R and alpha -- dA from (dyb, x, C1 = K) and dB from (xa, dy, C2 = N) in the
+ * backward of models.py:66.  A single gradient is bound by the latency of its one burst of loads, so the pair
+ * costs little more than one.  `workspace`: q4_lora_grad_workspace_bytes(M, C1, R) +
+ * q4_lora_grad_workspace_bytes(M, C2, R) bytes, 256-byte aligned, contents irrelevant. */
+int q4_lora_grad_pair_f32(const void *p1, const void *in1, float *out1, int o1_sr, int o1_sc, int C1,
+                          const void *p2, const void *in2, float *out2, int o2_sr, int o2_sc, int C2,
+                          float alpha, int M, int R, void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

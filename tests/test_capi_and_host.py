@@ -86,6 +86,9 @@ def test_error_codes_and_validation_need_no_gpu():
     assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 64, 4096, 12, fake, 1 << 20, None) == -2   # R not 8/16
     assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 2048, 4096, 8, None, 0, None) == -3
     assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 2048, 4096, 8, fake, 1024, None) == -3
+    assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, None, 1, 8, 4096, 1.0, 2048, 8, fake, 1 << 24, None) == -1
+    assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, fake, 1, 8, 4100, 1.0, 2048, 8, fake, 1 << 24, None) == -2
+    assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, fake, 1, 8, 4096, 1.0, 2048, 8, fake, 1 << 22, None) == -3  # needs 2 x 4 MiB
     assert L.q4_gemv_workspace_bytes(16, 4096, 11008) == 16 * 11008 * 8
     assert L.q4_gemv_workspace_bytes(0, 4096, 11008) == 0
 

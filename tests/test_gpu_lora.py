@@ -109,3 +109,23 @@ def test_fused_lora_function_against_oracle_fp32_adapters(oracle):
         assert g.shape == ref.shape
         assert np.abs(g - ref).max() <= 1e-2 * np.abs(ref).max()
     assert Ad.grad.dtype == torch.float32 and Bd.grad.dtype == torch.float32
+
+
+@pytest.mark.parametrize("M,C1,C2,R", [(2048, 4096, 4096, 8), (300, 1408, 512, 16), (50, 512, 11008, 8), (1000, 11008, 4096, 16)])
+def test_lora_grad_pair_equals_the_two_single_launches(M, C1, C2, R):
+    """Both gradients in one launch (different column counts, hence different grids and split counts) give the
+    bits of the two separate launches."""
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    g = torch.Generator().manual_seed(M + C1 + R)
+    p1 = torch.randn(M, R, generator=g).half().cuda()
+    p2 = torch.randn(M, R, generator=g).half().cuda()
+    in1 = torch.randn(M, C1, generator=g).half().cuda()
+    in2 = torch.randn(M, C2, generator=g).half().cuda()
+    want1 = quant_hip.lora_grad(p1, in1, 2.0)
+    want2 = quant_hip.lora_grad(p2, in2, 2.0, transposed=True)
+    got1, got2 = quant_hip.lora_grad_pair(p1, in1, p2, in2, 2.0)
+    assert got1.shape == (R, C1) and got2.shape == (C2, R)
+    assert torch.equal(got1, want1) and torch.equal(got2, want2)
+    ref1 = 2.0 * p1.float().t() @ in1.float()
+    assert float((got1 - ref1).abs().max() / ref1.abs().max()) <= 1e-3
