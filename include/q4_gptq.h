@@ -84,26 +84,27 @@ int q4_gemv_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, co
                 int M, int K, int N, int G,
                 void *workspace, size_t workspace_bytes, void *stream);
 
-/* The same product for an act-order layer whose packed rows were sorted by group with q4_permute_rows
- * (1 <= M <= 4, K >= 1024 and M * (2*K + 4096) <= 65536 bytes, i.e. the activation rows fit in LDS:
- * K <= 30720 at M=1, K <= 6144 at M=4): `qweight_sorted` is that sorted copy, `perm` [K] int32 the permutation it was made with
- * (perm[p] = original index of sorted row p), `groupsize` = K / G.  x is the ORIGINAL activation matrix: the
- * kernel gathers x[:, perm[p]] itself (through LDS) while its weight loads are in flight, which replaces the separate gather
+/* The same product for an act-order layer whose packed rows were sorted by group with q4_permute_rows.
+ * Limits: 1 <= M <= 4, K >= 1024 and M * (2*K + 4096) <= 65536 bytes, i.e. the activation rows fit in LDS
+ * (K <= 30720 at M=1, K <= 6144 at M=4).  `qweight_sorted` is the sorted copy, `perm` [K] int32 the
+ * permutation it was made with (perm[p] = original index of sorted row p, every value in [0, K): the kernel
+ * does not range-check it), `groupsize` = K / G.  x is the ORIGINAL activation matrix: the kernel gathers
+ * x[:, perm[p]] itself, through LDS, while its weight loads are in flight, which replaces the separate gather
  * the caller would otherwise run before q4_gemv_f16.  The values are those of the reference's act-order
  * product (quant_cuda_kernel.cu:443-536 with per-row g_idx).  Workspace as for q4_gemv_f16. */
-/* The same product for the v1 layout (one fp16 scale and one fp16 zero value per column, W = s*q - zero):
- *   y fp16 [M, N] = x fp16 [M, K] @ W,  1 <= M <= 16.
- * Replaces quant_cuda.vecquant4matmul_v1_faster (quant_cuda/quant_cuda.cpp:163-175; kernel
- * quant_cuda_kernel.cu:1244-1302, launcher :1304-1335) as called from matmul_utils_4bit.py:36-56.  `scales`, `zeros` fp16 [N],
- * 8-byte aligned.  Workspace as for q4_gemv_f16. */
-int q4_gemv_v1_f16(const void *x, const int32_t *qweight, const void *scales, const void *zeros, void *y,
-                   int accumulate, int M, int K, int N,
-                   void *workspace, size_t workspace_bytes, void *stream);
-
 int q4_gemv_sorted_f16(const void *x, const int32_t *qweight_sorted, const int32_t *qzeros, const void *scales,
                        const int32_t *perm, int groupsize, void *y, int accumulate,
                        int M, int K, int N, int G,
                        void *workspace, size_t workspace_bytes, void *stream);
+
+/* The same product for the v1 layout (one fp16 scale and one fp16 zero value per column, W = s*q - zero):
+ *   y fp16 [M, N] = x fp16 [M, K] @ W,  1 <= M <= 16.
+ * Replaces quant_cuda.vecquant4matmul_v1_faster (quant_cuda/quant_cuda.cpp:163-175; kernel
+ * quant_cuda_kernel.cu:1244-1302, launcher :1304-1335) as called from matmul_utils_4bit.py:36-56.
+ * `scales`, `zeros` fp16 [N], 8-byte aligned.  Workspace as for q4_gemv_f16. */
+int q4_gemv_v1_f16(const void *x, const int32_t *qweight, const void *scales, const void *zeros, void *y,
+                   int accumulate, int M, int K, int N,
+                   void *workspace, size_t workspace_bytes, void *stream);
 
 /* Forward GEMM, any M >= 1:
  *   y fp16 [M, N] = x fp16 [M, K] @ W  (+ bias fp16 [N])  (+ lora_scale * xa fp16 [M, R] @ Bm [R, N])
