@@ -18,42 +18,50 @@ def _decoder_layer_type():
     return LlamaDecoderLayer
 
 
-class NewForward:
-    """Recompute-in-backward wrapper around one decoder block."""
+class _ForwardPatch:
+    """Replaces `target.forward` by `self.new_forward`; the original stays reachable as `old_forward_for_cp`
+    (the attribute name the reference uses, gradient_checkpointing.py:18,41)."""
 
-    def __init__(self, layer):
-        self.layer = layer
+    def __init__(self, target):
+        self._target = target
         self.apply_patch()
 
     def apply_patch(self):
-        self.layer.old_forward_for_cp = self.layer.forward
-        self.layer.forward = self.new_forward
+        self._target.old_forward_for_cp = self._target.forward
+        self._target.forward = self.new_forward
+
+    def new_forward(self, *args, **kwargs):          # pragma: no cover - overridden
+        raise NotImplementedError
+
+
+class NewForward(_ForwardPatch):
+    """Recompute-in-backward wrapper around one decoder block (`.layer`)."""
+
+    @property
+    def layer(self):
+        return self._target
 
     def new_forward(self, *args, **kwargs):
-        def run(*inputs):
-            return self.layer.old_forward_for_cp(*inputs, **kwargs)
-
-        if not self.layer.training:
-            return run(*args)
+        block = self._target
+        if not block.training:
+            return block.old_forward_for_cp(*args, **kwargs)
         # keyword arguments (masks, position embeddings, caches) ride in the closure, as in the reference
-        return checkpoint(run, *args, use_reentrant=True)
+        return checkpoint(lambda *inputs: block.old_forward_for_cp(*inputs, **kwargs), *args, use_reentrant=True)
 
 
-class VarWrapper:
-    """Cuts the graph after the embedding: its output becomes a leaf that requires grad."""
+class VarWrapper(_ForwardPatch):
+    """Cuts the graph after the embedding (`.model`): its output becomes a leaf that requires grad."""
 
     def __init__(self, model):
-        self.model = model
-        self.apply_patch()
+        super().__init__(model)
         print("Var Wrapper Patch Applied")
 
-    def apply_patch(self):
-        self.model.old_forward_for_cp = self.model.forward
-        self.model.forward = self.new_forward
+    @property
+    def model(self):
+        return self._target
 
     def new_forward(self, *args, **kwargs):
-        out = self.model.old_forward_for_cp(*args, **kwargs)
-        return out.detach().requires_grad_(True)
+        return self._target.old_forward_for_cp(*args, **kwargs).detach().requires_grad_(True)
 
 
 def checkpoint_locations(n_layers: int, checkpoint_ratio=1) -> np.ndarray:
