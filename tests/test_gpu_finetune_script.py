@@ -69,3 +69,27 @@ def test_finetune_module_trains_and_saves_an_adapter(tmp_path, oracle, grad_chck
         text_base, _ = inference.main(base_args)
         assert isinstance(text_lora, str) and text_lora.startswith("alpha beta gamma")
         assert text_base.startswith("alpha beta gamma")
+
+
+def test_finetune_module_on_alpaca_records_with_evaluation(tmp_path, oracle):
+    """Alpaca-style JSON records, a validation split and periodic evaluation (no-grad forward of the LoRA layers with
+    many rows) through the same flow."""
+    from alpaca_lora_4bit_amd import finetune
+    ckpt = str(tmp_path / "ckpt")
+    build(ckpt, oracle, seed=6, with_tokenizer=True)
+    rnd = random.Random(2)
+    records = [{"instruction": " ".join(rnd.choice(WORDS) for _ in range(4)), "input": "",
+                "output": " ".join(rnd.choice(WORDS) for _ in range(6))} for _ in range(40)]
+    data = str(tmp_path / "alpaca.json")
+    with open(data, "w") as fh:
+        json.dump(records, fh)
+    out = str(tmp_path / "lora_out")
+    model, tokenizer, trainer = finetune.main([
+        data, "--ds_type", "alpaca", "--llama_q4_config_dir", ckpt, "--llama_q4_model",
+        os.path.join(ckpt, "model.safetensors"), "--groupsize", str(GROUPSIZE), "--lora_out_dir", out,
+        "--mbatch_size", "4", "--batch_size", "4", "--epochs", "1", "--lr", "1e-3", "--cutoff_len", "96",
+        "--warmup_steps", "1", "--logging_steps", "2", "--val_set_size", "0.2", "--lora_dropout", "0.05"])
+    evals = [h["eval_loss"] for h in trainer.state.log_history if "eval_loss" in h]
+    losses = [h["loss"] for h in trainer.state.log_history if "loss" in h]
+    assert evals and all(e == e and e > 0 for e in evals) and losses and all(l == l for l in losses)
+    assert os.path.exists(os.path.join(out, "adapter_model.safetensors"))
