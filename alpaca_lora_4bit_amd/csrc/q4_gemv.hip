@@ -1,4 +1,8 @@
-// Decode GEMV / skinny GEMM for 1 <= M <= 16:  y[M,N] = x[M,K] @ W   (HBM-bound).
+// Weight-streaming products for few activation rows:  y[M,N] = x[M,K] @ W   (HBM-bound).
+//   gemv_seq_kernel       1 <= M <= 16, sequential groups (also the v1 layout: one scale / zero per column)
+//   gemv_seq_perm_kernel  1 <= M <= 4, act-order layer with rows sorted by group: gathers x through the permutation
+//   gemv_gidx_kernel      1 <= M <= 16, act-order with per-row groups read through g_idx
+//   skinny_seq_kernel     17 <= M <= 64, sequential groups (fp32 partial rows + ordered reduction)
 //
 // Work split.  A workgroup owns a strip of 64 columns; its W wavefronts (W = blockDim.x / 64)
 // take consecutive chunks of 32*NSTEP rows, and gridDim.y workgroups share one strip when K is
@@ -7,15 +11,16 @@
 // consecutive rows of four adjacent columns.  A packed word is exactly the 8-deep k-slice that
 // lane l feeds to v_mfma_f32_16x16x32_f16 as its B operand, so the four words go to four MFMAs
 // whose column index i stands for column n0 + 4i + j (j = 0..3).  The A operand is x (row
-// m = l % 16, the same 8 k values; rows >= M are zero), so all M <= 16 activation rows ride
+// m = l % 16, the same 8 k values; rows >= M repeat row M-1), so all M <= 16 activation rows ride
 // along and the weights are read from HBM once.  Every load of a chunk is issued before the
 // first is consumed, in straight-line code: with ~90 KB of weights per CU the kernel is one
 // burst of loads followed by a short arithmetic tail.
 //
-// Sequential groups (no act-order).  The B operand holds the raw codes as fp16 (1024 + q)
-// and a fifth MFMA with an all-ones B operand yields X = sum_k x over the same rows, so per
-// group only   y += s * (acc - (1025 + z) * X)   is evaluated (fp32) instead of one
-// multiply-subtract per weight.  Mathematically equal to sum_k x*(s*q - s*(z+1))
+// Sequential groups (no act-order).  The B operand holds the raw codes as fp16 (1024 + q for the
+// nibbles in bits 0-3 of a half, 64 + q for those in bits 4-7) and two more MFMAs with constant B
+// operands yield O = sum_k x*offset and X = sum_k x over the same rows, so per group only
+//   y += s * ((acc - O) - (z + 1) * X)   is evaluated (fp32) instead of one multiply-subtract per
+// weight.  Mathematically equal to sum_k x*(s*q - s*(z+1))
 // (src/alpaca_lora_4bit/quant_cuda/quant_cuda_kernel.cu:1026-1037); not bit-identical to it,
 // nor is the reference to itself (fp16 partial sums and atomicAdd order, :1037,1040).
 //
