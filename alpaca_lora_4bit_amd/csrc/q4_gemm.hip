@@ -577,16 +577,39 @@ static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
     static const int env_cfg = getenv("Q4_GEMM_CFG") ? atoi(getenv("Q4_GEMM_CFG")) : -1;
     static const int env_splits = getenv("Q4_GEMM_SPLITS") ? atoi(getenv("Q4_GEMM_SPLITS")) : 0;
     GemmPlan p;
-    const bool tall = (long)(nout / BN) * ((M + 255) / 256) >= 200;
-    p.cfg = env_cfg >= 0 ? env_cfg : (tall ? 2 : 0);
-    const int bm = p.cfg == 0 ? 128 : 256;
-    const long tiles = (long)(nout / BN) * ((M + bm - 1) / bm);
     const int nsteps = red / BK;
+    // Tiles of 256 rows (8 wavefronts, one dequantized slab of W for 256 activation rows) do about twice the work per
+    // CU and unit of time that 128-row tiles do, so they are used whenever they can occupy the 256 CUs in one round:
+    // enough of them outright, or few enough that splitting the reduction floor(256 / tiles) ways gives every CU one
+    // workgroup (never more than 256 workgroups: a second, nearly empty round costs more than the split gains).
+    const long t256 = (long)(nout / BN) * ((M + 255) / 256);
     int splits = 1;
-    if (tiles < 192) {
-        splits = (int)((384 + tiles - 1) / tiles);
-        if (splits > 8) splits = 8;                            // measured: more splits only add prologues and partial tiles
-        if (splits > nsteps / 4) splits = nsteps / 4;          // at least four steps per workgroup
+    if (t256 >= 200) {
+        p.cfg = 2;
+    } else if (t256 <= 128 && M >= 192 && nsteps >= 8 * (int)(256 / t256) &&
+               (size_t)(256 / t256 > 8 ? 8 : 256 / t256) * (size_t)M * (size_t)nout * sizeof(float) <= workspace_bytes) {
+        p.cfg = 2;                                             // only with room for all its partial tiles
+        splits = (int)(256 / t256);
+        if (splits > 8) splits = 8;
+    } else {
+        p.cfg = 0;
+        const long tiles = (long)(nout / BN) * ((M + 127) / 128);
+        if (tiles < 192) {
+            splits = (int)((384 + tiles - 1) / tiles);
+            if (splits > 8) splits = 8;                        // measured: more splits only add prologues and partial tiles
+            if (splits > nsteps / 4) splits = nsteps / 4;      // at least four steps per workgroup
+        }
+    }
+    if (env_cfg >= 0 && env_cfg != p.cfg) {                    // experiments: forced tile shape, splits as before
+        p.cfg = env_cfg;
+        const int bm = p.cfg == 0 ? 128 : 256;
+        const long tiles = (long)(nout / BN) * ((M + bm - 1) / bm);
+        splits = 1;
+        if (tiles < 192) {
+            splits = (int)((384 + tiles - 1) / tiles);
+            if (splits > 8) splits = 8;
+            if (splits > nsteps / 4) splits = nsteps / 4;
+        }
     }
     if (env_splits > 0) splits = env_splits > nsteps ? nsteps : env_splits;
     while (splits > 1 && (size_t)splits * (size_t)M * (size_t)nout * sizeof(float) > workspace_bytes) --splits;
