@@ -579,12 +579,13 @@ static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
     GemmPlan p;
     const int nsteps = red / BK;
     // Tiles of 256 rows (8 wavefronts, one dequantized slab of W for 256 activation rows) do about twice the work per
-    // CU and unit of time that 128-row tiles do, so they are used whenever they can occupy the 256 CUs in one round:
-    // enough of them outright, or few enough that splitting the reduction floor(256 / tiles) ways gives every CU one
-    // workgroup (never more than 256 workgroups: a second, nearly empty round costs more than the split gains).
+    // CU and unit of time that 128-row tiles do, so they are used from 192 rows on: as they are when there are more
+    // than 128 of them (even 130 of them on 256 CUs beat 260 tiles of 128 rows), otherwise with the reduction split
+    // floor(256 / tiles) ways so that every CU gets one workgroup (never more than 256 workgroups: a second, nearly
+    // empty round costs more than the split gains).
     const long t256 = (long)(nout / BN) * ((M + 255) / 256);
     int splits = 1;
-    if (t256 >= 200) {
+    if (t256 > 128 && M >= 192) {
         p.cfg = 2;
     } else if (t256 <= 128 && M >= 192 && nsteps >= 8 * (int)(256 / t256) &&
                (size_t)(256 / t256 > 8 ? 8 : 256 / t256) * (size_t)M * (size_t)nout * sizeof(float) <= workspace_bytes) {
