@@ -8,10 +8,11 @@
 //
 // Tiling.  A workgroup computes a BM x 128 output tile with 2*WGM wavefronts (WGM along M, 2
 // along N), each owning (BM/WGM) x 64 outputs as (BM/WGM/32) x 2 accumulators of
-// v_mfma_f32_32x32x16_f16.  Large problems use BM = 256 with 8 wavefronts of 64 x 64 (two per SIMD:
+// v_mfma_f32_32x32x16_f16.  From 192 rows on BM = 256 with 8 wavefronts of 64 x 64 (two per SIMD:
 // while one waits or dequantizes the other multiplies, and one dequantized slab of W serves 256
-// activation rows); problems with fewer than ~200 such tiles use BM = 128 with 4 wavefronts so that
-// every CU still gets a workgroup.  The reduction runs in steps of 64.  Both LDS tiles are stored "row = output index, minor = reduction index" with 8 halves of
+// activation rows), with the reduction split over several workgroups when there are too few tiles
+// for the CUs (plan_gemm); fewer rows use BM = 128 with 4 wavefronts.  The reduction runs in steps
+// of 64.  Both LDS tiles are stored "row = output index, minor = reduction index" with 8 halves of
 // padding per row (stride 144 B): the 128-bit operand fetches of 16 consecutive lanes then hit
 // 64 distinct banks.  LDS is double buffered in four distinct arrays (110 KB at BM = 256).
 //
