@@ -66,7 +66,8 @@ def test_gemm_equals_dense_matmul_of_dequantized_weight(oracle):
 
 
 @pytest.mark.parametrize("act", [False, True])
-@pytest.mark.parametrize("M,K,N,r", [(2048, 4096, 4096, 8), (130, 256, 384, 16), (64, 512, 128, 64)])
+@pytest.mark.parametrize("M,K,N,r", [(2048, 4096, 4096, 8), (130, 256, 384, 16), (64, 512, 128, 64),
+                                     (1024, 4096, 4096, 8), (512, 11008, 4096, 16)])   # 256-row tiles, reduction split 2 / 4 ways
 def test_gemm_lora_steps(oracle, M, K, N, r, act):
     """Config 2 shape (and small ones): forward with bias + adapter, backward-dx with adapter."""
     import torch
