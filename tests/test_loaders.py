@@ -111,3 +111,58 @@ def test_fused_qkv_and_gate_up_keep_the_logits(tmp_path, oracle):
     for a, b in ((after, before), (after1, before1)):
         assert (a - b).abs().max().item() <= 2e-3 * b.abs().max().item()
     assert make_quant_attn(model) == 0                       # idempotent: nothing left to fuse
+
+
+@pytest.mark.gpu
+def test_saved_adapter_injected_on_fused_qkv(tmp_path, oracle):
+    """inject_lora_layers(model, lora_path) (model_attn_mlp_patch.py:283-335 of the reference): a saved q/v adapter
+    lands on the fused qkv layer as one block-structured adapter; logits equal those of the unfused model carrying
+    the same adapter on q_proj and v_proj, at prefill and at one decode row, and a second call replaces the first."""
+    import json
+    from safetensors.torch import save_file
+    from alpaca_lora_4bit_amd import autograd_4bit as ag, finetune, models
+    from alpaca_lora_4bit_amd.model_attn_mlp_patch import inject_lora_layers as inject_saved, make_quant_attn
+    path = str(tmp_path / "ckpt")
+    build(path, oracle, seed=6, with_tokenizer=True)
+    load = lambda: ag.load_llama_model_4bit_low_ram(path, os.path.join(path, "model.safetensors"), groupsize=GROUPSIZE,
+                                                    half=True, device_map={"": 0})[0]
+    r, alpha = 8, 16
+    gen = torch.Generator().manual_seed(11)
+
+    def write_adapter(folder, scale):
+        os.makedirs(folder)
+        state = {}
+        for i in range(2):
+            for proj in ("q_proj", "v_proj"):
+                base = f"base_model.model.model.layers.{i}.self_attn.{proj}"
+                state[f"{base}.lora_A.weight"] = (torch.randn(r, 256, generator=gen) * 0.05).float()
+                state[f"{base}.lora_B.weight"] = (torch.randn(256, r, generator=gen) * scale).float()
+        save_file(state, os.path.join(folder, "adapter_model.safetensors"))
+        json.dump({"r": r, "lora_alpha": alpha, "peft_type": "LORA"}, open(os.path.join(folder, "adapter_config.json"), "w"))
+
+    first, second = str(tmp_path / "lora_a"), str(tmp_path / "lora_b")
+    write_adapter(first, 0.05)
+    write_adapter(second, 0.08)
+    ids = torch.tensor([[1] + [5 + (11 * i) % 200 for i in range(23)]]).cuda()
+
+    fused = load()
+    with torch.no_grad():
+        plain = fused(ids).logits.float()
+    assert make_quant_attn(fused) == 2
+    with pytest.raises(ValueError):
+        inject_saved(load(), first)                                         # not fused yet
+    for folder in (first, second):                                          # the second call replaces the first adapter
+        layers = inject_saved(fused, folder)
+        assert len(layers) == 2 and all(l.lora_A["default"].weight.shape == (2 * r, 256) for l in layers)
+        assert all(abs(l.scaling["default"] - alpha / r) < 1e-12 for l in layers)
+        k_rows = layers[0].lora_B["default"].weight[256:512]
+        assert float(k_rows.abs().max()) == 0.0                             # nothing lands on k_proj
+        ref = load()
+        models.inject_lora_layers(ref, target_modules=("q_proj", "v_proj"), r=r, lora_alpha=alpha)
+        assert finetune.load_adapter(ref, folder) == 8
+        ref.half()
+        with torch.no_grad():
+            for rows in (ids, ids[:, :1]):
+                want, got = ref(rows).logits.float(), fused(rows).logits.float()
+                assert (got - want).abs().max().item() <= 4e-3 * want.abs().max().item()
+        assert (ref(ids).logits.float() - plain).abs().max().item() > 0.05 * plain.abs().max().item()   # the adapter matters
