@@ -8,7 +8,7 @@
 //
 // Tiling.  A workgroup computes a BM x 128 output tile with 2*WGM wavefronts (WGM along M, 2
 // along N), each owning (BM/WGM) x 64 outputs as (BM/WGM/32) x 2 accumulators of
-// v_mfma_f32_32x32x16_f16.  From 192 rows on BM = 256 with 8 wavefronts of 64 x 64 (two per SIMD:
+// v_mfma_f32_32x32x16_f16.  From 129 rows on BM = 256 with 8 wavefronts of 64 x 64 (two per SIMD:
 // while one waits or dequantizes the other multiplies, and one dequantized slab of W serves 256
 // activation rows), with the reduction split over several workgroups when there are too few tiles
 // for the CUs (plan_gemm); fewer rows use BM = 128 with 4 wavefronts.  The reduction runs in steps
@@ -580,15 +580,15 @@ static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
     GemmPlan p;
     const int nsteps = red / BK;
     // Tiles of 256 rows (8 wavefronts, one dequantized slab of W for 256 activation rows) do about twice the work per
-    // CU and unit of time that 128-row tiles do, so they are used from 192 rows on: as they are when there are more
+    // CU and unit of time that 128-row tiles do, so they are used from 129 rows on: as they are when there are more
     // than 128 of them (even 130 of them on 256 CUs beat 260 tiles of 128 rows), otherwise with the reduction split
     // floor(256 / tiles) ways so that every CU gets one workgroup (never more than 256 workgroups: a second, nearly
     // empty round costs more than the split gains).
     const long t256 = (long)(nout / BN) * ((M + 255) / 256);
     int splits = 1;
-    if (t256 > 128 && M >= 192) {
+    if (t256 > 128 && M > 128) {
         p.cfg = 2;
-    } else if (t256 <= 128 && M >= 192 && nsteps >= 8 * (int)(256 / t256) &&
+    } else if (t256 <= 128 && M > 128 && nsteps >= 8 * (int)(256 / t256) &&
                (size_t)(256 / t256 > 8 ? 8 : 256 / t256) * (size_t)M * (size_t)nout * sizeof(float) <= workspace_bytes) {
         p.cfg = 2;                                             // only with room for all its partial tiles
         splits = (int)(256 / t256);
