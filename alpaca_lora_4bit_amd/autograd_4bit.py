@@ -279,11 +279,24 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
               dA  = scaling * dyb^T @ x   [r, K]        dB = scaling * dy^T @ xa   [N, r]
     A: lora_A.weight [r, K], B: lora_B.weight [N, r] (any float dtype; products run in fp16
     with fp32 accumulation, like the reference under autocast).  fp32 / fp16 adapter matrices are
-    read in place by the kernels through strides: no cast, transposed or pre-scaled copies."""
+    read in place by the kernels through strides: no cast, transposed or pre-scaled copies.
+
+    Above matmul_utils_4bit.dense_switch_rows rows the same sums run as dense dequantization + library GEMMs
+    (the rank-r product writes the output once, the big product accumulates onto it)."""
 
     @staticmethod
     def _kernel_dtype(w):
         return w if w.dtype in (torch.float16, torch.float32) else w.float()
+
+    @staticmethod
+    def _dense_product(act, w, small, adapter, scaling, bias=None):
+        """act @ w + scaling * small @ adapter (+ bias), fp16 out; `w`, `adapter` may be transposed views."""
+        adapter = adapter if adapter.dtype == torch.float16 else adapter.to(torch.float16)
+        if bias is not None:
+            out = torch.addmm(bias, small, adapter, alpha=scaling)
+        else:
+            out = torch.mm(small * scaling, adapter)
+        return out.addmm_(act, w)
 
     @staticmethod
     @custom_fwd(device_type='cuda', cast_inputs=None)
@@ -298,8 +311,12 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
         a = AutogradMatmul4bitLora._kernel_dtype(lora_a.detach())
         b = AutogradMatmul4bitLora._kernel_dtype(lora_b.detach())
         xa = quant_hip.lora_down(x2, a)
-        y = quant_hip.gemm_fwd(x2, qweight, zeros, scales, g_idx, groupsize, bias=bias,
-                               xa=xa, lora_bt=b.t(), lora_scale=scaling, out_shape=tuple(x.shape[:-1]) + (N,))
+        if mm4b.use_dense_route(x2.shape[0]):
+            w = mm4b.dense_weight(qweight, scales, zeros, g_idx, groupsize)
+            y = AutogradMatmul4bitLora._dense_product(x2, w, xa, b.t(), scaling, bias).view(tuple(x.shape[:-1]) + (N,))
+        else:
+            y = quant_hip.gemm_fwd(x2, qweight, zeros, scales, g_idx, groupsize, bias=bias,
+                                   xa=xa, lora_bt=b.t(), lora_scale=scaling, out_shape=tuple(x.shape[:-1]) + (N,))
         ctx.save_for_backward(x2, xa, qweight, scales, zeros, g_idx, a, b)
         ctx.scaling = scaling
         ctx.groupsize = groupsize
@@ -318,9 +335,13 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
         dyb = quant_hip.lora_down(dy, b.t())
         dx = da = db = None
         if ctx.needs_input_grad[0]:
-            dx = quant_hip.gemm_bwd_dx(dy, qweight, zeros, scales, g_idx, ctx.groupsize, dyb=dyb, lora_a=a,
-                                       lora_scale=ctx.scaling,
-                                       out_shape=tuple(grad_output.shape[:-1]) + (qweight.shape[0] * 8,))
+            dx_shape = tuple(grad_output.shape[:-1]) + (qweight.shape[0] * 8,)
+            if mm4b.use_dense_route(dy.shape[0]):
+                w = mm4b.dense_weight(qweight, scales, zeros, g_idx, ctx.groupsize)
+                dx = AutogradMatmul4bitLora._dense_product(dy, w.t(), dyb, a, ctx.scaling).view(dx_shape)
+            else:
+                dx = quant_hip.gemm_bwd_dx(dy, qweight, zeros, scales, g_idx, ctx.groupsize, dyb=dyb, lora_a=a,
+                                           lora_scale=ctx.scaling, out_shape=dx_shape)
         r = a.shape[0]
         need_a, need_b = ctx.needs_input_grad[6], ctx.needs_input_grad[7]
         if need_a and need_b and r in quant_hip.LORA_GRAD_RANKS:

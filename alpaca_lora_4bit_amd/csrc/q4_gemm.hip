@@ -658,7 +658,7 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     a.phase_step = env_phase < 0 ? 0 : env_phase;
     const int nout = fwd ? N : K;
     const bool gidx = g_idx != nullptr;
-    // 17..32 rows, forward, no adapter: the weight-streaming kernel (one pass over the packed weights)
+    // 17..64 rows, forward, no adapter: the weight-streaming kernel (one pass over the packed weights)
     if (fwd && a.R == 0 && q4_skinny_applicable(M, K, N, groupsize, gidx) && workspace &&
         workspace_bytes >= q4_skinny_workspace(M, K, N))
         return q4_launch_skinny(act, qweight, qzeros, scales, groupsize, bias, out, M, K, N, workspace, stream);

@@ -6,8 +6,12 @@ What changed underneath (none of it visible in the signatures):
 * rows <= auto_switch_thd (default 16, the most the GEMV kernel takes) go to one GEMV launch
   that reads the packed weights once for all rows; the reference launches one grid slice per row
   and switches to recons + matmul above 8 rows (matmul_utils_4bit.py:15,164-167).
-* larger inputs go to the fused dequant + MFMA GEMM.  No dense [K, N] buffer exists, so
-  `get_buffer` / `cache_buffer` / `buffer_mat_dic` are kept only as inert names.
+* larger inputs go to the fused dequant + MFMA GEMM, which needs no dense [K, N] buffer.
+* above `dense_switch_rows` rows (default 2048) the reference's own scheme is faster again on this GPU and is
+  used: dense dequantization (one launch at 70 % of HBM bandwidth) into a buffer from `get_buffer`, then a
+  library GEMM.  The dequantization is then a small fraction of the product, and the library's GEMM has no
+  dequantization competing with its matrix instructions for issue slots.  `cache_buffer` keeps its meaning
+  (one process-global buffer per shape, or a fresh one per call when False).
 * `act_order` and `faster_mode` no longer select kernels: whether `g_idx` is a real
   permutation is detected per tensor (quant_hip.classify_g_idx).  The reference's default
   kernel ignores g_idx unless the user sets `act_order = True` by hand (:75-87); here a
@@ -34,18 +38,25 @@ faster_mode = 'old_faster'
 valid_faster_mode = ('faster', 'old_faster')
 act_order = False
 cache_buffer = True
+dense_switch_rows = 2048          # rows above this: dense dequant + library GEMM; 0 or None: always the fused GEMM
 
 
-def get_buffer(shape_of_qweight, dtype=torch.float16, device='cuda', bits=4):
-    """Dense [K, N] scratch of the reference (matmul_utils_4bit.py:22-33).  Nothing in this
-    package uses it; it is provided for callers that dequantize explicitly."""
+def get_buffer(shape_of_qweight, dtype=torch.float16, device='cuda', bits=4, zero=True):
+    """Dense [K, N] scratch of the reference (matmul_utils_4bit.py:22-33): used above `dense_switch_rows` rows
+    and by callers that dequantize explicitly.  Like the reference's, the cached buffer is shared by every layer
+    of that shape, so calls on two streams at once must set `cache_buffer = False`."""
     target_shape = (shape_of_qweight[0] * (32 // bits), shape_of_qweight[1])
+    make = torch.zeros if zero else torch.empty
     if not cache_buffer:
-        return torch.zeros(target_shape, dtype=dtype, device=device)
-    buf = buffer_mat_dic.get(target_shape)
-    if buf is None or buf.device != torch.device(device) or buf.dtype != dtype:
-        buf = torch.zeros(target_shape, dtype=dtype, device=device)
-        buffer_mat_dic[target_shape] = buf
+        return make(target_shape, dtype=dtype, device=device)
+    device = torch.device(device)
+    if device.type == 'cuda' and device.index is None:
+        device = torch.device('cuda', torch.cuda.current_device())
+    key = (target_shape, device)
+    buf = buffer_mat_dic.get(key)
+    if buf is None or buf.dtype != dtype:
+        buf = make(target_shape, dtype=dtype, device=device)
+        buffer_mat_dic[key] = buf
     return buf
 
 
@@ -79,9 +90,22 @@ def _matmul4bit_v2(x, qweight, scales, zeros, g_idx, groupsize=None):
     return y.to(dtype)
 
 
+def use_dense_route(rows):
+    """True when `rows` activation rows go through dense dequantization + a library GEMM."""
+    return bool(dense_switch_rows) and rows > dense_switch_rows
+
+
+def dense_weight(qweight, scales, zeros, g_idx, groupsize=None):
+    """W fp16 [K, N] in the buffer of `get_buffer` (every element is overwritten)."""
+    buf = get_buffer(qweight.shape, dtype=torch.float16, device=qweight.device, zero=False)
+    return quant_hip.dequant(qweight, zeros, _half_scales(scales), g_idx, _groupsize_of(qweight, scales, groupsize),
+                             out=buf)
+
+
 def _matmul4bit_v2_recons(x, qweight, scales, zeros, g_idx, transpose=False, groupsize=None):
-    """x @ W (or x @ W.T with transpose=True) through the fused dequant-MFMA GEMM; the
-    reference dequantizes into a dense buffer and calls torch.matmul (matmul_utils_4bit.py:114-127)."""
+    """x @ W (or x @ W.T with transpose=True).  Up to `dense_switch_rows` rows through the fused dequant-MFMA GEMM;
+    above, as the reference does for every size: dequantize into a dense buffer and call torch.matmul
+    (matmul_utils_4bit.py:114-127)."""
     if debug:
         print('_matmul4bit_v2_recons')
     if not transpose:
@@ -90,6 +114,8 @@ def _matmul4bit_v2_recons(x, qweight, scales, zeros, g_idx, transpose=False, gro
         assert qweight.shape[1] == x.shape[-1]
     gs = _groupsize_of(qweight, scales, groupsize)
     lead = tuple(x.shape[:-1])
+    if use_dense_route(_rows(x)) and x.is_cuda:
+        return _dense_matmul(x, dense_weight(qweight, scales, zeros, g_idx, gs), transpose)
     if not transpose:
         return quant_hip.gemm_fwd(x, qweight, zeros, _half_scales(scales), g_idx, gs,
                                   out_shape=lead + (qweight.shape[1],))

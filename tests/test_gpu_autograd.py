@@ -229,3 +229,66 @@ def test_backend_switch_and_errors():
         autograd_4bit.switch_backend_to("triton")
     with pytest.raises(ValueError):
         autograd_4bit.switch_backend_to("metal")
+
+
+@pytest.mark.parametrize("act", [False, True])
+def test_dense_route_above_the_row_switch(oracle, act):
+    """Above matmul_utils_4bit.dense_switch_rows rows the product runs as dense dequantization + library GEMM (the
+    reference's recons scheme, matmul_utils_4bit.py:114-127): same values as the fused GEMM for the plain layer
+    (no-grad and autograd, with bias) and for the LoRA layer (y, dx, dA, dB), and the fused kernels are not called."""
+    import torch
+    from alpaca_lora_4bit_amd import autograd_4bit, matmul_utils_4bit as mm4b, models, quant_hip
+    K, N, r, rows = 256, 384, 8, 2304
+    assert mm4b.dense_switch_rows == 2048
+    layer = oracle.make_layer(K, N, 128, act_order=act, seed=31)
+    A, B = oracle.make_lora(K, N, r, seed=31)
+    x = oracle.make_activations(rows, K, seed=61)
+    dy = oracle.make_activations(rows, N, seed=62)
+    bias = (np.random.default_rng(7).standard_normal(N) * 0.1).astype(np.float16)
+    W = oracle.dequant_v2(layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"]).astype(np.float64)
+
+    fused_calls = []
+    real_fwd, real_bwd = quant_hip.gemm_fwd, quant_hip.gemm_bwd_dx
+    quant_hip.gemm_fwd = lambda *a, **k: (fused_calls.append("fwd"), real_fwd(*a, **k))[1]
+    quant_hip.gemm_bwd_dx = lambda *a, **k: (fused_calls.append("bwd"), real_bwd(*a, **k))[1]
+    try:
+        plain = _fill(autograd_4bit.Autograd4bitQuantLinear(K, N, groupsize=128), layer)
+        plain.bias = torch.from_numpy(bias).cuda()
+        yref = x.astype(np.float64) @ W + bias.astype(np.float64)
+        xt = torch.from_numpy(x).cuda()
+        with torch.no_grad():
+            assert rel_err(plain(xt).cpu().numpy(), yref) <= TOL
+        xg = xt.clone().requires_grad_(True)
+        y = plain(xg)
+        y.backward(torch.from_numpy(dy).cuda())
+        assert rel_err(y.detach().cpu().numpy(), yref) <= TOL
+        assert rel_err(xg.grad.cpu().numpy(), dy.astype(np.float64) @ W.T) <= TOL
+
+        m = models.Linear4bitLt("default", K, N, 128, False, r=r, lora_alpha=2 * r, lora_dropout=0.0).cuda()
+        _fill(m, layer)
+        m.bias = torch.from_numpy(bias).cuda()
+        m.lora_A["default"].weight.data = torch.from_numpy(A).cuda()
+        m.lora_B["default"].weight.data = torch.from_numpy(B).cuda()
+        yl = oracle.lora_forward(x, W, A, B, 2.0) + bias.astype(np.float64)
+        dxl, dAl, dBl = oracle.lora_backward(x, dy, W, A, B, 2.0)
+        xg = xt.clone().requires_grad_(True)
+        with torch.amp.autocast(device_type="cuda"):
+            y = m(xg)
+        y.backward(torch.from_numpy(dy).cuda())
+        assert y.dtype == torch.float16 and y.shape == (rows, N)
+        assert rel_err(y.detach().cpu().numpy(), yl) <= TOL
+        assert rel_err(xg.grad.cpu().numpy(), dxl) <= TOL
+        assert rel_err(m.lora_A["default"].weight.grad.cpu().numpy(), dAl) <= TOL
+        assert rel_err(m.lora_B["default"].weight.grad.cpu().numpy(), dBl) <= TOL
+        assert fused_calls == []
+
+        # one row fewer than the switch: the fused kernels again, same numbers
+        mm4b.dense_switch_rows = rows
+        try:
+            with torch.no_grad():
+                assert rel_err(plain(xt).cpu().numpy(), yref) <= TOL
+        finally:
+            mm4b.dense_switch_rows = 2048
+        assert fused_calls == ["fwd"]
+    finally:
+        quant_hip.gemm_fwd, quant_hip.gemm_bwd_dx = real_fwd, real_bwd
