@@ -55,7 +55,9 @@ struct GemmArgs {
     half_t* out;              // fwd: y [M,N]      bwd: dx [M,K]
     int M, K, N, G;
     int phase_step;           // rotation of the reduction loop per row tile, in steps of 64
-    float* part;              // split-K: fp32 partial outputs [gridDim.z][M][NOUT] (gridDim.z > 1 only)
+    float* part;              // split-K: fp32 partial outputs [gridDim.z][M][part_cols] (gridDim.z > 1 only)
+    int col_tile0;            // first column tile of this launch (a launch may cover a range of column tiles)
+    int part_cols;            // columns held by `part`: those of this launch's column tiles
 };
 
 // Which output tile a workgroup computes, and where in the reduction it starts.
@@ -69,13 +71,14 @@ struct GemmArgs {
 struct TileMap {
     int tile_c, tile_r, phase;
 };
-__device__ __forceinline__ TileMap map_tile(int phase_step, int nsteps) {   // nsteps: steps of THIS workgroup
+__device__ __forceinline__ TileMap map_tile(int phase_step, int nsteps, int col_tile0) {   // nsteps: steps of THIS workgroup
     const int nc = gridDim.x, nr = gridDim.y, total = nc * nr;
     int id = blockIdx.y * nc + blockIdx.x;
     if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
     TileMap m;
     m.tile_c = id / nr;
     m.tile_r = id - m.tile_c * nr;
+    m.tile_c += col_tile0;
     m.phase = (m.tile_r * phase_step) % nsteps;
     return m;
 }
@@ -328,7 +331,7 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     const int NOUT = FWD ? a.N : a.K;
     const int RED = FWD ? a.K : a.N;
     const StepRange sr = split_steps(RED / BK);
-    const TileMap tm = map_tile(a.phase_step, sr.cnt);
+    const TileMap tm = map_tile(a.phase_step, sr.cnt, a.col_tile0);
     const int m0 = tm.tile_r * BM;
     const int c0 = tm.tile_c * BN;           // first output column of the tile
     const int rows_valid = min(BM, a.M - m0);
@@ -488,7 +491,7 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     if (gridDim.z > 1) {
         // split-K: fp32 partial sums straight from the accumulators (32 lanes cover one 128-byte row segment);
         // the bias rides with split 0, the reduction kernel adds the splits in order and rounds once
-        float* const pz = a.part + (size_t)blockIdx.z * a.M * NOUT;
+        float* const pz = a.part + (size_t)blockIdx.z * a.M * a.part_cols - (size_t)a.col_tile0 * BN;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -498,7 +501,7 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int m = m0 + wm * WROWS + 32 * i + 8 * (r >> 2) + lrow + (r & 3);
-                    if (m < a.M) pz[(size_t)m * NOUT + col] = acc[i][j][r] + bv;
+                    if (m < a.M) pz[(size_t)m * a.part_cols + col] = acc[i][j][r] + bv;
                 }
             }
         return;
@@ -547,37 +550,69 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __
     *reinterpret_cast<half4_t*>(out + i) = h;
 }
 
+// The same for partial sums that cover only the columns [col0, col0 + part_cols) of the output rows.
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_cols_kernel(const float* __restrict__ part, half_t* __restrict__ out,
+                                                                      int M, int part_cols, int out_cols, int col0, int splits) {
+    const long total = (long)M * part_cols;
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= total) return;                       // part_cols is a multiple of 128
+    float4_t v = *reinterpret_cast<const float4_t*>(part + i);
+    for (int s = 1; s < splits; ++s) {
+        const float4_t u = *reinterpret_cast<const float4_t*>(part + (size_t)s * total + i);
+        v[0] += u[0]; v[1] += u[1]; v[2] += u[2]; v[3] += u[3];
+    }
+    const long m = i / part_cols, c = i - m * part_cols;
+    half4_t h = {(half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3]};
+    *reinterpret_cast<half4_t*>(out + m * out_cols + col0 + c) = h;
+}
+
+// tail_cols > 0: the last tail_cols column tiles run as a second launch with the reduction split tail_splits ways
+// (the main launch then covers whole rounds of the CUs, and the remainder does not cost a whole round).
 template <int BM, int WGM, bool FWD, bool GIDX>
-static hipError_t launch_gemm(const GemmArgs& a, int nout, int splits, hipStream_t stream) {
-    const dim3 grid(nout / BN, (a.M + BM - 1) / BM, splits);
-    hipLaunchKernelGGL((gemm_kernel<BM, WGM, FWD, GIDX>), grid, dim3(128 * WGM), 0, stream, a);
+static hipError_t launch_gemm(GemmArgs a, int nout, int splits, int tail_cols, int tail_splits, hipStream_t stream) {
+    const int nc = nout / BN, nr = (a.M + BM - 1) / BM;
+    a.col_tile0 = 0;
+    a.part_cols = nout;
+    hipLaunchKernelGGL((gemm_kernel<BM, WGM, FWD, GIDX>), dim3(nc - tail_cols, nr, splits), dim3(128 * WGM), 0, stream, a);
     if (splits > 1) {
         const long total = (long)a.M * nout;
         hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream,
                            a.part, a.out, total, splits);
     }
+    if (tail_cols > 0) {
+        a.col_tile0 = nc - tail_cols;
+        a.part_cols = tail_cols * BN;
+        hipLaunchKernelGGL((gemm_kernel<BM, WGM, FWD, GIDX>), dim3(tail_cols, nr, tail_splits), dim3(128 * WGM), 0, stream, a);
+        const long total = (long)a.M * a.part_cols;
+        hipLaunchKernelGGL(gemm_splitk_reduce_cols_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream,
+                           a.part, a.out, a.M, a.part_cols, nout, a.col_tile0 * BN, tail_splits);
+    }
     return hipGetLastError();
 }
 
+struct GemmPlan {
+    int cfg, splits;
+    int tail_cols, tail_splits;      // cfg 2 only: column tiles of the split second launch (0: none)
+};
+
 template <bool FWD, bool GIDX>
-static hipError_t launch_gemm_cfg(int cfg, const GemmArgs& a, int nout, int splits, hipStream_t stream) {
-    switch (cfg) {
-        case 0: return launch_gemm<128, 2, FWD, GIDX>(a, nout, splits, stream);    // 128 x 128, 4 wavefronts of 64 x 64
-        case 1: return launch_gemm<256, 2, FWD, GIDX>(a, nout, splits, stream);    // 256 x 128, 4 wavefronts of 128 x 64
-        default: return launch_gemm<256, 4, FWD, GIDX>(a, nout, splits, stream);   // 256 x 128, 8 wavefronts of 64 x 64
+static hipError_t launch_gemm_cfg(const GemmPlan& p, const GemmArgs& a, int nout, hipStream_t stream) {
+    switch (p.cfg) {
+        case 0: return launch_gemm<128, 2, FWD, GIDX>(a, nout, p.splits, 0, 1, stream);    // 128 x 128, 4 wavefronts of 64 x 64
+        case 1: return launch_gemm<256, 2, FWD, GIDX>(a, nout, p.splits, 0, 1, stream);    // 256 x 128, 4 wavefronts of 128 x 64
+        default: return launch_gemm<256, 4, FWD, GIDX>(a, nout, p.splits, p.tail_cols, p.tail_splits, stream);   // 256 x 128, 8 wavefronts of 64 x 64
     }
 }
 
 // Launch plan shared by q4_launch_gemm and q4_gemm_plan_workspace.  Few output tiles (small M) leave most CUs
 // idle while each tile walks the whole reduction: the reduction is then split over gridDim.z workgroups that
 // write fp32 partial tiles, about 1.5 workgroups per CU in total.
-struct GemmPlan {
-    int cfg, splits;
-};
 static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
     static const int env_cfg = getenv("Q4_GEMM_CFG") ? atoi(getenv("Q4_GEMM_CFG")) : -1;
     static const int env_splits = getenv("Q4_GEMM_SPLITS") ? atoi(getenv("Q4_GEMM_SPLITS")) : 0;
+    static const int env_tail = getenv("Q4_GEMM_TAIL") ? atoi(getenv("Q4_GEMM_TAIL")) : 1;
     GemmPlan p;
+    p.tail_cols = 0; p.tail_splits = 1;
     const int nsteps = red / BK;
     // Tiles of 256 rows (8 wavefronts, one dequantized slab of W for 256 activation rows) do about twice the work per
     // CU and unit of time that 128-row tiles do, so they are used from 129 rows on: as they are when there are more
@@ -588,6 +623,21 @@ static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
     int splits = 1;
     if (t256 > 128 && M > 128) {
         p.cfg = 2;
+        // More tiles than CUs and a last round that fills at most half of them: the column tiles of that
+        // remainder run as a second launch with the reduction split so that it takes a fraction of a round.
+        const int nr = (M + 255) / 256;
+        const long rem = t256 % 256;
+        if (env_tail && t256 > 256 && rem > 0) {
+            const int tcols = (int)((rem + nr - 1) / nr);
+            const long tt = (long)tcols * nr;
+            int ts = tt <= 128 ? (int)(256 / tt) : 1;
+            if (ts > 8) ts = 8;
+            while (ts > 1 && nsteps < 8 * ts) --ts;
+            if (ts > 1 && (size_t)ts * (size_t)M * (size_t)tcols * BN * sizeof(float) <= workspace_bytes) {
+                p.tail_cols = tcols;
+                p.tail_splits = ts;
+            }
+        }
     } else if (t256 <= 128 && M > 128 && nsteps >= 8 * (int)(256 / t256) &&
                (size_t)(256 / t256 > 8 ? 8 : 256 / t256) * (size_t)M * (size_t)nout * sizeof(float) <= workspace_bytes) {
         p.cfg = 2;                                             // only with room for all its partial tiles
@@ -604,6 +654,7 @@ static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
     }
     if (env_cfg >= 0 && env_cfg != p.cfg) {                    // experiments: forced tile shape, splits as before
         p.cfg = env_cfg;
+        p.tail_cols = 0;
         const int bm = p.cfg == 0 ? 128 : 256;
         const long tiles = (long)(nout / BN) * ((M + bm - 1) / bm);
         splits = 1;
@@ -613,7 +664,7 @@ static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
             if (splits > nsteps / 4) splits = nsteps / 4;
         }
     }
-    if (env_splits > 0) splits = env_splits > nsteps ? nsteps : env_splits;
+    if (env_splits > 0) { splits = env_splits > nsteps ? nsteps : env_splits; p.tail_cols = 0; }
     while (splits > 1 && (size_t)splits * (size_t)M * (size_t)nout * sizeof(float) > workspace_bytes) --splits;
     p.splits = splits < 1 ? 1 : splits;
     return p;
@@ -666,8 +717,8 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     const GemmPlan p = plan_gemm(M, fwd ? K : N, nout, workspace ? workspace_bytes : 0);
     a.part = reinterpret_cast<float*>(workspace);
     hipError_t e;
-    if (fwd) e = gidx ? launch_gemm_cfg<true, true>(p.cfg, a, nout, p.splits, stream) : launch_gemm_cfg<true, false>(p.cfg, a, nout, p.splits, stream);
-    else e = gidx ? launch_gemm_cfg<false, true>(p.cfg, a, nout, p.splits, stream) : launch_gemm_cfg<false, false>(p.cfg, a, nout, p.splits, stream);
+    if (fwd) e = gidx ? launch_gemm_cfg<true, true>(p, a, nout, stream) : launch_gemm_cfg<true, false>(p, a, nout, stream);
+    else e = gidx ? launch_gemm_cfg<false, true>(p, a, nout, stream) : launch_gemm_cfg<false, false>(p, a, nout, stream);
     return e == hipSuccess ? 0 : -4;
 }
 
@@ -677,6 +728,7 @@ extern "C" size_t q4_gemm_plan_workspace(int fwd, int M, int K, int N) {
     const int nout = fwd ? N : K;
     const GemmPlan p = plan_gemm(M, fwd ? K : N, nout, ~(size_t)0);
     size_t need = p.splits > 1 ? (size_t)p.splits * (size_t)M * (size_t)nout * sizeof(float) : 0;
+    if (p.tail_cols > 0) need = (size_t)p.tail_splits * (size_t)M * (size_t)p.tail_cols * BN * sizeof(float);
     if (fwd && M > 16 && M <= 64) {               // the skinny kernel's partial rows (it may or may not apply)
         const size_t sk = q4_skinny_workspace(M, K, N);
         if (sk > need) need = sk;

@@ -170,3 +170,47 @@ def test_gemm_forward_streaming_kernel_several_strips_per_workgroup(oracle, M, K
     y2 = quant_hip.gemm_fwd(torch.from_numpy(x).cuda(), t["qweight"], t["qzeros"], t["scales"], None, 128)
     assert y.shape == (M, N) and torch.equal(y, y2)
     assert np.abs(y.float().cpu().numpy() - ref).max() <= 1e-2 * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("act", [False, True])
+@pytest.mark.parametrize("M,red,nout,tail_cols,tail_splits", [(1024, 1024, 11008, 22, 2), (520, 1024, 11008, 1, 2),
+                                                              (1536, 4096, 11008, 1, 8)])
+def test_gemm_remainder_tiles_run_as_a_split_second_launch(oracle, M, red, nout, tail_cols, tail_splits, act):
+    """More 256-row tiles than CUs with a last round that fills at most half of them: the remainder's column tiles
+    go to a second launch with the reduction split; forward (bias + adapter) and backward-dx (adapter) must cover
+    every column exactly once."""
+    import torch
+    from alpaca_lora_4bit_amd import _lib, quant_hip
+    r, scaling = 8, 2.0
+    for fwd in (True, False):
+        K, N = (red, nout) if fwd else (nout, red)
+        assert _lib.lib().q4_gemm_workspace_bytes(int(fwd), M, K, N) == tail_splits * M * tail_cols * 128 * 4
+        layer = oracle.make_layer(K, N, 128, act_order=act, seed=53)
+        t = to_cuda_layer(layer)
+        A, B = oracle.make_lora(K, N, r, seed=53)
+        A16, B16 = A.astype(np.float16), B.astype(np.float16)
+        W = oracle.dequant_v2(layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"]).astype(np.float64)
+        x = oracle.make_activations(M, K, seed=43)
+        dy = oracle.make_activations(M, N, seed=44)
+        if fwd:
+            bias = (np.random.default_rng(2).standard_normal(N) * 0.1).astype(np.float16)
+            ref = oracle.lora_forward(x, W, A16, B16, scaling, bias=bias)
+            xt = _t(x)
+            got = quant_hip.gemm_fwd(xt, t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 128, bias=_t(bias),
+                                     xa=xt @ _t(A16).t(), lora_bt=_t(B16).t(), lora_scale=scaling)
+            plain = quant_hip.gemm_fwd(xt, t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 128)
+            ref_plain = x.astype(np.float64) @ W
+        else:
+            ref, _, _ = oracle.lora_backward(x, dy, W, A16, B16, scaling)
+            dyt = _t(dy)
+            got = quant_hip.gemm_bwd_dx(dyt, t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 128,
+                                        dyb=dyt @ _t(B16), lora_a=_t(A16), lora_scale=scaling)
+            plain = quant_hip.gemm_bwd_dx(dyt, t["qweight"], t["qzeros"], t["scales"], t["g_idx"], 128)
+            ref_plain = dy.astype(np.float64) @ W.T
+        torch.cuda.synchronize()
+        for out, want in ((got, ref), (plain, ref_plain)):
+            out = out.cpu().numpy()
+            assert rel_err(out, want) <= TOL
+            edge = (nout // 128 - tail_cols) * 128                  # first column of the second launch
+            assert rel_err(out[:, edge - 128:edge + 128], want[:, edge - 128:edge + 128]) <= TOL
+            assert rel_err(out[:, -128:], want[:, -128:]) <= TOL
