@@ -303,6 +303,8 @@ def gemv_v1(x, qweight, scales, zeros, out=None, accumulate=False, out_shape=Non
     _require(K % 32 == 0 and N % 64 == 0, "K must be a multiple of 32 and N of 64")
     x2 = _flat_half(x, K, dev, "x")
     M = x2.shape[0]
+    if M == 0 and out is None:                              # empty batch: nothing to launch
+        return torch.empty(_out_shape(out_shape, 0, N), dtype=torch.float16, device=dev)
     _require(1 <= M <= MAX_GEMV_ROWS, f"gemv handles 1..{MAX_GEMV_ROWS} rows, got {M}")
     if out is None:
         _require(not accumulate, "accumulate needs an output tensor")
@@ -352,6 +354,8 @@ def gemv(x, qweight, qzeros, scales, g_idx=None, groupsize=None, out=None, accum
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     x2 = _flat_half(x, K, dev, "x")
     M = x2.shape[0]
+    if M == 0 and out is None:                              # empty batch: nothing to launch
+        return torch.empty(_out_shape(out_shape, 0, N), dtype=torch.float16, device=dev)
     _require(1 <= M <= MAX_GEMV_ROWS, f"gemv handles 1..{MAX_GEMV_ROWS} rows, got {M}")
     if out is None:
         _require(not accumulate, "accumulate needs an output tensor")
@@ -413,6 +417,8 @@ def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, 
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     x2 = _flat_half(x, K, dev, "x")
     M = x2.shape[0]
+    if M == 0:                                               # empty batch: nothing to launch
+        return torch.empty(_out_shape(out_shape, 0, N), dtype=torch.float16, device=dev)
     if bias is not None:
         _require(bias.dtype == torch.float16 and tuple(bias.shape) == (N,) and bias.is_contiguous()
                  and bias.device == dev, "bias must be a contiguous float16 [N] tensor on the same device")
@@ -441,6 +447,8 @@ def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=Non
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     dy2 = _flat_half(dy, N, dev, "grad_output")
     M = dy2.shape[0]
+    if M == 0:
+        return torch.empty(_out_shape(out_shape, 0, K), dtype=torch.float16, device=dev)
     plan = _actorder_plan(qweight, scales, g_idx, groupsize, G)
     if plan is not None:
         # dx comes out in sorted row order and is scattered back; the adapter matrix [R, K] is gathered too
@@ -472,7 +480,9 @@ def lora_down(inp, w):
     M, C = inp.shape
     _require(w.dim() == 2 and w.shape[1] == C and w.device == inp.device, "w must be an [R, C] view on the same device")
     R = w.shape[0]
-    _require(1 <= R <= 64 and C % 32 == 0 and M >= 1, "lora_down needs 1 <= R <= 64 and C % 32 == 0")
+    if M == 0:
+        return torch.empty((0, R), dtype=torch.float16, device=inp.device)
+    _require(1 <= R <= 64 and C % 32 == 0, "lora_down needs 1 <= R <= 64 and C % 32 == 0")
     f32 = _adapter_dtype_flag(w, "w")
     sr, sc = w.stride()
     _require(sr >= 1 and sc >= 1, "w must have positive strides")
@@ -493,8 +503,10 @@ def lora_grad(p, inp, alpha, transposed=False):
              and inp.shape[0] == p.shape[0], "inp must be a contiguous float16 [M, C] tensor on the same device")
     M, R = p.shape
     C = inp.shape[1]
-    _require(R in LORA_GRAD_RANKS and C % 8 == 0 and M >= 1, "lora_grad needs R in (8, 16) and C % 8 == 0")
+    _require(R in LORA_GRAD_RANKS and C % 8 == 0, "lora_grad needs R in (8, 16) and C % 8 == 0")
     dev = p.device
+    if M == 0:                                               # empty batch: the gradient is zero
+        return torch.zeros((C, R) if transposed else (R, C), dtype=torch.float32, device=dev)
     if transposed:
         out = torch.empty((C, R), dtype=torch.float32, device=dev)
         sr, sc = 1, R
@@ -523,8 +535,10 @@ def lora_grad_pair(p1, inp1, p2, inp2, alpha):
     _require(p1.shape == p2.shape and p1.device == p2.device, "the two rank-R operands must share shape and device")
     M, R = p1.shape
     C1, C2 = inp1.shape[1], inp2.shape[1]
-    _require(R in LORA_GRAD_RANKS and C1 % 8 == 0 and C2 % 8 == 0 and M >= 1, "lora_grad needs R in (8, 16) and C % 8 == 0")
+    _require(R in LORA_GRAD_RANKS and C1 % 8 == 0 and C2 % 8 == 0, "lora_grad needs R in (8, 16) and C % 8 == 0")
     dev = p1.device
+    if M == 0:
+        return (torch.zeros((R, C1), dtype=torch.float32, device=dev), torch.zeros((C2, R), dtype=torch.float32, device=dev))
     out1 = torch.empty((R, C1), dtype=torch.float32, device=dev)
     out2 = torch.empty((C2, R), dtype=torch.float32, device=dev)
     L = _lib.lib()

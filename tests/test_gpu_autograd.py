@@ -292,3 +292,30 @@ def test_dense_route_above_the_row_switch(oracle, act):
         assert fused_calls == ["fwd"]
     finally:
         quant_hip.gemm_fwd, quant_hip.gemm_bwd_dx = real_fwd, real_bwd
+
+
+@pytest.mark.parametrize("shape", [(0,), (2, 0), (0, 3)])
+def test_empty_batches(oracle, shape):
+    """Inputs without rows ([0, K], [2, 0, K], [0, 3, K]) give outputs without rows, in both modes, and zero
+    adapter gradients; nothing is launched."""
+    import torch
+    from alpaca_lora_4bit_amd import autograd_4bit, models
+    K, N, r = 256, 384, 8
+    layer = oracle.make_layer(K, N, 128, seed=37)
+    plain = _fill(autograd_4bit.Autograd4bitQuantLinear(K, N, groupsize=128), layer)
+    plain.bias = torch.ones(N, dtype=torch.float16, device="cuda")
+    lora = models.Linear4bitLt("default", K, N, 128, False, r=r, lora_alpha=16, lora_dropout=0.0).cuda()
+    _fill(lora, layer)
+    x = torch.zeros(shape + (K,), dtype=torch.float16, device="cuda")
+    for m in (plain, lora):
+        with torch.no_grad():
+            y = m(x)
+        assert y.shape == shape + (N,) and y.dtype == torch.float16
+        xg = x.clone().requires_grad_(True)
+        with torch.amp.autocast(device_type="cuda"):
+            y = m(xg)
+        assert y.shape == shape + (N,)
+        y.sum().backward()
+        assert xg.grad is not None and xg.grad.shape == x.shape
+    for w in (lora.lora_A["default"].weight, lora.lora_B["default"].weight):
+        assert w.grad is not None and float(w.grad.abs().max()) == 0.0
