@@ -7,6 +7,11 @@ Steps as in the reference: load the packed model, `model.half()` and halve `scal
 4-bit layer (`:15-22`), wrap `generate` in autocast (`:24-27`), sample with the reference's settings (`:33-44`:
 temperature 0.9, top-p 0.95, top-k 40, repetition penalty 1.1, 20 new tokens), print the text and the seconds taken.
 `--lora` applies an adapter directory written by `alpaca_lora_4bit_amd.finetune` (or by peft) first.
+
+Two additions for decode speed, both off by default: `--fuse` concatenates q/k/v and gate/up into one launch each
+(model_attn_mlp_patch.make_quant_attn / make_fused_mlp, as the reference's model server does, server/server.py:100-113),
+and `--hip_graph` (greedy only) captures the one-token step once as a HIP graph and replays it per token, which
+removes the host time of the ~1000 small launches a decoder step consists of.
 """
 import argparse
 import time
@@ -30,6 +35,8 @@ def _parse(argv):
     p.add_argument("--prompt", default="I think the meaning of life is")
     p.add_argument("--max_new_tokens", type=int, default=20)
     p.add_argument("--greedy", action="store_true", help="argmax decoding instead of sampling")
+    p.add_argument("--fuse", action="store_true", help="one launch for q+k+v and one for gate+up")
+    p.add_argument("--hip_graph", action="store_true", help="greedy decoding with the token step replayed as a HIP graph")
     return p.parse_args(argv)
 
 
@@ -44,6 +51,51 @@ def prepare_model(model):
             m.scales = m.scales.half()
             m.bias = m.bias.half()
     return model
+
+
+def greedy_generate_graph(model, input_ids, max_new_tokens, eos_token_id=None):
+    """Greedy decoding of one sequence: eager prefill into a static KV cache, then the one-token forward captured
+    once as a HIP graph and replayed for every further token (token id and position live in device buffers that the
+    replays read).  Returns the ids [1, prompt + new] like `generate` does; stops early at `eos_token_id`."""
+    from transformers import StaticCache
+    dev = input_ids.device
+    prompt = input_ids.shape[1]
+    with torch.no_grad():
+        cache = StaticCache(config=model.config, max_cache_len=prompt + max_new_tokens)
+        out = model(input_ids=input_ids, past_key_values=cache, use_cache=True,
+                    cache_position=torch.arange(prompt, device=dev))
+        tok_buf = out.logits[:, -1].argmax(-1, keepdim=True).clone()
+        tokens = [tok_buf.clone()]
+        if max_new_tokens > 1 and not (eos_token_id is not None and int(tok_buf[0, 0]) == eos_token_id):
+            pos_buf = torch.tensor([prompt], device=dev)
+
+            def step():
+                o = model(input_ids=tok_buf, past_key_values=cache, use_cache=True, cache_position=pos_buf)
+                return o.logits[:, -1].argmax(-1, keepdim=True)
+
+            def advance(nxt):
+                tok_buf.copy_(nxt)
+                pos_buf.add_(1)
+                tokens.append(nxt.clone())
+                return eos_token_id is not None and int(nxt[0, 0]) == eos_token_id
+
+            # the second token comes from one eager step (on a side stream, as graph capture wants its warm-up):
+            # every lazy allocation and per-layer check of the kernels' host side has then happened before capture
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                second = step()
+            torch.cuda.current_stream().wait_stream(side)
+            done = advance(second)
+            if not done and max_new_tokens > 2:
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    nxt = step()
+                for _ in range(max_new_tokens - 2):
+                    graph.replay()
+                    if advance(nxt):
+                        break
+    return torch.cat([input_ids] + tokens, dim=1)
 
 
 def main(argv=None):
@@ -65,6 +117,10 @@ def main(argv=None):
     print("Fitting 4bit scales and zeros to half")
     prepare_model(model)
 
+    if args.fuse:
+        from .model_attn_mlp_patch import make_fused_mlp, make_quant_attn
+        print("Fused", make_quant_attn(model), "attention blocks and", make_fused_mlp(model), "MLP blocks")
+
     print("Apply AMP Wrapper ...")
     AMPWrapper(model).apply_generate()
 
@@ -74,9 +130,16 @@ def main(argv=None):
     if args.greedy:
         options.update(do_sample=False, temperature=None, top_p=None, top_k=None)
     start = time.time()
-    with torch.no_grad():
-        generated = model.generate(inputs=batch["input_ids"], **options)
-    text = tokenizer.decode(generated["sequences"].cpu().tolist()[0])
+    if args.hip_graph:
+        if not args.greedy:
+            raise ValueError("--hip_graph decodes greedily: pass --greedy as well")
+        with torch.amp.autocast(device_type="cuda"):
+            sequences = greedy_generate_graph(model, batch["input_ids"], args.max_new_tokens,
+                                              eos_token_id=getattr(tokenizer, "eos_token_id", None))
+    else:
+        with torch.no_grad():
+            sequences = model.generate(inputs=batch["input_ids"], **options)["sequences"]
+    text = tokenizer.decode(sequences.cpu().tolist()[0])
     seconds = time.time() - start
     print(text)
     print(seconds)

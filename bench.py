@@ -228,16 +228,12 @@ def bench_lora_step(reps, seed=5):
                 eager_ms=eager * 1e3, eager_tokens_per_s=M / eager)
 
 
-def bench_llama7b_lora_train_step(reps=4, seed=11, n_layers=32, batch=4, seq=256):
-    """configs[4] of the benchmark definition: random-init 32-layer LLaMA-7B decoder, every q/k/v/o/gate/up/down projection a 4-bit
-    GPTQ layer (groupsize 128), LoRA r=8 alpha=16 on q_proj / v_proj, one forward + backward + AdamW step on
-    batch 4 x seq 256 random token ids under fp16 autocast, gradient checkpointing off.  Eager PyTorch around
-    the HIP kernels (attention = torch SDPA, lm_head = library GEMM)."""
+def _random_llama7b(gen, n_layers=32):
+    """Random-init LLaMA-7B decoder whose q/k/v/o/gate/up/down projections are 4-bit GPTQ layers (groupsize 128),
+    fp16 everywhere else."""
     import torch
     from transformers import LlamaConfig, LlamaForCausalLM
     from alpaca_lora_4bit_amd import autograd_4bit as ag
-    from alpaca_lora_4bit_amd.models import inject_lora_layers
-    gen = torch.Generator(device="cuda").manual_seed(seed)
     config = LlamaConfig(vocab_size=32000, hidden_size=4096, intermediate_size=11008, num_hidden_layers=n_layers,
                          num_attention_heads=32, num_key_value_heads=32, max_position_embeddings=2048,
                          tie_word_embeddings=False)
@@ -270,6 +266,59 @@ def bench_llama7b_lora_train_step(reps=4, seed=11, n_layers=32, batch=4, seq=256
             mod.inv_freq = inv_freq.clone()
             if hasattr(mod, "original_inv_freq"):
                 mod.original_inv_freq = inv_freq.clone()
+    return model
+
+
+def bench_llama7b_decode(new_tokens=64, prompt=16, seed=13):
+    """Greedy generation with the random-init 4-bit LLaMA-7B through transformers' own `generate` (eager PyTorch,
+    KV cache on), batch 1: tokens/s as the reference's inference.py prints it, first with one launch per projection,
+    then with q+k+v and gate+up fused (model_attn_mlp_patch.make_quant_attn / make_fused_mlp), then with the token
+    step replayed as a HIP graph (prefill, capture and replays all inside the timed region)."""
+    import torch
+    from alpaca_lora_4bit_amd.model_attn_mlp_patch import make_fused_mlp, make_quant_attn
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    model = _random_llama7b(gen)
+    model.eval()
+    ids = torch.randint(0, 32000, (1, prompt), device="cuda", generator=gen)
+
+    def run():
+        with torch.no_grad():
+            model.generate(input_ids=ids, max_new_tokens=8, min_new_tokens=8, do_sample=False)       # warm-up
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            out = model.generate(input_ids=ids, max_new_tokens=new_tokens, min_new_tokens=new_tokens, do_sample=False)
+            torch.cuda.synchronize()
+        assert out.shape[1] == prompt + new_tokens
+        return new_tokens / (time.perf_counter() - t0)
+
+    res = {"new_tokens": new_tokens, "prompt": prompt, "tokens_per_s": run()}
+    make_quant_attn(model)
+    make_fused_mlp(model)
+    res["tokens_per_s_fused_qkv_gate_up"] = run()
+    # the same greedy decode with the one-token step replayed as a HIP graph (inference.greedy_generate_graph)
+    from alpaca_lora_4bit_amd.inference import greedy_generate_graph
+    greedy_generate_graph(model, ids, 8)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out = greedy_generate_graph(model, ids, new_tokens)
+    torch.cuda.synchronize()
+    assert out.shape[1] == prompt + new_tokens
+    res["tokens_per_s_fused_hip_graph"] = new_tokens / (time.perf_counter() - t0)
+    del model
+    torch.cuda.empty_cache()
+    return res
+
+
+def bench_llama7b_lora_train_step(reps=4, seed=11, n_layers=32, batch=4, seq=256):
+    """configs[4] of the benchmark definition: random-init 32-layer LLaMA-7B decoder, every q/k/v/o/gate/up/down projection a 4-bit
+    GPTQ layer (groupsize 128), LoRA r=8 alpha=16 on q_proj / v_proj, one forward + backward + AdamW step on
+    batch 4 x seq 256 random token ids under fp16 autocast, gradient checkpointing off.  Eager PyTorch around
+    the HIP kernels (attention = torch SDPA, lm_head = library GEMM)."""
+    import torch
+    from alpaca_lora_4bit_amd import autograd_4bit as ag
+    from alpaca_lora_4bit_amd.models import inject_lora_layers
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    model = _random_llama7b(gen, n_layers)
     lora = inject_lora_layers(model, target_modules=("q_proj", "v_proj"), r=8, lora_alpha=16)
     with torch.no_grad():
         for l in lora.values():
@@ -386,6 +435,8 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--llama7b-step-only", action="store_true",
                     help="run only the config-4 full-model LoRA training step (32-layer LLaMA-7B shapes, random init)")
+    ap.add_argument("--llama7b-decode-only", action="store_true",
+                    help="run only the greedy decode of the random-init 4-bit LLaMA-7B through transformers' generate")
     ap.add_argument("--dequant-only", action="store_true",
                     help="run only the dense dequantization of a 4096x11008 layer (short run for profiling)")
     ap.add_argument("--lora-step-only", action="store_true",
@@ -402,6 +453,10 @@ def main():
     torch.cuda.set_device(0)
     from alpaca_lora_4bit_amd import quant_hip  # noqa: F401  (fails loudly if the HIP library is missing)
 
+    if args.llama7b_decode_only:
+        r = bench_llama7b_decode()
+        print(json.dumps({"workload": "llama7b_greedy_decode_b1", **{k: (round(v, 2) if isinstance(v, float) else v) for k, v in r.items()}}))
+        return
     if args.llama7b_step_only:
         r = bench_llama7b_lora_train_step(max(args.steps, 2))
         print(json.dumps({"workload": "config4_llama7b_lora_train_step_b4_s256", **{k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()}}))
@@ -479,6 +534,11 @@ def main():
                                                                   for k, v in c4.items()}
         except Exception as e:                       # the headline line must not depend on the installed transformers
             extra["config4_llama7b_lora_train_step_b4_s256"] = {"error": f"{type(e).__name__}: {e}"[:300]}
+        try:
+            dec = bench_llama7b_decode()
+            extra["llama7b_greedy_decode_b1"] = {k: (round(v, 2) if isinstance(v, float) else v) for k, v in dec.items()}
+        except Exception as e:
+            extra["llama7b_greedy_decode_b1"] = {"error": f"{type(e).__name__}: {e}"[:300]}
         out["extra"] = extra
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()

@@ -93,3 +93,38 @@ def test_finetune_module_on_alpaca_records_with_evaluation(tmp_path, oracle):
     losses = [h["loss"] for h in trainer.state.log_history if "loss" in h]
     assert evals and all(e == e and e > 0 for e in evals) and losses and all(l == l for l in losses)
     assert os.path.exists(os.path.join(out, "adapter_model.safetensors"))
+
+
+def test_hip_graph_decode_gives_the_eager_tokens(tmp_path, oracle):
+    """inference.greedy_generate_graph: every replay of the captured one-token step (with host reads and eager
+    copies between the replays) must pick the token that transformers' eager `generate` picks; plain layers, fused
+    q+k+v / gate+up layers, and the command-line flow with an adapter."""
+    from alpaca_lora_4bit_amd import autograd_4bit as ag, inference
+    from alpaca_lora_4bit_amd.model_attn_mlp_patch import make_fused_mlp, make_quant_attn
+    ckpt = str(tmp_path / "ckpt")
+    build(ckpt, oracle, seed=8, with_tokenizer=True)
+    weights = os.path.join(ckpt, "model.safetensors")
+    model, tokenizer = ag.load_llama_model_4bit_low_ram(ckpt, weights, groupsize=GROUPSIZE, half=True, device_map={"": 0})
+    ids = torch.tensor([[1] + [7 + (13 * i) % 180 for i in range(9)]]).cuda()
+    new = 24
+    for fused in (False, True):
+        if fused:
+            assert make_quant_attn(model) == 2 and make_fused_mlp(model) == 2
+        with torch.no_grad():
+            want = model.generate(input_ids=ids, max_new_tokens=new, min_new_tokens=new, do_sample=False)
+        # eos id -1 never matches: it makes the loop read every token on the host between two replays
+        got = inference.greedy_generate_graph(model, ids, new, eos_token_id=-1 if fused else None)
+        assert got.shape == want.shape == (1, ids.shape[1] + new)
+        assert got.tolist() == want.tolist()
+        assert len(set(want[0, ids.shape[1]:].tolist())) > 3             # not a degenerate constant continuation
+    # the flow from the command line with --fuse and --hip_graph: plain argmax decoding (no repetition penalty)
+    args = [ckpt, weights, "--groupsize", str(GROUPSIZE), "--prompt", "alpha beta gamma", "--max_new_tokens", "12",
+            "--greedy"]
+    prompt = tokenizer("alpha beta gamma", return_tensors="pt", add_special_tokens=False)["input_ids"].cuda()
+    with torch.no_grad():
+        want = model.generate(input_ids=prompt, max_new_tokens=12, do_sample=False,
+                              eos_token_id=getattr(tokenizer, "eos_token_id", None))
+    text_graph, _ = inference.main(args + ["--fuse", "--hip_graph"])
+    assert text_graph == tokenizer.decode(want[0].tolist())
+    with pytest.raises(ValueError):
+        inference.main(args[:-1] + ["--hip_graph"])
