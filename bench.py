@@ -14,6 +14,7 @@ restatement of the reference's recons+matmul algorithm on a bounded sample.
 Secondary figures (M=4/16, config 0, the config-2 LoRA fwd+bwd step, config 3) go under "extra".
 """
 import argparse
+import contextlib
 import json
 import os
 import sys
@@ -258,7 +259,8 @@ def _random_llama7b(gen, n_layers=32):
                 p_.normal_(0, 0.02, generator=gen)
             else:
                 p_.fill_(1.0)
-    ag.model_to_half(model)
+    with contextlib.redirect_stdout(sys.stderr):     # stdout carries the one JSON line only
+        ag.model_to_half(model)
     head_dim = config.hidden_size // config.num_attention_heads
     inv_freq = 1.0 / (10000.0 ** (torch.arange(0, head_dim, 2, device="cuda", dtype=torch.float32) / head_dim))
     for mod in model.modules():                      # rotary tables are plain buffers that to_empty left blank
@@ -529,13 +531,15 @@ def main():
         g3 = bench_gemm_only(512, 5120, 13824, True, 10)
         extra["config3_actorder_M512"] = {k: {kk: round(vv, 4) for kk, vv in v.items()} for k, v in g3.items()}
         try:
-            c4 = bench_llama7b_lora_train_step(4)
+            with contextlib.redirect_stdout(sys.stderr):
+                c4 = bench_llama7b_lora_train_step(4)
             extra["config4_llama7b_lora_train_step_b4_s256"] = {k: (round(v, 4) if isinstance(v, float) else v)
                                                                   for k, v in c4.items()}
         except Exception as e:                       # the headline line must not depend on the installed transformers
             extra["config4_llama7b_lora_train_step_b4_s256"] = {"error": f"{type(e).__name__}: {e}"[:300]}
         try:
-            dec = bench_llama7b_decode()
+            with contextlib.redirect_stdout(sys.stderr):
+                dec = bench_llama7b_decode()
             extra["llama7b_greedy_decode_b1"] = {k: (round(v, 2) if isinstance(v, float) else v) for k, v in dec.items()}
         except Exception as e:
             extra["llama7b_greedy_decode_b1"] = {"error": f"{type(e).__name__}: {e}"[:300]}
