@@ -118,9 +118,9 @@ int q4_gemv_v1_f16(const void *x, const int32_t *qweight, const void *scales, co
  * Both GEMM entry points need K % 128 == 0, N % 128 == 0, K*N < 2^33, and with g_idx == NULL also
  * groupsize % 64 == 0 and every |scale| < 64 (the sequential-group dequant forms s*q with a fused
  * multiply-add on 1024+q; pass g_idx to lift the restriction on the scales).
- * `workspace` (optional, may be NULL; 256-byte aligned, contents irrelevant): with few output tiles (small M)
- * the reduction is split over several workgroups per tile that leave fp32 partial tiles in it, added in a
- * fixed order by a second kernel.  q4_gemm_workspace_bytes(fwd, M, K, N) is the size that allows the
+ * `workspace` (optional, may be NULL; 256-byte aligned, contents irrelevant): with few output tiles (small M),
+ * and for the tiles of a last round that would fill at most half of the CUs, the reduction is split over
+ * several workgroups per tile that leave fp32 partial tiles in it, added in a fixed order by a second kernel.  q4_gemm_workspace_bytes(fwd, M, K, N) is the size that allows the
  * preferred split (0 when none is wanted); a smaller workspace means fewer splits, none means no split. */
 size_t q4_gemm_workspace_bytes(int fwd, int M, int K, int N);
 int q4_gemm_fwd_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
