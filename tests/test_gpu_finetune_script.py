@@ -120,6 +120,19 @@ def test_hip_graph_decode_gives_the_eager_tokens(tmp_path, oracle, act_order):
         assert got.shape == want.shape == (1, ids.shape[1] + new)
         assert got.tolist() == want.tolist()
         assert len(set(want[0, ids.shape[1]:].tolist())) > 3             # not a degenerate constant continuation
+    # layers with a LoRA adapter (the three-launch decode path of Linear4bitLt) inside the captured step
+    from alpaca_lora_4bit_amd import models
+    lora_model, _ = ag.load_llama_model_4bit_low_ram(ckpt, weights, groupsize=GROUPSIZE, half=True, device_map={"": 0})
+    layers = models.inject_lora_layers(lora_model, target_modules=("q_proj", "v_proj"), r=8, lora_alpha=16)
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    with torch.no_grad():
+        for l in layers.values():
+            l.lora_B["default"].weight.normal_(0, 0.2, generator=gen)
+    lora_model.eval()
+    with torch.no_grad(), torch.amp.autocast(device_type="cuda"):
+        want = lora_model.generate(input_ids=ids, max_new_tokens=new, min_new_tokens=new, do_sample=False)
+        got = inference.greedy_generate_graph(lora_model, ids, new)
+    assert got.tolist() == want.tolist()
     # the flow from the command line with --fuse and --hip_graph: plain argmax decoding (no repetition penalty)
     args = [ckpt, weights, "--groupsize", str(GROUPSIZE), "--prompt", "alpha beta gamma", "--max_new_tokens", "12",
             "--greedy"]
