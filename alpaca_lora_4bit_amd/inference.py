@@ -10,8 +10,9 @@ temperature 0.9, top-p 0.95, top-k 40, repetition penalty 1.1, 20 new tokens), p
 
 Two additions for decode speed, both off by default: `--fuse` concatenates q/k/v and gate/up into one launch each
 (model_attn_mlp_patch.make_quant_attn / make_fused_mlp, as the reference's model server does, server/server.py:100-113),
-and `--hip_graph` (greedy only) captures the one-token step once as a HIP graph and replays it per token, which
-removes the host time of the ~1000 small launches a decoder step consists of.
+and `--hip_graph` captures the one-token step once as a HIP graph and replays it per token, which removes the host
+time of the ~1000 small launches a decoder step consists of; the choice of the next token (argmax with `--greedy`,
+otherwise the reference's sampling settings) runs eagerly between two replays.
 """
 import argparse
 import time
@@ -36,7 +37,7 @@ def _parse(argv):
     p.add_argument("--max_new_tokens", type=int, default=20)
     p.add_argument("--greedy", action="store_true", help="argmax decoding instead of sampling")
     p.add_argument("--fuse", action="store_true", help="one launch for q+k+v and one for gate+up")
-    p.add_argument("--hip_graph", action="store_true", help="greedy decoding with the token step replayed as a HIP graph")
+    p.add_argument("--hip_graph", action="store_true", help="decode with the token step replayed as a HIP graph")
     return p.parse_args(argv)
 
 
@@ -53,49 +54,89 @@ def prepare_model(model):
     return model
 
 
-def greedy_generate_graph(model, input_ids, max_new_tokens, eos_token_id=None):
-    """Greedy decoding of one sequence: eager prefill into a static KV cache, then the one-token forward captured
-    once as a HIP graph and replayed for every further token (token id and position live in device buffers that the
-    replays read).  Returns the ids [1, prompt + new] like `generate` does; stops early at `eos_token_id`."""
+def _token_picker(sampling):
+    """Returns pick(ids_so_far, logits) -> next token [1, 1].  `sampling` None: argmax.  Otherwise a dict with the
+    reference's settings (inference.py:33-44: repetition_penalty, temperature, top_k, top_p) applied through
+    transformers' own logits processors in the order `generate` applies them, then one multinomial draw."""
+    if sampling is None:
+        return lambda ids, logits: logits.argmax(-1, keepdim=True)
+    from transformers import (LogitsProcessorList, RepetitionPenaltyLogitsProcessor, TemperatureLogitsWarper,
+                              TopKLogitsWarper, TopPLogitsWarper)
+    procs = LogitsProcessorList()
+    if sampling.get("repetition_penalty", 1.0) != 1.0:
+        procs.append(RepetitionPenaltyLogitsProcessor(penalty=sampling["repetition_penalty"]))
+    if sampling.get("temperature", 1.0) != 1.0:
+        procs.append(TemperatureLogitsWarper(sampling["temperature"]))
+    if sampling.get("top_k"):
+        procs.append(TopKLogitsWarper(top_k=sampling["top_k"]))
+    if sampling.get("top_p", 1.0) < 1.0:
+        procs.append(TopPLogitsWarper(top_p=sampling["top_p"]))
+
+    def pick(ids, logits):
+        scores = procs(ids, logits.float())
+        return torch.multinomial(torch.softmax(scores, dim=-1), num_samples=1)
+    return pick
+
+
+def generate_graph(model, input_ids, max_new_tokens, eos_token_id=None, sampling=None, use_graph=True):
+    """Decoding of one sequence with the model's one-token forward captured once as a HIP graph and replayed for
+    every further token: eager prefill into a static KV cache, the second token from one eager step (the warm-up
+    that graph capture wants: every lazy allocation and per-layer check of the kernels' host side happens there),
+    then replays.  Token id and position live in device buffers that the replays read; the choice of the next
+    token (argmax, or the logits processors + multinomial of `sampling`) runs eagerly between two replays.
+    `use_graph=False` runs the same loop without capture.  Returns the ids [1, prompt + new] like `generate`;
+    stops early at `eos_token_id`."""
     from transformers import StaticCache
     dev = input_ids.device
     prompt = input_ids.shape[1]
+    pick = _token_picker(sampling)
     with torch.no_grad():
         cache = StaticCache(config=model.config, max_cache_len=prompt + max_new_tokens)
         out = model(input_ids=input_ids, past_key_values=cache, use_cache=True,
                     cache_position=torch.arange(prompt, device=dev))
-        tok_buf = out.logits[:, -1].argmax(-1, keepdim=True).clone()
-        tokens = [tok_buf.clone()]
-        if max_new_tokens > 1 and not (eos_token_id is not None and int(tok_buf[0, 0]) == eos_token_id):
-            pos_buf = torch.tensor([prompt], device=dev)
+        ids = input_ids
+        tok_buf = torch.empty((1, 1), dtype=input_ids.dtype, device=dev)
+        pos_buf = torch.tensor([prompt - 1], device=dev)
 
-            def step():
-                o = model(input_ids=tok_buf, past_key_values=cache, use_cache=True, cache_position=pos_buf)
-                return o.logits[:, -1].argmax(-1, keepdim=True)
+        def advance(logits):
+            nonlocal ids
+            nxt = pick(ids, logits)
+            tok_buf.copy_(nxt)
+            pos_buf.add_(1)
+            ids = torch.cat([ids, nxt], dim=1)
+            return eos_token_id is not None and int(nxt[0, 0]) == eos_token_id
 
-            def advance(nxt):
-                tok_buf.copy_(nxt)
-                pos_buf.add_(1)
-                tokens.append(nxt.clone())
-                return eos_token_id is not None and int(nxt[0, 0]) == eos_token_id
+        def step():
+            o = model(input_ids=tok_buf, past_key_values=cache, use_cache=True, cache_position=pos_buf)
+            return o.logits[:, -1]
 
-            # the second token comes from one eager step (on a side stream, as graph capture wants its warm-up):
-            # every lazy allocation and per-layer check of the kernels' host side has then happened before capture
+        done = advance(out.logits[:, -1])
+        if not done and max_new_tokens > 1:
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
-                second = step()
+                logits = step()
             torch.cuda.current_stream().wait_stream(side)
-            done = advance(second)
-            if not done and max_new_tokens > 2:
-                graph = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(graph):
-                    nxt = step()
-                for _ in range(max_new_tokens - 2):
-                    graph.replay()
-                    if advance(nxt):
+            done = advance(logits)
+            remaining = max_new_tokens - 2
+            if not done and remaining > 0:
+                if use_graph:
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph):
+                        logits = step()
+                for _ in range(remaining):
+                    if use_graph:
+                        graph.replay()
+                    else:
+                        logits = step()
+                    if advance(logits):
                         break
-    return torch.cat([input_ids] + tokens, dim=1)
+    return ids
+
+
+def greedy_generate_graph(model, input_ids, max_new_tokens, eos_token_id=None):
+    """`generate_graph` with argmax decoding."""
+    return generate_graph(model, input_ids, max_new_tokens, eos_token_id=eos_token_id)
 
 
 def main(argv=None):
@@ -131,11 +172,10 @@ def main(argv=None):
         options.update(do_sample=False, temperature=None, top_p=None, top_k=None)
     start = time.time()
     if args.hip_graph:
-        if not args.greedy:
-            raise ValueError("--hip_graph decodes greedily: pass --greedy as well")
+        sampling = None if args.greedy else {k: SAMPLING[k] for k in ("repetition_penalty", "temperature", "top_k", "top_p")}
         with torch.amp.autocast(device_type="cuda"):
-            sequences = greedy_generate_graph(model, batch["input_ids"], args.max_new_tokens,
-                                              eos_token_id=getattr(tokenizer, "eos_token_id", None))
+            sequences = generate_graph(model, batch["input_ids"], args.max_new_tokens,
+                                       eos_token_id=getattr(tokenizer, "eos_token_id", None), sampling=sampling)
     else:
         with torch.no_grad():
             sequences = model.generate(inputs=batch["input_ids"], **options)["sequences"]

@@ -142,5 +142,13 @@ def test_hip_graph_decode_gives_the_eager_tokens(tmp_path, oracle, act_order):
                               eos_token_id=getattr(tokenizer, "eos_token_id", None))
     text_graph, _ = inference.main(args + ["--fuse", "--hip_graph"])
     assert text_graph == tokenizer.decode(want[0].tolist())
-    with pytest.raises(ValueError):
-        inference.main(args[:-1] + ["--hip_graph"])
+    # sampling (the reference's settings) between the replays: same draws as the same loop without capture
+    sampling = {k: inference.SAMPLING[k] for k in ("repetition_penalty", "temperature", "top_k", "top_p")}
+    runs = []
+    for use_graph in (True, False, True):
+        torch.manual_seed(1234)
+        runs.append(inference.generate_graph(model, ids, new, sampling=sampling, use_graph=use_graph).tolist())
+    assert runs[0] == runs[1] == runs[2]
+    assert runs[0] != inference.greedy_generate_graph(model, ids, new).tolist()
+    text_sampled, _ = inference.main(args[:-1] + ["--hip_graph"])
+    assert text_sampled.startswith("alpha beta gamma")
