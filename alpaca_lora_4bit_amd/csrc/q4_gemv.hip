@@ -215,33 +215,42 @@ struct SeqChunk {
         // B operands of the two extra MFMAs: per-position offsets (1024 | 64) and all ones
         const half8_t offs = make_half8(0x64006400u, 0x54005400u, 0x64006400u, 0x54005400u);
         const half8_t ones = make_half8(0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u);
+        // pass 1 (needs the activations only): A operands and the two weight-independent products
+        half8_t av[NSTEP];
+        float4_t acco_g[NG], accx_g[NG];
 #pragma unroll
         for (int gi = 0; gi < NG; ++gi) {
-            float4_t acc[4], acco, accx;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
-            acco = float4_t{0.f, 0.f, 0.f, 0.f};
-            accx = float4_t{0.f, 0.f, 0.f, 0.f};
+            acco_g[gi] = float4_t{0.f, 0.f, 0.f, 0.f};
+            accx_g[gi] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int tt = 0; tt < GS; ++tt) {
                 const int t = gi * GS + tt;
-                // A operand in the order the nibble split below produces: (e0,e4)(e1,e5)(e2,e6)(e3,e7)
-                const half8_t av = make_half8(__builtin_amdgcn_perm(xv[t].z, xv[t].x, 0x05040100u),
-                                              __builtin_amdgcn_perm(xv[t].z, xv[t].x, 0x07060302u),
-                                              __builtin_amdgcn_perm(xv[t].w, xv[t].y, 0x05040100u),
-                                              __builtin_amdgcn_perm(xv[t].w, xv[t].y, 0x07060302u));
+                av[t] = make_half8(__builtin_amdgcn_perm(xv[t].z, xv[t].x, 0x05040100u),
+                                   __builtin_amdgcn_perm(xv[t].z, xv[t].x, 0x07060302u),
+                                   __builtin_amdgcn_perm(xv[t].w, xv[t].y, 0x05040100u),
+                                   __builtin_amdgcn_perm(xv[t].w, xv[t].y, 0x07060302u));
+                acco_g[gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[t], offs, acco_g[gi], 0, 0, 0);
+                accx_g[gi] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[t], ones, accx_g[gi], 0, 0, 0);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int gi = 0; gi < NG; ++gi) {
+            float4_t acc[4];
+            const float4_t acco = acco_g[gi], accx = accx_g[gi];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int tt = 0; tt < GS; ++tt) {
+                const int t = gi * GS + tt;
                 const uint32_t w[4] = {wv[t].x, wv[t].y, wv[t].z, wv[t].w};
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    // a code in mantissa bits 0..3 of fp16 1024.0 reads 1024 + q, in bits 4..7 of fp16 64.0
-                    // it reads 64 + q: five ALU ops per word instead of one shift per nibble
                     const uint32_t hi = w[j] >> 8;
                     const half8_t bv = make_half8((w[j] & 0x000F000Fu) | 0x64006400u, (w[j] & 0x00F000F0u) | 0x54005400u,
                                                   (hi & 0x000F000Fu) | 0x64006400u, (hi & 0x00F000F0u) | 0x54005400u);
-                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, acc[j], 0, 0, 0);
+                    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[t], bv, acc[j], 0, 0, 0);
                 }
-                acco = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, offs, acco, 0, 0, 0);
-                accx = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, ones, accx, 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);      // consume the loads in the order they return
             }
             const half2_t s01 = as_half2(sv[gi].x), s23 = as_half2(sv[gi].y);
@@ -290,8 +299,10 @@ __global__ __launch_bounds__(NSTEP >= 16 ? 512 : 1024) void gemv_seq_kernel(Gemv
 
     if (k0 < a.K) {                               // wave-uniform; K % (32*NSTEP) == 0 (checked on the host)
         SeqChunk<NSTEP, GSTEPS, V1> ch;
-        ch.load_weights(a, k0, n0 + 4 * c, kk);
+        // activations first: they come from the caches and return early, so the operand shuffles and the two
+        // weight-independent products run while the packed words are still on their way from HBM
         ch.load_x(a.x + (size_t)min(c, a.M - 1) * a.K + k0 + 8 * kk);
+        ch.load_weights(a, k0, n0 + 4 * c, kk);
         // Keep the burst a burst: the scheduler must not sink loads below the arithmetic.
         __builtin_amdgcn_sched_barrier(0);
         ch.multiply(a, yacc, c);
