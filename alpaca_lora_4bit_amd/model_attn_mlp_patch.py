@@ -6,7 +6,7 @@ attention / MLP classes.  Here the concatenation is the same (fuse_quant_linears
 keep their own forward: each original projection is replaced by a slice view of the shared fused layer,
 so whatever attention / MLP implementation the installed transformers has calls `q_proj(x)`, `k_proj(x)`,
 `v_proj(x)` as before and the first of those calls runs the single fused launch for all three.
-At M=1 the fused gate+up GEMV of LLaMA-7B reaches 51 % of HBM peak against 40 % for two launches.
+At M=1 the fused gate+up GEMV of LLaMA-7B reaches about 50 % of HBM peak against 40 % for two launches.
 
 `inject_lora_layers(model, lora_path)` (model_attn_mlp_patch.py:283-335) puts a saved q/v adapter onto the fused
 qkv layers: the per-projection adapters become ONE adapter of rank r_q + r_v whose B matrix is block-structured
