@@ -438,12 +438,9 @@ void skinny_seq_kernel(SkinnyArgs a) {
     const int vz = (g * (a.N >> 3) + (c >> 1)) * 4;
     const int wstep = 16 * a.N;                    // bytes between the words of two steps (4 packed rows)
 
-    // weights of the first strip, then the activations of the chunk
     uint4_t wv[NSTEP];
-    uint2_t sv = buf_load64(rs, vs, dead + strip0 * 128);
-    uint32_t zv = buf_load32(rz, vz, dead + strip0 * 32);
-#pragma unroll
-    for (int t = 0; t < NSTEP; ++t) wv[t] = buf_load128(rw, vw, dead + strip0 * 256 + t * wstep);
+    uint2_t sv;
+    uint32_t zv;
     // Activations: a lane of the MFMA A operand wants 16 bytes of row c, so a direct load would touch 16
     // rows (16 cache lines) per quarter wavefront and the vector cache would spend its time on tag lookups.
     // Load row-contiguous instead (a quarter wavefront = 256 contiguous bytes of one row) and turn the tile
@@ -460,6 +457,13 @@ void skinny_seq_kernel(SkinnyArgs a) {
                 const int vx = (min(16 * rb + 4 * i + kk, a.M - 1) * a.K + 8 * c) * 2;
                 xv[rb][i] = buf_load128(rx, vx, dead + k0 * 2);
             }
+        // the weights of the first strip right behind the activations: those come from the caches and return
+        // first (loads return in issue order), so the turn through LDS and the offset products below run while
+        // the packed words are still on their way from HBM
+        sv = buf_load64(rs, vs, dead + strip0 * 128);
+        zv = buf_load32(rz, vz, dead + strip0 * 32);
+#pragma unroll
+        for (int t = 0; t < NSTEP; ++t) wv[t] = buf_load128(rw, vw, dead + strip0 * 256 + t * wstep);
         __builtin_amdgcn_sched_barrier(0);        // one burst of loads, nothing sunk below the arithmetic
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
