@@ -366,6 +366,14 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     slab[0].init(t, a, c0);
     slab[1].init(t, a, c0);
 
+    // bias of this lane's two output columns, requested before everything else: its latency hides under the
+    // prologue instead of sitting in the epilogue
+    float bias_v[2] = {0.f, 0.f};
+    if (FWD && a.bias) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) bias_v[j] = (float)a.bias[c0 + (wave & 1) * 64 + 32 * j + (lane & 31)];
+    }
+
     float16_t acc[TM][2];
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -497,7 +505,7 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const int col = c0 + wn * 64 + 32 * j + lc;
-                const float bv = (FWD && a.bias && blockIdx.z == 0) ? (float)a.bias[col] : 0.f;
+                const float bv = blockIdx.z == 0 ? bias_v[j] : 0.f;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int m = m0 + wm * WROWS + 32 * i + 8 * (r >> 2) + lrow + (r & 3);
@@ -513,7 +521,7 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-            const float bv = (FWD && a.bias) ? (float)a.bias[c0 + wn * 64 + 32 * j + lc] : 0.f;
+            const float bv = bias_v[j];
 #pragma unroll
             for (int r = 0; r < 16; ++r)
                 stage[(8 * (r >> 2) + lrow + (r & 3)) * LDS_STRIDE + 32 * j + lc] = (half_t)(acc[i][j][r] + bv);

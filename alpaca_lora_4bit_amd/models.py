@@ -178,7 +178,7 @@ class Linear4bitLt(Autograd4bitQuantLinear, LoraLayer):
             name = self._fusable_adapter(x)
             if name is not None:
                 bias = None
-                if not self.disable_bias:
+                if not self.disable_bias and not autograd_4bit._is_all_zero(self.bias):
                     bias = self.bias if self.bias.dtype == torch.float16 else self.bias.half()
                 return autograd_4bit.AutogradMatmul4bitLora.apply(
                     x, self.qweight, self.scales, self.qzeros, self.g_idx, bias,
