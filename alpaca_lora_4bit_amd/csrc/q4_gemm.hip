@@ -46,6 +46,7 @@ struct GemmArgs {
     const half_t* scales;     // [G, N]
     const int32_t* g_idx;     // [K] or null
     int groupsize;
+    uint32_t gs_inv31;        // ceil(2^31 / (groupsize / 64)): reduction offset -> group without a division
     const half_t* bias;       // fwd only, [N] or null
     const half_t* la;         // fwd: xa [M,R]     bwd: dyb [M,R]   (or null)
     const void* lb;           // adapter matrix (fp16 or fp32), element (r, c) at lb[r*lb_sr + c*lb_sc]; fwd: c = n, bwd: c = k
@@ -99,6 +100,12 @@ __device__ __forceinline__ int red_of(int stage, StepRange sr, int phase) {
     int v = min(stage, sr.cnt - 1) + phase;
     if (v >= sr.cnt) v -= sr.cnt;
     return (sr.begin + v) * BK;
+}
+
+// Group of reduction row k (a multiple of 64; sequential groups of a multiple of 64 rows):
+// floor((k/64) / (groupsize/64)) as a multiply-high, exact while k * groupsize < 2^40.
+__device__ __forceinline__ int group_of(const GemmArgs& a, int k) {
+    return (int)__umulhi((uint32_t)k >> 5, a.gs_inv31);
 }
 
 __device__ __forceinline__ float adapter_at(const GemmArgs& a, size_t idx) {
@@ -159,9 +166,9 @@ struct FwdSlab {
         if constexpr (I < NW) {
             w[I] = buf_load32(r.w, voff_w + I * wstride, (kred0 >> 3) * a.N * 4);
         } else if constexpr (I == NW) {
-            s_raw = buf_load16(r.s, voff_s, (kred0 / a.groupsize) * a.N * 2);
+            s_raw = buf_load16(r.s, voff_s, group_of(a, kred0) * a.N * 2);
         } else {
-            z_raw = buf_load32(r.z, voff_z, (kred0 / a.groupsize) * (a.N >> 3) * 4);
+            z_raw = buf_load32(r.z, voff_z, group_of(a, kred0) * (a.N >> 3) * 4);
         }
     }
     __device__ __forceinline__ void load(const GemmArgs& a, const SlabRsrc& r, int, int kred0) {
@@ -706,6 +713,7 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     a.scales = reinterpret_cast<const half_t*>(scales);
     a.g_idx = g_idx;
     a.groupsize = groupsize;
+    a.gs_inv31 = groupsize >= 64 ? (uint32_t)(((1ull << 31) + (uint64_t)(groupsize / 64) - 1) / (uint64_t)(groupsize / 64)) : 0u;
     a.bias = reinterpret_cast<const half_t*>(bias);
     a.la = reinterpret_cast<const half_t*>(la);
     a.lb = lb;
