@@ -189,10 +189,7 @@ def bench_lora_step(reps, seed=5):
         m.lora_B["default"].weight.grad = None
 
     # eager: Python launches every kernel
-    for _ in range(3):
-        step()
-        clear()
-    torch.cuda.synchronize()
+    _spin_up(lambda: (step(), clear()))
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     e0.record()
     for _ in range(reps):
@@ -214,8 +211,7 @@ def bench_lora_step(reps, seed=5):
     with torch.cuda.graph(g, stream=s):
         step()
     with torch.cuda.stream(s):
-        g.replay()
-        s.synchronize()
+        _spin_up(g.replay)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record(s)
         for _ in range(reps):
@@ -361,6 +357,18 @@ def bench_llama7b_lora_train_step(reps=4, seed=11, n_layers=32, batch=4, seq=256
     return out
 
 
+def _spin_up(fn, seconds=0.05):
+    """Runs fn() back to back for about `seconds` of GPU time: after an idle gap (allocation, host work) the
+    clocks need tens of milliseconds of load to come up, and a short timing loop would read 5-15 % slow."""
+    import torch
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            fn()
+        torch.cuda.synchronize()
+
+
 def bench_gemm_only(M, K, N, act_order, reps, seed=7):
     import torch
     from alpaca_lora_4bit_amd import quant_hip
@@ -371,9 +379,7 @@ def bench_gemm_only(M, K, N, act_order, reps, seed=7):
     res = {}
     for name, fn in (("fwd", lambda: quant_hip.gemm_fwd(x, lay["qweight"], lay["qzeros"], lay["scales"], lay["g_idx"], 128)),
                      ("bwd_dx", lambda: quant_hip.gemm_bwd_dx(dy, lay["qweight"], lay["qzeros"], lay["scales"], lay["g_idx"], 128))):
-        for _ in range(3):
-            fn()
-        torch.cuda.synchronize()
+        _spin_up(fn)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(reps):
