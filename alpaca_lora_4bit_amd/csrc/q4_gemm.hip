@@ -410,7 +410,7 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     auto step = [&](int s, auto cur_tag) {
         constexpr int CUR = decltype(cur_tag)::value;
         constexpr int NM = TM * 2 * KS;                        // MFMAs per step
-        constexpr int BAR = NM - 4;                            // MFMA index after which the barrier sits
+        constexpr int BAR = NM - 3;                            // MFMA index after which the barrier sits (NM-2 .. NM-5 measured: within 3 %)
         // Side work of a step: NL global loads (stage s+2 -> register set CUR) and NC consumer items
         // (stage s+1: register set CUR^1 -> LDS[CUR^1]; NSL dequantization slices with the NA activation
         // stores spread evenly among them).  One load per MFMA slot from slot 0 on (never a burst: eight
