@@ -223,3 +223,20 @@ def test_checkpointed_blocks_give_the_same_gradients():
     with torch.no_grad():
         model(input_ids=ids, use_cache=False)
     assert calls["n"] == 1                                # no checkpointing outside training mode
+
+
+def test_token_picker_of_the_graph_decode():
+    """inference._token_picker: argmax without sampling settings; with the reference's settings (inference.py:33-44)
+    the draw comes from the top-k set after repetition penalty and temperature, through transformers' processors."""
+    import torch
+    from alpaca_lora_4bit_amd import inference
+    logits = torch.tensor([[0.1, 2.0, 5.0, 4.9, -1.0, 3.0]])
+    ids = torch.tensor([[2, 2]])
+    assert inference._token_picker(None)(ids, logits).tolist() == [[2]]
+    torch.manual_seed(0)
+    pick = inference._token_picker({"repetition_penalty": 1.1, "temperature": 0.9, "top_k": 2, "top_p": 0.95})
+    draws = {int(pick(ids, logits.clone())) for _ in range(200)}
+    assert draws <= {2, 3} and draws == {2, 3}            # top-2 after the penalty on token 2: {3, 2}
+    # a huge penalty on the already generated token 2 leaves token 3 as the only survivor of top-p
+    pick = inference._token_picker({"repetition_penalty": 50.0, "temperature": 0.1, "top_k": 2, "top_p": 0.5})
+    assert {int(pick(ids, logits.clone())) for _ in range(50)} == {3}
