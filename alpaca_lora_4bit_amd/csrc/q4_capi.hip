@@ -19,6 +19,9 @@ int q4_launch_lora_grad(const void*, const void*, float*, int, int, float, int, 
 int q4_launch_lora_grad_pair(const void*, const void*, float*, int, int, int, const void*, const void*, float*, int, int, int,
                              float, int, int, void*, hipStream_t);
 size_t q4_lora_grad_workspace(int, int, int);
+size_t q4_noalloc_scratch_bytes(void);
+void* q4_noalloc_scratch_ptr(int*);
+int q4_launch_zero_words(void*, size_t, hipStream_t);
 }
 
 namespace {
@@ -38,7 +41,7 @@ int check_layer(const void* qweight, const void* qzeros, const void* scales, con
 }
 }  // namespace
 
-extern "C" int q4_abi_version(void) { return 7; }
+extern "C" int q4_abi_version(void) { return 8; }
 
 extern "C" const char* q4_error_string(int code) {
     switch (code) {
@@ -48,6 +51,8 @@ extern "C" const char* q4_error_string(int code) {
         case Q4_ERR_WORKSPACE: return "workspace missing or too small";
         case Q4_ERR_LAUNCH: return "kernel launch failed";
         case Q4_ERR_MISALIGNED: return "pointer not 16-byte aligned";
+        case Q4_ERR_TOO_LARGE: return "problem larger than the library's built-in scratch (see q4_gemv_noalloc_max_outputs)";
+        case Q4_ERR_RUNTIME: return "a HIP runtime call failed (see hipGetLastError)";
         default: return "unknown error";
     }
 }
@@ -94,15 +99,22 @@ extern "C" int q4_permute_rows(const int32_t* qweight, const int32_t* perm, int3
     return q4_launch_permute_rows(qweight, perm, out, K, N, (hipStream_t)stream);
 }
 
-static int gemv_common(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
-                       const int32_t* g_idx, const int32_t* perm, int groupsize, void* y, int accumulate,
-                       int M, int max_rows, int K, int N, int G, void* workspace, size_t workspace_bytes, void* stream) {
+static int gemv_check(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                      const int32_t* g_idx, int groupsize, const void* y, int M, int max_rows, int K, int N, int G) {
     int rc = check_layer(qweight, qzeros, scales, g_idx, groupsize, K, N, G);
     if (rc != Q4_OK) return rc;
     if (!x || !y) return Q4_ERR_NULL_POINTER;
     if (M < 1 || M > max_rows || K > 32 * 255 * 8 * 16) return Q4_ERR_BAD_SHAPE;
     if ((long long)(K / 8) * N * 4 >= 0x70000000ll) return Q4_ERR_BAD_SHAPE;      /* 32-bit buffer offsets */
     if (misaligned(x) || misaligned(y)) return Q4_ERR_MISALIGNED;
+    return Q4_OK;
+}
+
+static int gemv_common(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                       const int32_t* g_idx, const int32_t* perm, int groupsize, void* y, int accumulate,
+                       int M, int max_rows, int K, int N, int G, void* workspace, size_t workspace_bytes, void* stream) {
+    int rc = gemv_check(x, qweight, qzeros, scales, g_idx, groupsize, y, M, max_rows, K, N, G);
+    if (rc != Q4_OK) return rc;
     if (!workspace || workspace_bytes < q4_gemv_workspace_bytes(M, K, N)) return Q4_ERR_WORKSPACE;
     if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
     return q4_launch_gemv(x, qweight, qzeros, scales, g_idx, perm, groupsize, y, accumulate, M, K, N, G, workspace,
@@ -114,6 +126,26 @@ extern "C" int q4_gemv_f16(const void* x, const int32_t* qweight, const int32_t*
                            int M, int K, int N, int G, void* workspace, size_t workspace_bytes, void* stream) {
     return gemv_common(x, qweight, qzeros, scales, g_idx, nullptr, groupsize, y, accumulate, M, 16, K, N, G, workspace,
                        workspace_bytes, stream);
+}
+
+extern "C" size_t q4_gemv_noalloc_max_outputs(void) { return q4_noalloc_scratch_bytes() / 8; }
+
+extern "C" int q4_gemv_noalloc_f16(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                                   const int32_t* g_idx, int groupsize, void* y, int accumulate,
+                                   int M, int K, int N, int G, void* stream) {
+    // every check of the allocating entry point first, so that a rejected call enqueues nothing
+    int rc = gemv_check(x, qweight, qzeros, scales, g_idx, groupsize, y, M, 16, K, N, G);
+    if (rc != Q4_OK) return rc;
+    const size_t words = (size_t)M * (size_t)N;
+    if (words > q4_gemv_noalloc_max_outputs()) return Q4_ERR_TOO_LARGE;
+    int herr = 0;
+    void* scratch = q4_noalloc_scratch_ptr(&herr);
+    if (!scratch) return Q4_ERR_RUNTIME;
+    // the array keeps whatever the previous call on this device left (zeros, unless that call was cut short)
+    rc = q4_launch_zero_words(scratch, words, (hipStream_t)stream);
+    if (rc != Q4_OK) return rc;
+    return gemv_common(x, qweight, qzeros, scales, g_idx, nullptr, groupsize, y, accumulate, M, 16, K, N, G, scratch,
+                       words * 8, stream);
 }
 
 extern "C" int q4_gemv_sorted_f16(const void* x, const int32_t* qweight_sorted, const int32_t* qzeros, const void* scales,

@@ -866,3 +866,46 @@ extern "C" int q4_launch_skinny(const void* x, const int32_t* qweight, const int
     if (S > 1) return q4_launch_splitk_reduce(a.part, y, (long)M * N, S, stream);
     return 0;
 }
+
+// ------------------------------------------------------------------ split-K accumulators owned by the library
+// For callers that cannot allocate (q4_gemv_noalloc_f16): the [M, N] 64-bit accumulators live in a file-scope
+// device array instead of a caller workspace.  Every device that loads this library holds its own copy at its
+// own address; host code must never hand the array's NAME to a kernel (on the host it is only a stand-in
+// symbol), so the device address is looked up once per device and kept.
+namespace q4 {
+constexpr size_t kNoAllocWords = (size_t)16 * 32768;          // M * N <= 524 288 accumulators = 4 MiB per device
+static __device__ __align__(256) unsigned long long noalloc_scratch[kNoAllocWords];
+
+__global__ __launch_bounds__(256) void zero_words_kernel(unsigned long long* p, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0ull;
+}
+}  // namespace q4
+
+extern "C" size_t q4_noalloc_scratch_bytes(void) { return q4::kNoAllocWords * sizeof(unsigned long long); }
+
+// Device address of the array on the CURRENT device (looked up on the first call per device), or null with
+// *err set to the HIP error.
+extern "C" void* q4_noalloc_scratch_ptr(int* err) {
+    constexpr int kMaxDevices = 64;
+    static void* volatile ptrs[kMaxDevices];
+    *err = 0;
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) { *err = e != hipSuccess ? (int)e : -1; return nullptr; }
+    void* p = ptrs[dev];
+    if (p) return p;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(q4::noalloc_scratch));
+    if (e != hipSuccess || !p) { *err = e != hipSuccess ? (int)e : -1; return nullptr; }
+    ptrs[dev] = p;                                              // racing first calls store the same address
+    return p;
+}
+
+// Zeroes the first `words` accumulators with a small kernel (a fill kernel, not a memset node, so that the call
+// may be recorded into a HIP graph).
+extern "C" int q4_launch_zero_words(void* p, size_t words, hipStream_t stream) {
+    if (words == 0) return 0;
+    hipLaunchKernelGGL(q4::zero_words_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream,
+                       reinterpret_cast<unsigned long long*>(p), (int)words);
+    return hipGetLastError() == hipSuccess ? 0 : -4;
+}

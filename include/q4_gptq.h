@@ -34,6 +34,8 @@ extern "C" {
 #define Q4_ERR_WORKSPACE (-3)      /* workspace missing or smaller than *_workspace_bytes() */
 #define Q4_ERR_LAUNCH (-4)         /* hipLaunch reported an error (see hipGetLastError) */
 #define Q4_ERR_MISALIGNED (-5)     /* a pointer is not 16-byte aligned */
+#define Q4_ERR_TOO_LARGE (-6)      /* larger than the library's built-in scratch (allocation-free entry point) */
+#define Q4_ERR_RUNTIME (-7)        /* a HIP runtime call other than a launch failed */
 
 /* Library ABI version (bumped when a signature changes). */
 int q4_abi_version(void);
@@ -83,6 +85,19 @@ int q4_gemv_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, co
                 const int32_t *g_idx, int groupsize, void *y, int accumulate,
                 int M, int K, int N, int G,
                 void *workspace, size_t workspace_bytes, void *stream);
+
+/* q4_gemv_f16 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same product, same arguments
+ * minus the workspace: the split-K accumulators live in a device array inside the library (4 MiB per device that
+ * runs the library, held until the process ends), so the call needs M * N <= q4_gemv_noalloc_max_outputs()
+ * = 524 288 (e.g. 16 rows x 32 768 columns) and returns Q4_ERR_TOO_LARGE beyond that.  It calls no hipMalloc /
+ * hipFree and no allocating library routine; it enqueues a small fill kernel that zeroes the accumulators and
+ * then the same kernels as q4_gemv_f16, and gives bit-identical results.  All calls on one device share the
+ * one array: calls that overlap on a device (two streams, two threads) race -- order them on one stream. */
+size_t q4_gemv_noalloc_max_outputs(void);
+int q4_gemv_noalloc_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+                        const int32_t *g_idx, int groupsize, void *y, int accumulate,
+                        int M, int K, int N, int G, void *stream);
 
 /* The same product for an act-order layer whose packed rows were sorted by group with q4_permute_rows.
  * Limits: 1 <= M <= 4, K >= 1024 and M * (2*K + 4096) <= 65536 bytes, i.e. the activation rows fit in LDS

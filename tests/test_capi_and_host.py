@@ -36,7 +36,7 @@ def test_error_codes_and_validation_need_no_gpu():
     from alpaca_lora_4bit_amd import _lib
     L = _lib.lib()
     assert L.q4_error_string(0) == b"ok"
-    for code in (-1, -2, -3, -4, -5):
+    for code in (-1, -2, -3, -4, -5, -6, -7):
         assert L.q4_error_string(code) not in (b"ok", b"unknown error")
     assert L.q4_error_string(-99) == b"unknown error"
     # null pointers
@@ -89,6 +89,12 @@ def test_error_codes_and_validation_need_no_gpu():
     assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, None, 1, 8, 4096, 1.0, 2048, 8, fake, 1 << 24, None) == -1
     assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, fake, 1, 8, 4100, 1.0, 2048, 8, fake, 1 << 24, None) == -2
     assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, fake, 1, 8, 4096, 1.0, 2048, 8, fake, 1 << 22, None) == -3  # needs 2 x 4 MiB
+    # allocation-free GEMV: validated like q4_gemv_f16, plus the size of the built-in accumulator array
+    assert L.q4_gemv_noalloc_max_outputs() == 16 * 32768
+    assert L.q4_gemv_noalloc_f16(fake, fake, fake, fake, None, 128, fake, 0, 16, 256, 32832, 2, None) == -6
+    assert L.q4_gemv_noalloc_f16(fake, fake, fake, fake, None, 128, fake, 0, 17, 256, 128, 2, None) == -2
+    assert L.q4_gemv_noalloc_f16(None, fake, fake, fake, None, 128, fake, 0, 1, 256, 128, 2, None) == -1
+    assert L.q4_gemv_noalloc_f16(fake, fake, fake, fake, None, 128, odd, 0, 1, 256, 128, 2, None) == -5
     assert L.q4_gemv_workspace_bytes(16, 4096, 11008) == 16 * 11008 * 8
     assert L.q4_gemv_workspace_bytes(0, 4096, 11008) == 0
 
