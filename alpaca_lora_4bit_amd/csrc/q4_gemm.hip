@@ -697,7 +697,7 @@ extern "C" {
 int q4_skinny_applicable(int M, int K, int N, int groupsize, int has_gidx);
 size_t q4_skinny_workspace(int M, int K, int N);
 int q4_launch_skinny(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales, int groupsize,
-                     const void* bias, void* y, int M, int K, int N, void* workspace, hipStream_t stream);
+                     const void* bias, void* y, int M, int K, int N, int G, void* workspace, hipStream_t stream);
 }
 
 extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros,
@@ -728,7 +728,7 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     // 17..64 rows, forward, no adapter: the weight-streaming kernel (one pass over the packed weights)
     if (fwd && a.R == 0 && q4_skinny_applicable(M, K, N, groupsize, gidx) && workspace &&
         workspace_bytes >= q4_skinny_workspace(M, K, N))
-        return q4_launch_skinny(act, qweight, qzeros, scales, groupsize, bias, out, M, K, N, workspace, stream);
+        return q4_launch_skinny(act, qweight, qzeros, scales, groupsize, bias, out, M, K, N, G, workspace, stream);
     // tile configuration: 256-row tiles once they still give every CU a workgroup; split-K for few tiles
     const GemmPlan p = plan_gemm(M, fwd ? K : N, nout, workspace ? workspace_bytes : 0);
     a.part = reinterpret_cast<float*>(workspace);

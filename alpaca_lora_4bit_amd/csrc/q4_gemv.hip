@@ -406,7 +406,7 @@ struct SkinnyArgs {
     int groupsize;
     half_t* y;                // written directly when gridDim.y == 1
     float* part;              // [gridDim.y][M][N]
-    int M, K, N;
+    int M, K, N, G;           // G: rows of scales / qzeros (ceil(K / groupsize): the last group may be partial)
     int strips_per_wg;
 };
 
@@ -424,7 +424,7 @@ void skinny_seq_kernel(SkinnyArgs a) {
     const int nl = min(a.strips_per_wg, (a.N >> 6) - strip0);
     const int k0 = (blockIdx.y * NW + wave) * (32 * NSTEP);
     const int dead = k0 < a.K ? 0 : kFar;          // wave-uniform
-    const int G = a.K / a.groupsize, g = dead ? 0 : k0 / a.groupsize;
+    const int G = a.G, g = dead ? 0 : k0 / a.groupsize;
     const int S = gridDim.y;
 
     const rsrc_t rw = make_rsrc(a.qweight, (unsigned)((size_t)(a.K >> 3) * a.N * 4));
@@ -836,7 +836,7 @@ extern "C" size_t q4_skinny_workspace(int M, int K, int N) {
 }
 
 extern "C" int q4_launch_skinny(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
-                                int groupsize, const void* bias, void* y, int M, int K, int N,
+                                int groupsize, const void* bias, void* y, int M, int K, int N, int G,
                                 void* workspace, hipStream_t stream) {
     using namespace q4;
     SkinnyArgs a;
@@ -848,7 +848,7 @@ extern "C" int q4_launch_skinny(const void* x, const int32_t* qweight, const int
     a.groupsize = groupsize;
     a.y = reinterpret_cast<half_t*>(y);
     a.part = reinterpret_cast<float*>(workspace);
-    a.M = M; a.K = K; a.N = N;
+    a.M = M; a.K = K; a.N = N; a.G = G;
     const int S = skinny_splits(K);
     const int strips = N / kColsPerWave;
     // neighbouring strips per workgroup: enough for the whole grid to be resident at once (two workgroups
