@@ -6,7 +6,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libq4gptq.so")
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _lib = None
 
@@ -33,6 +33,16 @@ SIGNATURES = {
     "q4_lora_grad_f32": (_i, [_vp, _vp, _vp, _i, _i, _f, _i, _i, _i, _vp, _sz, _vp]),
     "q4_lora_grad_pair_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _vp, _sz, _vp]),
 }
+
+
+class GemvLayer(ctypes.Structure):
+    """q4_gemv_layer_t of include/q4_gptq.h."""
+    _fields_ = [("x", _vp), ("qweight", _vp), ("qzeros", _vp), ("scales", _vp), ("y", _vp), ("N", _i)]
+
+
+MAX_GEMV_GROUP = 4
+SIGNATURES["q4_gemv_grouped_workspace_bytes"] = (_sz, [_i, _i])
+SIGNATURES["q4_gemv_grouped_f16"] = (_i, [ctypes.POINTER(GemvLayer), _i, _i, _i, _i, _i, _vp, _sz, _vp])
 
 
 class Q4Error(RuntimeError):

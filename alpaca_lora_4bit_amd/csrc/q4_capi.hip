@@ -19,6 +19,8 @@ int q4_launch_lora_grad(const void*, const void*, float*, int, int, float, int, 
 int q4_launch_lora_grad_pair(const void*, const void*, float*, int, int, int, const void*, const void*, float*, int, int, int,
                              float, int, int, void*, hipStream_t);
 size_t q4_lora_grad_workspace(int, int, int);
+int q4_launch_gemv_group(int, const void* const*, const int32_t* const*, const int32_t* const*, const void* const*,
+                         void* const*, const int*, int, int, int, int, int, void*, hipStream_t);
 size_t q4_noalloc_scratch_bytes(void);
 void* q4_noalloc_scratch_ptr(int*);
 int q4_launch_zero_words(void*, size_t, hipStream_t);
@@ -41,7 +43,7 @@ int check_layer(const void* qweight, const void* qzeros, const void* scales, con
 }
 }  // namespace
 
-extern "C" int q4_abi_version(void) { return 8; }
+extern "C" int q4_abi_version(void) { return 9; }
 
 extern "C" const char* q4_error_string(int code) {
     switch (code) {
@@ -126,6 +128,34 @@ extern "C" int q4_gemv_f16(const void* x, const int32_t* qweight, const int32_t*
                            int M, int K, int N, int G, void* workspace, size_t workspace_bytes, void* stream) {
     return gemv_common(x, qweight, qzeros, scales, g_idx, nullptr, groupsize, y, accumulate, M, 16, K, N, G, workspace,
                        workspace_bytes, stream);
+}
+
+extern "C" size_t q4_gemv_grouped_workspace_bytes(int M, int total_N) {
+    if (M < 1 || total_N < 1) return 0;
+    return (size_t)M * (size_t)total_N * 8;
+}
+
+extern "C" int q4_gemv_grouped_f16(const q4_gemv_layer_t* layers, int n_layers, int groupsize, int accumulate,
+                                   int M, int K, void* workspace, size_t workspace_bytes, void* stream) {
+    if (!layers) return Q4_ERR_NULL_POINTER;
+    if (n_layers < 1 || n_layers > Q4_GEMV_MAX_GROUP) return Q4_ERR_BAD_SHAPE;
+    if (groupsize < 32 || (groupsize % 32) != 0 || K < 64) return Q4_ERR_BAD_SHAPE;
+    const int G = (K + groupsize - 1) / groupsize;
+    const void* x[Q4_GEMV_MAX_GROUP]; const int32_t* qw[Q4_GEMV_MAX_GROUP]; const int32_t* qz[Q4_GEMV_MAX_GROUP];
+    const void* sc[Q4_GEMV_MAX_GROUP]; void* y[Q4_GEMV_MAX_GROUP]; int N[Q4_GEMV_MAX_GROUP];
+    long long total_n = 0;
+    for (int i = 0; i < n_layers; ++i) {
+        const q4_gemv_layer_t& l = layers[i];
+        int rc = gemv_check(l.x, l.qweight, l.qzeros, l.scales, nullptr, groupsize, l.y, M, 16, K, l.N, G);
+        if (rc != Q4_OK) return rc;
+        x[i] = l.x; qw[i] = l.qweight; qz[i] = l.qzeros; sc[i] = l.scales; y[i] = l.y; N[i] = l.N;
+        total_n += l.N;
+    }
+    if (total_n > 0x7fffffff / 64) return Q4_ERR_BAD_SHAPE;
+    if (!workspace || workspace_bytes < q4_gemv_grouped_workspace_bytes(M, (int)total_n)) return Q4_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
+    return q4_launch_gemv_group(n_layers, x, qw, qz, sc, y, N, groupsize, accumulate, M, K, G, workspace,
+                                (hipStream_t)stream);
 }
 
 extern "C" size_t q4_gemv_noalloc_max_outputs(void) { return q4_noalloc_scratch_bytes() / 8; }

@@ -284,13 +284,12 @@ struct SeqChunk {
     }
 };
 
-template <int NSTEP, int GSTEPS, bool V1 = false>
-__global__ __launch_bounds__(NSTEP >= 16 ? 512 : 1024) void gemv_seq_kernel(GemvArgs a) {
+template <int NSTEP, int GSTEPS, bool V1>
+__device__ __forceinline__ void gemv_seq_body(const GemvArgs& a, int n0) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nwaves = blockDim.x >> 6;
     const int kk = lane >> 4, c = lane & 15;
-    const int n0 = blockIdx.x * kColsPerWave;
     const int k0 = (blockIdx.y * nwaves + wave) * (32 * NSTEP);
 
     float4_t yacc[4];
@@ -308,6 +307,29 @@ __global__ __launch_bounds__(NSTEP >= 16 ? 512 : 1024) void gemv_seq_kernel(Gemv
         ch.multiply(a, yacc, c);
     }
     gemv_finish(a, yacc, n0, wave, nwaves, kk, c);
+}
+
+template <int NSTEP, int GSTEPS, bool V1 = false>
+__global__ __launch_bounds__(NSTEP >= 16 ? 512 : 1024) void gemv_seq_kernel(GemvArgs a) {
+    gemv_seq_body<NSTEP, GSTEPS, V1>(a, blockIdx.x * kColsPerWave);
+}
+
+// Up to kMaxGroup layers with the same K, group size and row count M in ONE grid (q|k|v or gate|up of a decoder
+// block, read in place from their own tensors): blockIdx.x walks the strips of layer 0, then of layer 1, ...
+// A launch costs about 3 us of fixed time (dispatch, ramp, the reduction round trip) on top of the streaming
+// time of its bytes, so two or three layers in one launch run close to the time of the largest alone.
+constexpr int kMaxGroup = 4;
+struct GemvGroupArgs {
+    GemvArgs layer[kMaxGroup];
+    int strip_end[kMaxGroup];                     // running total of 64-column strips; unused entries = INT_MAX
+};
+
+template <int NSTEP, int GSTEPS>
+__global__ __launch_bounds__(1024) void gemv_seq_group_kernel(GemvGroupArgs g) {
+    const int bx = blockIdx.x;
+    const int li = (bx >= g.strip_end[0]) + (bx >= g.strip_end[1]) + (bx >= g.strip_end[2]);      // uniform
+    const int first = li == 0 ? 0 : g.strip_end[li - 1];
+    gemv_seq_body<NSTEP, GSTEPS, false>(g.layer[li], (bx - first) * kColsPerWave);
 }
 
 // The same for an act-order layer whose packed rows were sorted by group (q4_permute_rows): row p of the
@@ -788,6 +810,61 @@ extern "C" int q4_launch_gemv(const void* x, const int32_t* qweight, const int32
     return hipGetLastError() == hipSuccess ? 0 : -4;
 }
 
+
+template <int NSTEP>
+static void launch_seq_group(const q4::GemvPlan& p, dim3 grid, dim3 block, size_t lds, hipStream_t stream,
+                             const q4::GemvGroupArgs& g) {
+    using namespace q4;
+    switch (p.gsteps) {
+        case 0: hipLaunchKernelGGL((gemv_seq_group_kernel<NSTEP, 0>), grid, block, lds, stream, g); break;
+        case 1: if constexpr (NSTEP > 1) hipLaunchKernelGGL((gemv_seq_group_kernel<NSTEP, 1>), grid, block, lds, stream, g); break;
+        case 2: if constexpr (NSTEP > 2) hipLaunchKernelGGL((gemv_seq_group_kernel<NSTEP, 2>), grid, block, lds, stream, g); break;
+    }
+}
+
+// n layers (1..4) sharing M, K and the group size (sequential groups); layer i: x[i], packed tensors, y[i], N[i];
+// its accumulators start at workspace + 8*M*(N[0] + .. + N[i-1]).
+extern "C" int q4_launch_gemv_group(int n, const void* const* x, const int32_t* const* qweight,
+                                    const int32_t* const* qzeros, const void* const* scales, void* const* y,
+                                    const int* N, int groupsize, int accumulate, int M, int K, int G,
+                                    void* workspace, hipStream_t stream) {
+    using namespace q4;
+    GemvGroupArgs g;
+    int strips = 0;
+    size_t ws_off = 0;
+    for (int i = 0; i < kMaxGroup; ++i) {
+        const int j = i < n ? i : n - 1;              // unused slots repeat the last layer (never selected)
+        GemvArgs& a = g.layer[i];
+        a.x = reinterpret_cast<const half_t*>(x[j]);
+        a.qweight = reinterpret_cast<const uint32_t*>(qweight[j]);
+        a.qzeros = reinterpret_cast<const uint32_t*>(qzeros[j]);
+        a.scales = reinterpret_cast<const half_t*>(scales[j]);
+        a.g_idx = nullptr;
+        a.groupsize = groupsize;
+        a.y = reinterpret_cast<half_t*>(y[j]);
+        a.accumulate = accumulate;
+        a.M = M; a.K = K; a.N = N[j]; a.G = G;
+        a.acc64 = reinterpret_cast<unsigned long long*>(workspace) + ws_off;
+        a.perm = nullptr;
+        a.v1_zeros = nullptr;
+        if (i < n) {
+            strips += N[i] / kColsPerWave;
+            ws_off += (size_t)M * N[i];
+            g.strip_end[i] = strips;
+        } else {
+            g.strip_end[i] = 0x7fffffff;
+        }
+    }
+    const GemvPlan p = plan_gemv(K, N[0], groupsize, true, 4);
+    const dim3 grid(strips, p.splits), block(64 * p.waves);
+    const size_t lds = (size_t)p.waves * M * 64 * sizeof(float);
+    switch (p.nstep) {
+        case 4: launch_seq_group<4>(p, grid, block, lds, stream, g); break;
+        case 2: launch_seq_group<2>(p, grid, block, lds, stream, g); break;
+        default: launch_seq_group<1>(p, grid, block, lds, stream, g); break;
+    }
+    return hipGetLastError() == hipSuccess ? 0 : -4;
+}
 
 // v1 layout: scales and zeros are fp16 [N]; one group spanning K.
 extern "C" int q4_launch_gemv_v1(const void* x, const int32_t* qweight, const void* scales, const void* zeros, void* y,

@@ -389,6 +389,60 @@ def gemv(x, qweight, qzeros, scales, g_idx=None, groupsize=None, out=None, accum
     return out
 
 
+def gemv_grouped(xs, layers, groupsize, outs=None, accumulate=False):
+    """[x_i @ W_i] for up to 4 layers that share the number of rows (<= 16), K and the group size, in ONE launch
+    over the layers' own tensors (no concatenated copy): q|k|v or gate|up of a decoder block at decode time.
+    `xs` is one activation tensor shared by all layers or a list with one per layer; `layers` a list of
+    (qweight, qzeros, scales) or (qweight, qzeros, scales, g_idx) with sequential groups; returns the list of
+    outputs ([M, N_i] fp16 each).  The reference concatenates the packed tensors instead
+    (model_attn_mlp_patch.py:88-100, 180-190)."""
+    n = len(layers)
+    _require(1 <= n <= _lib.MAX_GEMV_GROUP, f"gemv_grouped takes 1..{_lib.MAX_GEMV_GROUP} layers")
+    if isinstance(xs, torch.Tensor):
+        xs = [xs] * n
+    _require(len(xs) == n, "one activation tensor per layer (or a single shared one)")
+    dev = K = M = None
+    desc = (_lib.GemvLayer * n)()
+    keep, shapes = [], []
+    flat = {}
+    for i, (x, lay) in enumerate(zip(xs, layers)):
+        qweight, qzeros, scales = lay[0], lay[1], lay[2]
+        g_idx = lay[3] if len(lay) > 3 else None
+        d, k, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
+        _require(g_idx is None or classify_g_idx(g_idx, groupsize, G) == "seq",
+                 "gemv_grouped needs sequential groups (no act-order)")
+        if dev is None:
+            dev, K = d, k
+        _require(d == dev and k == K, "grouped layers must share the device and K")
+        x2 = flat.get(id(x))
+        if x2 is None:
+            x2 = flat[id(x)] = _flat_half(x, K, dev, "x")
+        if M is None:
+            M = x2.shape[0]
+        _require(x2.shape[0] == M, "grouped layers must share the number of rows")
+        keep.append(x2)
+        shapes.append(N)
+        desc[i].x, desc[i].qweight, desc[i].qzeros, desc[i].scales, desc[i].N = (
+            x2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), N)
+    _require(groupsize % 32 == 0, "groupsize must be a multiple of 32")
+    _require(1 <= M <= MAX_GEMV_ROWS, f"gemv handles 1..{MAX_GEMV_ROWS} rows, got {M}")
+    if outs is None:
+        _require(not accumulate, "accumulate needs output tensors")
+        outs = [torch.empty((M, N), dtype=torch.float16, device=dev) for N in shapes]
+    _require(len(outs) == n, "one output per layer")
+    for i, (o, N) in enumerate(zip(outs, shapes)):
+        _require(o.dtype == torch.float16 and o.numel() == M * N and o.shape[-1] == N and o.is_contiguous()
+                 and o.device == dev, "outputs must be contiguous float16 [..., N_i] tensors with M rows on the same device")
+        desc[i].y = o.data_ptr()
+    L = _lib.lib()
+    with _device_ctx(dev):
+        ws = _workspace(dev, L.q4_gemv_grouped_workspace_bytes(M, sum(shapes)))
+        rc = L.q4_gemv_grouped_f16(desc, n, int(groupsize), int(bool(accumulate)), M, K, ws.data_ptr(), ws.numel(),
+                                   _stream(dev))
+    _lib.check(rc, "q4_gemv_grouped_f16")
+    return list(outs)
+
+
 def _adapter_dtype_flag(w, what):
     _require(w.dtype in (torch.float16, torch.float32), f"{what} must be float16 or float32")
     return int(w.dtype == torch.float32)

@@ -28,6 +28,7 @@ MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
 # HBM bytes per launch of the headline GEMV kernel, measured in two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE),
 # each scaled by what the same counter reads for a 256 MiB copy (--calibrate-copy): 23 587 KiB read + 432 KiB written.
 GEMV_TRAFFIC_BYTES = 24594000
+GEMV_TRAFFIC_SOURCE = "profiles/gemv_seq_mlp_decode_M1_hbm_traffic.md"
 
 
 def gemv_bytes(M, K, N, G, act_order=False):
@@ -81,7 +82,11 @@ def time_graph(fn, steps, warmup):
     return t1 - t0, e0.elapsed_time(e1) * 1e-3
 
 
-def bench_mlp_decode(M, steps, warmup, n_layers=32, seed=1):
+def bench_mlp_decode(M, steps, warmup, n_layers=32, seed=1, grouped=True):
+    """One step = one token (M rows) through the MLP products of n_layers decoder layers over distinct weights:
+    gate and up (which share their input) as ONE grouped launch on their own tensors, then down.
+    grouped=False issues gate and up as two launches.  Returns the whole-step figures and, from two more graphs
+    holding only the gate|up launches and only the down launches, the average duration of each kernel."""
     import torch
     from alpaca_lora_4bit_amd import quant_hip
     gen = torch.Generator(device="cuda").manual_seed(seed)
@@ -93,29 +98,49 @@ def bench_mlp_decode(M, steps, warmup, n_layers=32, seed=1):
             torch.empty((M, 11008), dtype=torch.float16, device="cuda"),
             torch.empty((M, 4096), dtype=torch.float16, device="cuda")]
 
+    def gate_up(lay):
+        if grouped:
+            quant_hip.gemv_grouped(x, [(l["qweight"], l["qzeros"], l["scales"]) for l in lay[:2]], 128, outs=outs[:2])
+        else:
+            for l, out in zip(lay[:2], outs[:2]):
+                quant_hip.gemv(x, l["qweight"], l["qzeros"], l["scales"], None, 128, out=out)
+
+    def down(lay):
+        l = lay[2]
+        quant_hip.gemv(h, l["qweight"], l["qzeros"], l["scales"], None, 128, out=outs[2])
+
     def step():
         for lay in layers:
-            for (l, inp, out) in zip(lay, (x, x, h), outs):
-                quant_hip.gemv(inp, l["qweight"], l["qzeros"], l["scales"], None, 128, out=out)
+            gate_up(lay)
+            down(lay)
 
     # sanity: the timed path computes the right thing (against the HIP dense dequant + fp32 matmul)
-    l0 = layers[0][0]
-    y = quant_hip.gemv(x, l0["qweight"], l0["qzeros"], l0["scales"], None, 128)
-    W = quant_hip.dequant(l0["qweight"], l0["qzeros"], l0["scales"], None, 128)
-    ref = x.float() @ W.float()
-    err = float((y.float() - ref).abs().max() / ref.abs().max())
-    assert err < 1e-2, f"gemv sanity check failed: {err}"
-    del W, ref
+    errs = []
+    gate_up(layers[0])
+    down(layers[0])
+    for l, inp, out in zip(layers[0], (x, x, h), outs):
+        W = quant_hip.dequant(l["qweight"], l["qzeros"], l["scales"], None, 128)
+        ref = inp.float() @ W.float()
+        errs.append(float((out.float() - ref).abs().max() / ref.abs().max()))
+        del W, ref
+    err = max(errs)
+    assert err < 1e-2, f"gemv sanity check failed: {errs}"
 
     wall, ev = time_graph(step, steps, warmup)
-    launches = 3 * n_layers
-    bytes_per_launch = gemv_bytes(M, 4096, 11008, 32)           # same total for the down shape
-    bytes_per_step = launches * bytes_per_launch
-    return dict(wall_s=wall, event_s=ev, steps=steps, launches_per_step=launches,
-                bytes_per_launch=bytes_per_launch, bytes_per_step=bytes_per_step,
+    _, ev_gu = time_graph(lambda: [gate_up(lay) for lay in layers], steps, 1)
+    _, ev_dn = time_graph(lambda: [down(lay) for lay in layers], steps, 1)
+    b_one = gemv_bytes(M, 4096, 11008, 32)                      # same total for the down shape
+    b_gu = 2 * b_one - 2 * M * 4096 if grouped else b_one       # grouped: the shared activations are read once
+    launches_gu = n_layers if grouped else 2 * n_layers
+    launches = launches_gu + n_layers
+    bytes_per_step = launches_gu * b_gu + n_layers * b_one
+    us_gu = ev_gu / (steps * launches_gu) * 1e6
+    us_dn = ev_dn / (steps * n_layers) * 1e6
+    return dict(wall_s=wall, event_s=ev, steps=steps, launches_per_step=launches, bytes_per_step=bytes_per_step,
                 gbs_wall=bytes_per_step * steps / wall / 1e9,
-                avg_launch_us=ev / (steps * launches) * 1e6,
-                gbs_kernel=bytes_per_launch / (ev / (steps * launches)) / 1e9, sanity_rel_err=err)
+                gate_up=dict(bytes=b_gu, us=us_gu, gbs=b_gu / us_gu / 1e3),
+                down=dict(bytes=b_one, us=us_dn, gbs=b_one / us_dn / 1e3),
+                sum_of_kernels_ms=(launches_gu * us_gu + n_layers * us_dn) * 1e-3, sanity_rel_err=err)
 
 
 def bench_single_gemv(K, N, M, act_order, reps, copies, seed=3):
@@ -494,22 +519,36 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16 (int4 weights, fp32 accumulate)", "data": "synthetic",
         "config": {"workload": "configs[1]: LLaMA-7B MLP decode GEMV, M=1, gate/up 4096->11008 + down 11008->4096, "
-                               "groupsize 128, no act-order; step = 32 layers x 3 GEMVs over 2.25 GB of distinct "
-                               "packed weights, replayed as one HIP graph",
+                               "groupsize 128, no act-order; step = 32 layers x (gate|up as one grouped launch on their "
+                               "own tensors + down) over 2.25 GB of distinct packed weights, replayed as one HIP graph",
                    "M": 1, "layers": 32, "launches_per_step": head["launches_per_step"],
                    "bytes_per_step": head["bytes_per_step"]},
         "pct_of_hbm_peak": round(100 * head["gbs_wall"] / HBM_PEAK_GBS, 2),
-        "roofline": {"bound": "hbm", "achieved": round(head["gbs_kernel"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(head["gbs_kernel"] / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES,
-                     "kernel": "q4::gemv_seq_kernel<4, 0, false>", "bytes_per_launch": head["bytes_per_launch"],
-                     "avg_launch_us": round(head["avg_launch_us"], 3)},
+        # dominant kernel = the grouped gate|up launch (two thirds of the step's bytes and most of its time)
+        "roofline": {"bound": "hbm", "achieved": round(head["gate_up"]["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(head["gate_up"]["gbs"] / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES,
+                     "traffic_source": GEMV_TRAFFIC_SOURCE,
+                     "kernel": "q4::gemv_seq_group_kernel<4, 0> (gate|up, N = 2 x 11008)",
+                     "bytes_per_launch": head["gate_up"]["bytes"], "avg_launch_us": round(head["gate_up"]["us"], 3),
+                     "other_kernel": {"kernel": "q4::gemv_seq_kernel<4, 0, false> (down, 11008 -> 4096)",
+                                      "bytes_per_launch": head["down"]["bytes"],
+                                      "avg_launch_us": round(head["down"]["us"], 3),
+                                      "frac": round(head["down"]["gbs"] / HBM_PEAK_GBS, 4)},
+                     "sum_of_kernel_durations_ms": round(head["sum_of_kernels_ms"], 4)},
     }
     if not args.no_extra:
         extra = {}
         for M in (4, 16):
             r = bench_mlp_decode(M, max(args.steps // 2, 5), 2)
-            extra[f"mlp_decode_M{M}"] = {"gbs": round(r["gbs_kernel"], 1), "us_per_gemv": round(r["avg_launch_us"], 3),
-                                         "frac_hbm": round(r["gbs_kernel"] / HBM_PEAK_GBS, 4)}
+            extra[f"mlp_decode_M{M}"] = {"step_gbs": round(r["gbs_wall"], 1),
+                                         "gate_up_grouped_us": round(r["gate_up"]["us"], 3),
+                                         "gate_up_grouped_frac_hbm": round(r["gate_up"]["gbs"] / HBM_PEAK_GBS, 4),
+                                         "down_us": round(r["down"]["us"], 3),
+                                         "down_frac_hbm": round(r["down"]["gbs"] / HBM_PEAK_GBS, 4)}
+        r = bench_mlp_decode(1, max(args.steps // 2, 5), 2, grouped=False)
+        extra["mlp_decode_M1_three_launches"] = {"step_gbs": round(r["gbs_wall"], 1), "gate_or_up_us": round(r["gate_up"]["us"], 3),
+                                                 "gate_or_up_frac_hbm": round(r["gate_up"]["gbs"] / HBM_PEAK_GBS, 4),
+                                                 "down_us": round(r["down"]["us"], 3)}
         # gate and up share x: concatenated along N they are one launch of twice the size
         gu = bench_single_gemv(4096, 22016, 1, False, 10, 16)
         extra["mlp_decode_M1_gate_up_fused_N22016"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in gu.items()}

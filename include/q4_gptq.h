@@ -86,6 +86,28 @@ int q4_gemv_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, co
                 int M, int K, int N, int G,
                 void *workspace, size_t workspace_bytes, void *stream);
 
+/* Several layers in ONE launch: y_i fp16 [M, N_i] = x_i fp16 [M, K] @ W_i for 1 <= n_layers <= Q4_GEMV_MAX_GROUP layers
+ * that share M, K and the group size (sequential groups only: g_idx[k] == k / groupsize), each read in place from
+ * its own tensors -- q_proj | k_proj | v_proj or gate_proj | up_proj of a decoder block with x_i all the same
+ * pointer.  The reference gets the same effect by concatenating the packed tensors of the projections along N
+ * (model_attn_mlp_patch.py:88-100, 180-190) and calling vecquant4matmul once; here the checkpoint tensors stay as
+ * they are.  `layers` is an array in HOST memory (copied into the kernel arguments; not referenced after the call
+ * returns).  Per layer the limits of q4_gemv_f16 apply; K <= 1 044 480.  `workspace`: q4_gemv_grouped_workspace_bytes(M,
+ * N_0 + .. + N_{n-1}) = 8 * M * sum(N_i) bytes, 256-byte aligned, zero before its first use, left zero by every call
+ * (a workspace kept for q4_gemv_f16 can be shared: same convention). */
+#define Q4_GEMV_MAX_GROUP 4
+typedef struct q4_gemv_layer {
+    const void *x;             /* fp16 [M, K] */
+    const int32_t *qweight;    /* int32 [K/8, N] */
+    const int32_t *qzeros;     /* int32 [G, N/8], G = ceil(K / groupsize) */
+    const void *scales;        /* fp16 [G, N] */
+    void *y;                   /* fp16 [M, N] */
+    int N;
+} q4_gemv_layer_t;
+size_t q4_gemv_grouped_workspace_bytes(int M, int total_N);
+int q4_gemv_grouped_f16(const q4_gemv_layer_t *layers, int n_layers, int groupsize, int accumulate,
+                        int M, int K, void *workspace, size_t workspace_bytes, void *stream);
+
 /* q4_gemv_f16 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same product, same arguments
  * minus the workspace: the split-K accumulators live in a device array inside the library (4 MiB per device that

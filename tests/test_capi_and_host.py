@@ -95,6 +95,22 @@ def test_error_codes_and_validation_need_no_gpu():
     assert L.q4_gemv_noalloc_f16(fake, fake, fake, fake, None, 128, fake, 0, 17, 256, 128, 2, None) == -2
     assert L.q4_gemv_noalloc_f16(None, fake, fake, fake, None, 128, fake, 0, 1, 256, 128, 2, None) == -1
     assert L.q4_gemv_noalloc_f16(fake, fake, fake, fake, None, 128, odd, 0, 1, 256, 128, 2, None) == -5
+    # grouped GEMV: descriptors in host memory, validated layer by layer
+    lay = (_lib.GemvLayer * 2)()
+    for d in lay:
+        d.x = d.qweight = d.qzeros = d.scales = d.y = 0x1000
+        d.N = 128
+    assert L.q4_gemv_grouped_workspace_bytes(4, 22016) == 4 * 22016 * 8
+    assert L.q4_gemv_grouped_f16(None, 2, 128, 0, 1, 256, fake, 1 << 20, None) == -1
+    assert L.q4_gemv_grouped_f16(lay, 5, 128, 0, 1, 256, fake, 1 << 20, None) == -2          # more than 4 layers
+    assert L.q4_gemv_grouped_f16(lay, 2, 100, 0, 1, 256, fake, 1 << 20, None) == -2          # groupsize % 32
+    assert L.q4_gemv_grouped_f16(lay, 2, 128, 0, 17, 256, fake, 1 << 20, None) == -2         # rows
+    assert L.q4_gemv_grouped_f16(lay, 2, 128, 0, 1, 256, fake, 2047, None) == -3             # needs 2 * 128 * 8 bytes
+    lay[1].N = 100
+    assert L.q4_gemv_grouped_f16(lay, 2, 128, 0, 1, 256, fake, 1 << 20, None) == -2          # N % 64 of the second layer
+    lay[1].N = 128
+    lay[1].y = 0
+    assert L.q4_gemv_grouped_f16(lay, 2, 128, 0, 1, 256, fake, 1 << 20, None) == -1
     assert L.q4_gemv_workspace_bytes(16, 4096, 11008) == 16 * 11008 * 8
     assert L.q4_gemv_workspace_bytes(0, 4096, 11008) == 0
 

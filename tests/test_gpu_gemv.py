@@ -136,3 +136,51 @@ def test_two_streams_and_two_threads_use_separate_workspaces(oracle):
     for i in range(2):
         assert all(torch.equal(y, want[i]) for y in got[i])
         assert all(torch.equal(y, want_g[i]) for y in got_g[i])
+
+
+@pytest.mark.parametrize("M", [1, 3, 16])
+@pytest.mark.parametrize("K,Ns,gs", [(4096, (11008, 11008), 128), (4096, (4096, 1024, 1024), 128), (512, (64, 192, 128, 320), 64),
+                                     (11008, (4096,), 128), (256, (128, 64), 32)])
+def test_gemv_grouped_matches_single_launches_and_oracle(oracle, K, Ns, gs, M):
+    """q4_gemv_grouped_f16: several layers in one launch, each read from its own tensors.  Same kernels and the same
+    fixed-order integer reduction as q4_gemv_f16, so each output is bit-identical to the single-layer launch;
+    both are held to the oracle."""
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    layers = [oracle.make_layer(K, N, gs, seed=K + 5 * N + i) for i, N in enumerate(Ns)]
+    ts = [to_cuda_layer(l) for l in layers]
+    xh = oracle.make_activations(M, K, seed=M + 3)
+    x = torch.from_numpy(xh).cuda()
+    outs = quant_hip.gemv_grouped(x, [(t["qweight"], t["qzeros"], t["scales"]) for t in ts], gs)
+    torch.cuda.synchronize()
+    assert len(outs) == len(Ns)
+    for lay, t, y in zip(layers, ts, outs):
+        single = quant_hip.gemv(x, t["qweight"], t["qzeros"], t["scales"], None, gs)
+        assert torch.equal(y, single)
+        ref = oracle.matmul_recons(xh, lay["qweight"], lay["qzeros"], lay["scales"], lay["g_idx"])
+        assert rel_err(y.cpu().numpy(), ref) <= TOL
+    # one activation tensor per layer, g_idx given (sequential), accumulate into existing outputs
+    xs = [torch.from_numpy(oracle.make_activations(M, K, seed=40 + i)).cuda() for i in range(len(Ns))]
+    base = [torch.full((M, N), 0.5, dtype=torch.float16, device="cuda") for N in Ns]
+    quant_hip.gemv_grouped(xs, [(t["qweight"], t["qzeros"], t["scales"], t["g_idx"]) for t in ts], gs, outs=base,
+                           accumulate=True)
+    for lay, xi, y in zip(layers, xs, base):
+        ref = oracle.matmul_recons(xi.cpu().numpy(), lay["qweight"], lay["qzeros"], lay["scales"], lay["g_idx"]) + 0.5
+        assert rel_err(y.cpu().numpy(), ref) <= TOL
+    for ws in quant_hip._workspaces.values():                 # accumulators left zeroed
+        assert int(ws[:65536].view(torch.int32).abs().sum()) == 0
+
+
+def test_gemv_grouped_rejects_act_order_and_mismatched_layers(oracle):
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    a = to_cuda_layer(oracle.make_layer(256, 128, 128, act_order=True, seed=1))
+    b = to_cuda_layer(oracle.make_layer(512, 128, 128, seed=2))
+    c = to_cuda_layer(oracle.make_layer(256, 128, 128, seed=3))
+    x = torch.zeros((1, 256), dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):
+        quant_hip.gemv_grouped(x, [(a["qweight"], a["qzeros"], a["scales"], a["g_idx"])], 128)
+    with pytest.raises(ValueError):
+        quant_hip.gemv_grouped(x, [(c["qweight"], c["qzeros"], c["scales"]), (b["qweight"], b["qzeros"], b["scales"])], 128)
+    with pytest.raises(ValueError):
+        quant_hip.gemv_grouped(x, [(c["qweight"], c["qzeros"], c["scales"])] * 5, 128)
