@@ -6,7 +6,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libq4gptq.so")
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 _lib = None
 
@@ -27,12 +27,19 @@ SIGNATURES = {
     "q4_dequant2_f16": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp]),
     "q4_gemm_workspace_bytes": (_sz, [_i, _i, _i, _i]),
     "q4_gemm_fwd_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _i, _vp, _i, _i, _i, _i, _vp, _sz, _vp]),
-    "q4_gemm_bwd_dx_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _i, _vp, _i, _i, _i, _i, _vp, _sz, _vp]),
-    "q4_lora_down_f16": (_i, [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp]),
+    "q4_gemm_bwd_dx_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _i, _vp, _i, _i, _i, _i, _vp, _vp, _sz, _vp]),
+    "q4_lora_down_f16": (_i, [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp, _vp]),
     "q4_lora_grad_workspace_bytes": (_sz, [_i, _i, _i]),
-    "q4_lora_grad_f32": (_i, [_vp, _vp, _vp, _i, _i, _f, _i, _i, _i, _vp, _sz, _vp]),
-    "q4_lora_grad_pair_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _vp, _sz, _vp]),
+    "q4_lora_grad_f32": (_i, [_vp, _vp, _vp, _i, _i, _f, _i, _i, _i, _vp, _vp, _sz, _vp]),
+    "q4_lora_grad_pair_f32": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _vp, _vp, _sz, _vp]),
+    "q4_dropout_scale": (_f, [_f]),
+    "q4_dropout_keep_u8": (_i, [_vp, _i, _i, _vp, _vp]),
 }
+
+
+class Dropout(ctypes.Structure):
+    """q4_dropout_t of include/q4_gptq.h."""
+    _fields_ = [("seed_lo", ctypes.c_uint32), ("seed_hi", ctypes.c_uint32), ("p", _f)]
 
 
 class GemvLayer(ctypes.Structure):

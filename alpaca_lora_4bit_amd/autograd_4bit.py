@@ -282,7 +282,13 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
     read in place by the kernels through strides: no cast, transposed or pre-scaled copies.
 
     Above matmul_utils_4bit.dense_switch_rows rows the same sums run as dense dequantization + library GEMMs
-    (the rank-r product writes the output once, the big product accumulates onto it)."""
+    (the rank-r product writes the output once, the big product accumulates onto it).
+
+    Dropout in front of lora_A (models.py:63-66; the reference's default is p = 0.05, arg_parser.py:48) stays
+    inside the same kernels: with drop_p > 0 the adapter sees xd = dropout(x) under a mask that is a pure
+    function of (drop_seed, row, column) and is regenerated wherever it is needed instead of being stored:
+        fwd   xa = xd @ A^T                       bwd   dA = scaling * dyb^T @ xd
+              dx = dy @ W^T + mask/(1-p) * (scaling * dyb @ A)          dB = scaling * dy^T @ xa"""
 
     @staticmethod
     def _kernel_dtype(w):
@@ -300,8 +306,10 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
 
     @staticmethod
     @custom_fwd(device_type='cuda', cast_inputs=None)
-    def forward(ctx, x, qweight, scales, zeros, g_idx, bias, lora_a, lora_b, scaling, groupsize):
+    def forward(ctx, x, qweight, scales, zeros, g_idx, bias, lora_a, lora_b, scaling, groupsize, drop_p=0.0,
+                drop_seed=0):
         K, N = qweight.shape[0] * 8, qweight.shape[1]
+        dropout = (int(drop_seed), float(drop_p)) if drop_p and drop_p > 0.0 else None
         x2 = x.reshape(-1, K)
         if x2.dtype != torch.float16:
             x2 = x2.half()
@@ -310,7 +318,7 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
             bias = bias.half()
         a = AutogradMatmul4bitLora._kernel_dtype(lora_a.detach())
         b = AutogradMatmul4bitLora._kernel_dtype(lora_b.detach())
-        xa = quant_hip.lora_down(x2, a)
+        xa = quant_hip.lora_down(x2, a, dropout=dropout)
         if mm4b.use_dense_route(x2.shape[0]):
             w = mm4b.dense_weight(qweight, scales, zeros, g_idx, groupsize)
             y = AutogradMatmul4bitLora._dense_product(x2, w, xa, b.t(), scaling, bias).view(tuple(x.shape[:-1]) + (N,))
@@ -321,6 +329,7 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
         ctx.scaling = scaling
         ctx.groupsize = groupsize
         ctx.ab_dtypes = (lora_a.dtype, lora_b.dtype)
+        ctx.dropout = dropout
         return y
 
     @staticmethod
@@ -333,23 +342,30 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
             dy = dy.half()
         dy = dy.contiguous()
         dyb = quant_hip.lora_down(dy, b.t())
+        dropout = ctx.dropout
         dx = da = db = None
         if ctx.needs_input_grad[0]:
             dx_shape = tuple(grad_output.shape[:-1]) + (qweight.shape[0] * 8,)
             if mm4b.use_dense_route(dy.shape[0]):
                 w = mm4b.dense_weight(qweight, scales, zeros, g_idx, ctx.groupsize)
-                dx = AutogradMatmul4bitLora._dense_product(dy, w.t(), dyb, a, ctx.scaling).view(dx_shape)
+                if dropout is None:
+                    dx = AutogradMatmul4bitLora._dense_product(dy, w.t(), dyb, a, ctx.scaling).view(dx_shape)
+                else:
+                    dx = quant_hip.masked_adapter_term(dyb, a, ctx.scaling, dropout).addmm_(dy, w.t()).view(dx_shape)
             else:
                 dx = quant_hip.gemm_bwd_dx(dy, qweight, zeros, scales, g_idx, ctx.groupsize, dyb=dyb, lora_a=a,
-                                           lora_scale=ctx.scaling, out_shape=dx_shape)
+                                           lora_scale=ctx.scaling, out_shape=dx_shape, dropout=dropout)
         r = a.shape[0]
         need_a, need_b = ctx.needs_input_grad[6], ctx.needs_input_grad[7]
         if need_a and need_b and r in quant_hip.LORA_GRAD_RANKS:
-            da, db = quant_hip.lora_grad_pair(dyb, x2, xa, dy, ctx.scaling)      # one launch for both gradients
+            da, db = quant_hip.lora_grad_pair(dyb, x2, xa, dy, ctx.scaling, dropout=dropout)   # one launch for both gradients
         else:
             if need_a:
                 if r in quant_hip.LORA_GRAD_RANKS:
-                    da = quant_hip.lora_grad(dyb, x2, ctx.scaling)
+                    da = quant_hip.lora_grad(dyb, x2, ctx.scaling, dropout=dropout)
+                elif dropout is not None:
+                    xd = x2 * quant_hip.dropout_keep_mask(x2.shape[0], x2.shape[1], dropout[0], dropout[1], x2.device)
+                    da = torch.mm(dyb.t(), xd).float().mul_(ctx.scaling * quant_hip.dropout_scale(dropout[1]))
                 else:
                     da = torch.mm(dyb.t(), x2).float().mul_(ctx.scaling)
             if need_b:
@@ -361,7 +377,7 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
             da = da.to(ctx.ab_dtypes[0])
         if db is not None:
             db = db.to(ctx.ab_dtypes[1])
-        return dx, None, None, None, None, None, da, db, None, None
+        return dx, None, None, None, None, None, da, db, None, None, None, None
 
 
 _LOADER_NAMES = ('load_llama_model_4bit_low_ram', 'load_llama_model_4bit_low_ram_and_offload',

@@ -9,15 +9,19 @@ int q4_launch_dequant(const int32_t*, const int32_t*, const void*, const int32_t
 int q4_launch_permute_rows(const int32_t*, const int32_t*, int32_t*, int, int, hipStream_t);
 int q4_launch_gemv(const void*, const int32_t*, const int32_t*, const void*, const int32_t*, const int32_t*, int, void*,
                    int, int, int, int, int, void*, hipStream_t);
+struct q4_drop_args { uint32_t seed_lo, seed_hi, thr15; float scale; };     // q4::DropArgs of q4_common.hpp
 int q4_launch_gemm(int, const void*, const int32_t*, const int32_t*, const void*, const int32_t*, int, const void*,
-                   const void*, const void*, int, int, int, float, int, void*, int, int, int, int, void*, size_t, hipStream_t);
+                   const void*, const void*, int, int, int, float, int, void*, int, int, int, int, const q4_drop_args*,
+                   void*, size_t, hipStream_t);
+int q4_launch_dropout_keep(uint8_t*, int, int, const q4_drop_args*, hipStream_t);
 size_t q4_gemm_plan_workspace(int, int, int, int);
 int q4_gemv_sorted_applicable(int, int);
 int q4_launch_gemv_v1(const void*, const int32_t*, const void*, const void*, void*, int, int, int, int, void*, hipStream_t);
-int q4_launch_lora_down(const void*, const void*, int, int, int, void*, int, int, int, hipStream_t);
-int q4_launch_lora_grad(const void*, const void*, float*, int, int, float, int, int, int, void*, hipStream_t);
+int q4_launch_lora_down(const void*, const void*, int, int, int, void*, int, int, int, const q4_drop_args*, hipStream_t);
+int q4_launch_lora_grad(const void*, const void*, float*, int, int, float, int, int, int, const q4_drop_args*, void*,
+                        hipStream_t);
 int q4_launch_lora_grad_pair(const void*, const void*, float*, int, int, int, const void*, const void*, float*, int, int, int,
-                             float, int, int, void*, hipStream_t);
+                             float, int, int, const q4_drop_args*, void*, hipStream_t);
 size_t q4_lora_grad_workspace(int, int, int);
 int q4_launch_gemv_group(int, const void* const*, const int32_t* const*, const int32_t* const*, const void* const*,
                          void* const*, const int*, int, int, int, int, int, void*, hipStream_t);
@@ -28,6 +32,19 @@ int q4_launch_zero_words(void*, size_t, hipStream_t);
 
 namespace {
 inline bool misaligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) != 0; }
+
+// Public dropout descriptor -> kernel arguments.  Returns false for p outside [0, 1).
+bool make_drop(const q4_dropout_t* d, q4_drop_args* out, const q4_drop_args** ptr) {
+    *ptr = nullptr;
+    if (!d) return true;
+    if (!(d->p >= 0.0f) || !(d->p < 1.0f)) return false;
+    uint32_t thr = (uint32_t)(d->p * 32768.0f + 0.5f);
+    if (thr > 32767u) thr = 32767u;
+    out->seed_lo = d->seed_lo; out->seed_hi = d->seed_hi; out->thr15 = thr;
+    out->scale = 32768.0f / (float)(32768u - thr);
+    if (thr != 0) *ptr = out;
+    return true;
+}
 
 int check_layer(const void* qweight, const void* qzeros, const void* scales, const void* g_idx,
                 int groupsize, int K, int N, int G) {
@@ -43,7 +60,7 @@ int check_layer(const void* qweight, const void* qzeros, const void* scales, con
 }
 }  // namespace
 
-extern "C" int q4_abi_version(void) { return 9; }
+extern "C" int q4_abi_version(void) { return 10; }
 
 extern "C" const char* q4_error_string(int code) {
     switch (code) {
@@ -204,9 +221,13 @@ extern "C" int q4_gemv_v1_f16(const void* x, const int32_t* qweight, const void*
 static int gemm_common(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros, const void* scales,
                        const int32_t* g_idx, int groupsize, const void* bias, const void* la, const void* lb,
                        int lb_sr, int lb_sc, int lb_is_f32, float lb_scale, int R,
-                       void* out, int M, int K, int N, int G, void* workspace, size_t workspace_bytes, void* stream) {
+                       void* out, int M, int K, int N, int G, const q4_dropout_t* drop,
+                       void* workspace, size_t workspace_bytes, void* stream) {
     int rc = check_layer(qweight, qzeros, scales, g_idx, groupsize, K, N, G);
     if (rc != Q4_OK) return rc;
+    q4_drop_args da;
+    const q4_drop_args* dp;
+    if (!make_drop(drop, &da, &dp)) return Q4_ERR_BAD_SHAPE;
     if (!act || !out) return Q4_ERR_NULL_POINTER;
     if (M < 1 || (K % 128) != 0 || (N % 128) != 0) return Q4_ERR_BAD_SHAPE;
     if (!g_idx && (groupsize % 64) != 0) return Q4_ERR_BAD_SHAPE;
@@ -220,7 +241,7 @@ static int gemm_common(int fwd, const void* act, const int32_t* qweight, const i
     if (lb && (lb_sr < 1 || lb_sc < 1)) return Q4_ERR_BAD_SHAPE;
     if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
     return q4_launch_gemm(fwd, act, qweight, qzeros, scales, g_idx, groupsize, bias, la, lb, lb_sr, lb_sc, lb_is_f32,
-                          lb_scale, R, out, M, K, N, G, workspace, workspace ? workspace_bytes : 0, (hipStream_t)stream);
+                          lb_scale, R, out, M, K, N, G, dp, workspace, workspace ? workspace_bytes : 0, (hipStream_t)stream);
 }
 
 extern "C" int q4_gemm_fwd_f16(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
@@ -229,16 +250,16 @@ extern "C" int q4_gemm_fwd_f16(const void* x, const int32_t* qweight, const int3
                                float lora_scale, int R, void* y, int M, int K, int N, int G,
                                void* workspace, size_t workspace_bytes, void* stream) {
     return gemm_common(1, x, qweight, qzeros, scales, g_idx, groupsize, bias, xa, lora_b, ldb_r, ldb_n, lora_is_f32,
-                       lora_scale, R, y, M, K, N, G, workspace, workspace_bytes, stream);
+                       lora_scale, R, y, M, K, N, G, nullptr, workspace, workspace_bytes, stream);
 }
 
 extern "C" int q4_gemm_bwd_dx_f16(const void* dy, const int32_t* qweight, const int32_t* qzeros, const void* scales,
                                   const int32_t* g_idx, int groupsize,
                                   const void* dyb, const void* lora_a, int lda_r, int lda_k, int lora_is_f32,
                                   float lora_scale, int R, void* dx, int M, int K, int N, int G,
-                                  void* workspace, size_t workspace_bytes, void* stream) {
+                                  const q4_dropout_t* drop, void* workspace, size_t workspace_bytes, void* stream) {
     return gemm_common(0, dy, qweight, qzeros, scales, g_idx, groupsize, nullptr, dyb, lora_a, lda_r, lda_k, lora_is_f32,
-                       lora_scale, R, dx, M, K, N, G, workspace, workspace_bytes, stream);
+                       lora_scale, R, dx, M, K, N, G, drop, workspace, workspace_bytes, stream);
 }
 
 extern "C" size_t q4_gemm_workspace_bytes(int fwd, int M, int K, int N) {
@@ -247,15 +268,18 @@ extern "C" size_t q4_gemm_workspace_bytes(int fwd, int M, int K, int N) {
 }
 
 extern "C" int q4_lora_down_f16(const void* in, const void* w, int w_sr, int w_sc, int w_is_f32, void* out,
-                                int M, int C, int R, void* stream) {
+                                int M, int C, int R, const q4_dropout_t* drop, void* stream) {
     if (!in || !w || !out) return Q4_ERR_NULL_POINTER;
+    q4_drop_args da;
+    const q4_drop_args* dp;
+    if (!make_drop(drop, &da, &dp)) return Q4_ERR_BAD_SHAPE;
     if (M < 1 || C < 32 || (C % 32) != 0 || R < 1 || R > 64 || w_sr < 1 || w_sc < 1) return Q4_ERR_BAD_SHAPE;
     /* 32-bit buffer offsets: the 16-row block of `in` and the span of the adapter matrix */
     if ((long long)C * 32 >= 0x70000000ll) return Q4_ERR_BAD_SHAPE;
     if (((long long)(R - 1) * w_sr + (long long)(C - 1) * w_sc + 1) * (w_is_f32 ? 4 : 2) >= 0x70000000ll) return Q4_ERR_BAD_SHAPE;
     if (misaligned(in) || (reinterpret_cast<uintptr_t>(out) & 1u) || (reinterpret_cast<uintptr_t>(w) & (w_is_f32 ? 3u : 1u)))
         return Q4_ERR_MISALIGNED;
-    return q4_launch_lora_down(in, w, w_sr, w_sc, w_is_f32, out, M, C, R, (hipStream_t)stream);
+    return q4_launch_lora_down(in, w, w_sr, w_sc, w_is_f32, out, M, C, R, dp, (hipStream_t)stream);
 }
 
 extern "C" size_t q4_lora_grad_workspace_bytes(int M, int C, int R) {
@@ -264,8 +288,12 @@ extern "C" size_t q4_lora_grad_workspace_bytes(int M, int C, int R) {
 }
 
 extern "C" int q4_lora_grad_f32(const void* p, const void* in, float* out, int o_sr, int o_sc, float alpha,
-                                int M, int C, int R, void* workspace, size_t workspace_bytes, void* stream) {
+                                int M, int C, int R, const q4_dropout_t* drop,
+                                void* workspace, size_t workspace_bytes, void* stream) {
     if (!p || !in || !out) return Q4_ERR_NULL_POINTER;
+    q4_drop_args da;
+    const q4_drop_args* dp;
+    if (!make_drop(drop, &da, &dp)) return Q4_ERR_BAD_SHAPE;
     if (M < 1 || C < 8 || (C % 8) != 0 || (R != 8 && R != 16) || o_sr < 1 || o_sc < 1) return Q4_ERR_BAD_SHAPE;
     if ((long long)M * C * 2 >= 0x70000000ll || C > (1 << 20)) return Q4_ERR_BAD_SHAPE;     /* 32-bit buffer offsets */
     if (misaligned(p) || misaligned(in) || (reinterpret_cast<uintptr_t>(out) & 3u)) return Q4_ERR_MISALIGNED;
@@ -274,13 +302,17 @@ extern "C" int q4_lora_grad_f32(const void* p, const void* in, float* out, int o
         if (!workspace || workspace_bytes < need) return Q4_ERR_WORKSPACE;
         if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
     }
-    return q4_launch_lora_grad(p, in, out, o_sr, o_sc, alpha, M, C, R, workspace, (hipStream_t)stream);
+    return q4_launch_lora_grad(p, in, out, o_sr, o_sc, alpha, M, C, R, dp, workspace, (hipStream_t)stream);
 }
 
 extern "C" int q4_lora_grad_pair_f32(const void* p1, const void* in1, float* out1, int o1_sr, int o1_sc, int C1,
                                      const void* p2, const void* in2, float* out2, int o2_sr, int o2_sc, int C2,
-                                     float alpha, int M, int R, void* workspace, size_t workspace_bytes, void* stream) {
+                                     float alpha, int M, int R, const q4_dropout_t* drop1,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
     if (!p1 || !in1 || !out1 || !p2 || !in2 || !out2) return Q4_ERR_NULL_POINTER;
+    q4_drop_args da;
+    const q4_drop_args* dp;
+    if (!make_drop(drop1, &da, &dp)) return Q4_ERR_BAD_SHAPE;
     if (M < 1 || (R != 8 && R != 16)) return Q4_ERR_BAD_SHAPE;
     const int Cs[2] = {C1, C2};
     const int strides[4] = {o1_sr, o1_sc, o2_sr, o2_sc};
@@ -297,5 +329,23 @@ extern "C" int q4_lora_grad_pair_f32(const void* p1, const void* in1, float* out
         if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
     }
     return q4_launch_lora_grad_pair(p1, in1, out1, o1_sr, o1_sc, C1, p2, in2, out2, o2_sr, o2_sc, C2, alpha, M, R,
-                                    workspace, (hipStream_t)stream);
+                                    dp, workspace, (hipStream_t)stream);
+}
+
+extern "C" float q4_dropout_scale(float p) {
+    q4_dropout_t d = {0u, 0u, p};
+    q4_drop_args da = {0u, 0u, 0u, 1.0f};
+    const q4_drop_args* dp;
+    if (!make_drop(&d, &da, &dp)) return 0.0f;
+    return dp ? da.scale : 1.0f;
+}
+
+extern "C" int q4_dropout_keep_u8(uint8_t* keep, int M, int C, const q4_dropout_t* drop, void* stream) {
+    if (!keep || !drop) return Q4_ERR_NULL_POINTER;
+    if (M < 1 || C < 2 || (C % 2) != 0) return Q4_ERR_BAD_SHAPE;
+    q4_drop_args da;
+    const q4_drop_args* dp;
+    if (!make_drop(drop, &da, &dp)) return Q4_ERR_BAD_SHAPE;
+    if (!dp) { da.seed_lo = drop->seed_lo; da.seed_hi = drop->seed_hi; da.thr15 = 0; da.scale = 1.0f; }
+    return q4_launch_dropout_keep(keep, M, C, &da, (hipStream_t)stream);
 }

@@ -87,4 +87,36 @@ __device__ __forceinline__ uint32_t buf_load16(rsrc_t r, int voff, int soff) {
     return (uint32_t)(unsigned short)__builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0);
 }
 
+// ---- counter-based dropout mask ----------------------------------------------------------------------------
+// The adapter input of Linear4bitLt is dropout(x) (src/alpaca_lora_4bit/models.py:66).  Nothing is stored for it:
+// element (row, col) of x is dropped iff a 15-bit draw that is a pure function of (seed, row, col) is below
+// thr15 = round(p * 32768), so forward (xa = dropout(x) @ A^T) and backward (dA = dyb^T @ dropout(x), and the
+// adapter's share of dx masked the same way) regenerate the same mask.  One 32-bit word serves the column pair
+// (2*pair, 2*pair + 1): bits 0..14 and 16..30.  The mixer is the "lowbias32" finalizer.
+struct DropArgs {
+    uint32_t seed_lo, seed_hi;
+    uint32_t thr15;           // 0: dropout off
+    float scale;              // 1 / (1 - thr15 / 32768): applied by the kernels to what survives
+};
+__device__ __forceinline__ uint32_t drop_row_key(const DropArgs& d, uint32_t row) { return row * 0x9E3779B1u + d.seed_lo; }
+__device__ __forceinline__ uint32_t drop_word(const DropArgs& d, uint32_t row_key, uint32_t pair) {
+    uint32_t h = row_key ^ (pair * 0x85EBCA6Bu + d.seed_hi);
+    h ^= h >> 16; h *= 0x7FEB352Du;
+    h ^= h >> 15; h *= 0x846CA68Bu;
+    h ^= h >> 16;
+    return h;
+}
+// 0xFFFF in the 16-bit half of a kept element, 0x0000 in that of a dropped one.  thr_pair = thr15 | thr15 << 16;
+// draws and threshold are 15-bit, so the signed 16-bit differences cannot overflow.
+typedef short short2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t drop_keep_mask(uint32_t word, uint32_t thr_pair) {
+    const short2_t v = __builtin_bit_cast(short2_t, word & 0x7FFF7FFFu);
+    const short2_t dropped = (v - __builtin_bit_cast(short2_t, thr_pair)) >> 15;    // all ones where draw < thr
+    return ~__builtin_bit_cast(uint32_t, dropped);
+}
+__device__ __forceinline__ bool drop_keeps(const DropArgs& d, uint32_t row, uint32_t col) {
+    const uint32_t w = drop_word(d, drop_row_key(d, row), col >> 1);
+    return ((w >> (16 * (col & 1))) & 0x7FFFu) >= d.thr15;
+}
+
 }  // namespace q4

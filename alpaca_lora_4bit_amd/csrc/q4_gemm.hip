@@ -59,6 +59,7 @@ struct GemmArgs {
     float* part;              // split-K: fp32 partial outputs [gridDim.z][M][part_cols] (gridDim.z > 1 only)
     int col_tile0;            // first column tile of this launch (a launch may cover a range of column tiles)
     int part_cols;            // columns held by `part`: those of this launch's column tiles
+    DropArgs drop;            // thr15 != 0: the adapter term of out[m, c] is kept only where dropout keeps (m, c)
 };
 
 // Which output tile a workgroup computes, and where in the reduction it starts.
@@ -463,11 +464,56 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
         });
     };
 
+    // rank-R adapter step: activations [M, R] (columns beyond R are zero) and the adapter matrix go through the LDS
+    // buffers pa / pb like one more reduction step
+    auto lora_step = [&](half_t* pa, half_t* pb) {
+        __syncthreads();
+        const rsrc_t rs_l = make_rsrc(a.la + (size_t)m0 * a.R, (unsigned)rows_valid * (unsigned)a.R * 2u);
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+            uint4_t v = {0u, 0u, 0u, 0u};
+            if (acol < a.R) v = buf_load128(rs_l, ((arow + APASS * i) * a.R + acol) * 2, 0);
+            *reinterpret_cast<uint4_t*>(pa + (arow + APASS * i) * LDS_STRIDE + acol) = v;
+        }
+        slab[0].store_lora(a, c0, pb, t);
+        __syncthreads();
+        for (int ks = 0; ks < (a.R + 15) / 16; ++ks) {
+            read_frags(af[0], bf[0], pa, pb, ks);
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][i], bf[0][j], acc[i][j], 0, 0, 0);
+        }
+    };
+    const bool lora_here = a.R > 0 && blockIdx.z == 0;
+    const bool lora_masked = lora_here && a.drop.thr15 != 0;              // uniform
+
     const int red0 = red_of(0, sr, tm.phase), red1 = red_of(1, sr, tm.phase);
     load_a(areg[0], red0);
     slab[0].load(a, rs, c0, red0);
     load_a(areg[1], red1);
     slab[1].load(a, rs, c0, red1);
+    if (lora_masked) {
+        // Dropout on the adapter input: the adapter's share of out[m, c] exists only where the mask keeps (m, c).
+        // So the adapter step runs FIRST, into the zeroed accumulators (through the second pair of LDS buffers,
+        // while the loads of the first two stages are in flight), the accumulators are masked, and the main
+        // loop adds the unmasked product on top.  The kept values carry 1/(1-p) through lb_scale.
+        lora_step(sA1, sB1);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm * WROWS + 32 * i + 8 * (r >> 2) + (lane >> 5) * 4 + (r & 3);
+                const uint32_t key = drop_row_key(a.drop, (uint32_t)m);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int col = c0 + wn * 64 + 32 * j + (lane & 31);
+                    const uint32_t w = drop_word(a.drop, key, (uint32_t)col >> 1);
+                    if (((w >> (16 * (col & 1))) & 0x7FFFu) < a.drop.thr15) acc[i][j][r] = 0.f;
+                }
+            }
+    }
     store_a(areg[0], sA0);
     static_for<0, NSL>([&](auto jc) { slab[0].template store_slice<decltype(jc)::value>(a, c0, red0, sB0); });
     __syncthreads();
@@ -477,27 +523,7 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
         step(s + 1, std::integral_constant<int, 1>{});
     }
     if (sr.cnt & 1) step(sr.cnt - 1, std::integral_constant<int, 0>{});   // an even number of steps precedes it: LDS[0]
-    if (a.R > 0 && blockIdx.z == 0) {
-        // rank-R adapter step: activations [M, R] (columns beyond R are zero), adapter matrix from lb
-        __syncthreads();
-        const rsrc_t rs_l = make_rsrc(a.la + (size_t)m0 * a.R, (unsigned)rows_valid * (unsigned)a.R * 2u);
-#pragma unroll
-        for (int i = 0; i < NA; ++i) {
-            uint4_t v = {0u, 0u, 0u, 0u};
-            if (acol < a.R) v = buf_load128(rs_l, ((arow + APASS * i) * a.R + acol) * 2, 0);
-            *reinterpret_cast<uint4_t*>(sA0 + (arow + APASS * i) * LDS_STRIDE + acol) = v;
-        }
-        slab[0].store_lora(a, c0, sB0, t);
-        __syncthreads();
-        for (int ks = 0; ks < (a.R + 15) / 16; ++ks) {
-            read_frags(af[0], bf[0], sA0, sB0, ks);
-#pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][i], bf[0][j], acc[i][j], 0, 0, 0);
-        }
-    }
+    if (lora_here && !lora_masked) lora_step(sA0, sB0);
 
     // epilogue: acc[i][j][r] is row 8*(r/4) + 4*(lane/32) + r%4, column lane%32 of its 32x32 tile.
     // Each wavefront transposes one 32 x 64 block at a time through its own 4.5 KB of LDS
@@ -703,10 +729,11 @@ int q4_launch_skinny(const void* x, const int32_t* qweight, const int32_t* qzero
 extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros,
                               const void* scales, const int32_t* g_idx, int groupsize, const void* bias,
                               const void* la, const void* lb, int lb_sr, int lb_sc, int lb_is_f32, float lb_scale, int R,
-                              void* out, int M, int K, int N, int G, void* workspace, size_t workspace_bytes,
-                              hipStream_t stream) {
+                              void* out, int M, int K, int N, int G, const q4::DropArgs* drop,
+                              void* workspace, size_t workspace_bytes, hipStream_t stream) {
     using namespace q4;
     GemmArgs a;
+    a.drop = drop ? *drop : DropArgs{0u, 0u, 0u, 1.0f};
     a.a = reinterpret_cast<const half_t*>(act);
     a.qweight = reinterpret_cast<const uint32_t*>(qweight);
     a.qzeros = reinterpret_cast<const uint32_t*>(qzeros);
@@ -717,7 +744,7 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     a.bias = reinterpret_cast<const half_t*>(bias);
     a.la = reinterpret_cast<const half_t*>(la);
     a.lb = lb;
-    a.lb_sr = lb_sr; a.lb_sc = lb_sc; a.lb_is_f32 = lb_is_f32; a.lb_scale = lb_scale;
+    a.lb_sr = lb_sr; a.lb_sc = lb_sc; a.lb_is_f32 = lb_is_f32; a.lb_scale = lb_scale * a.drop.scale;
     a.R = (la && lb) ? R : 0;
     a.out = reinterpret_cast<half_t*>(out);
     a.M = M; a.K = K; a.N = N; a.G = G;

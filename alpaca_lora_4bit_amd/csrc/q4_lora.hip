@@ -45,7 +45,7 @@ template <int RB, int WL, bool F32, int RQ>   // RQ: ceil(R/4) for kCols / kRows
 __global__ __launch_bounds__(64 * kDownWaves) void lora_down_kernel(const half_t* __restrict__ in,
                                                                     const void* __restrict__ w, int w_sr, int w_sc,
                                                                     half_t* __restrict__ out, int M, int C, int R,
-                                                                    int rows) {
+                                                                    int rows, DropArgs drop) {
     constexpr int NW = kDownWaves;
     constexpr int UN = WL == kAny ? (RB == 1 ? 4 : RB == 2 ? 2 : 1) : (RB == 1 ? 8 : 4);   // steps whose loads are issued together
     constexpr int ES = F32 ? 4 : 2;
@@ -65,6 +65,9 @@ __global__ __launch_bounds__(64 * kDownWaves) void lora_down_kernel(const half_t
     float4_t acc[RB];
 #pragma unroll
     for (int b = 0; b < RB; ++b) acc[b] = float4_t{0.f, 0.f, 0.f, 0.f};
+    // dropout of `in` (uniform branch): this lane's operand is row m0 + c, columns 32*s + 8*kk .. + 7 of step s
+    const uint32_t drop_key = drop_row_key(drop, (uint32_t)(m0 + c));
+    const uint32_t thr_pair = drop.thr15 | (drop.thr15 << 16);
 
     for (int s0 = s_begin; s0 < s_end; s0 += UN) {
         uint4_t av[UN];
@@ -190,6 +193,17 @@ __global__ __launch_bounds__(64 * kDownWaves) void lora_down_kernel(const half_t
                         bv[u][b][e] = F32 ? (half_t)__builtin_bit_cast(float, raw[u][b][e])
                                           : __builtin_bit_cast(half_t, (uint16_t)raw[u][b][e]);
         }
+        // dropout of `in`, after every load of the batch has been issued (steps past the slice hold zeros anyway)
+        if (drop.thr15) {
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                const uint32_t pair0 = (uint32_t)(s0 + u) * 16u + 4u * kk;
+                av[u].x &= drop_keep_mask(drop_word(drop, drop_key, pair0), thr_pair);
+                av[u].y &= drop_keep_mask(drop_word(drop, drop_key, pair0 + 1), thr_pair);
+                av[u].z &= drop_keep_mask(drop_word(drop, drop_key, pair0 + 2), thr_pair);
+                av[u].w &= drop_keep_mask(drop_word(drop, drop_key, pair0 + 3), thr_pair);
+            }
+        }
         // steps past the slice were loaded as zeros: they add nothing
 #pragma unroll
         for (int u = 0; u < UN; ++u)
@@ -209,7 +223,7 @@ __global__ __launch_bounds__(64 * kDownWaves) void lora_down_kernel(const half_t
 #pragma unroll
         for (int wv = 0; wv < NW; ++wv) v += red[wv][b][i];
         const int m = m0 + (i >> 4), j = 16 * b + (i & 15);
-        if ((i >> 4) < rows && m < M && j < R) out[(size_t)m * R + j] = (half_t)v;
+        if ((i >> 4) < rows && m < M && j < R) out[(size_t)m * R + j] = (half_t)(v * drop.scale);
     }
 }
 
@@ -239,6 +253,7 @@ struct GradProb {
     float* out;               // through o_sr, o_sc
     float* part;              // partial tiles [splits][col_blocks][NACC][64]
     int o_sr, o_sc, C, col_blocks, splits, rows_per_wg;
+    DropArgs drop;            // dropout mask applied to `in` (thr15 == 0: none); the result carries drop.scale
 };
 struct GradArgs {
     GradProb p[2];
@@ -255,7 +270,9 @@ __global__ __launch_bounds__(64 * kGradWaves) __attribute__((amdgpu_waves_per_eu
     float* __restrict__ out = q.out;
     float* __restrict__ part = q.part;
     const int o_sr = q.o_sr, o_sc = q.o_sc, C = q.C, rows_per_wg = q.rows_per_wg, M = ga.M;
-    const float alpha = ga.alpha;
+    const float alpha = ga.alpha * q.drop.scale;
+    const DropArgs drop = q.drop;
+    const uint32_t thr_pair = drop.thr15 | (drop.thr15 << 16);
     constexpr int CPT = 64 / R;                  // columns per thread: 8 (R = 8) or 4 (R = 16)
     constexpr int ND = CPT / 2;                  // dwords per thread and row
     constexpr int NPP = 8 * R / 64;              // pairs of P staged per lane and 16-row block
@@ -304,7 +321,16 @@ __global__ __launch_bounds__(64 * kGradWaves) __attribute__((amdgpu_waves_per_eu
             }
         }
     };
-    auto consume = [&](const RowRegs<ND, NPP>& x) {
+    auto consume = [&](RowRegs<ND, NPP>& x, int mb) {
+        if (drop.thr15) {                         // uniform: rows mb .. mb+15, this thread's column pairs c0/2 .. + ND-1
+#pragma unroll
+            for (int rr = 0; rr < 16; ++rr) {
+                const uint32_t key = drop_row_key(drop, (uint32_t)(mb + rr));
+#pragma unroll
+                for (int d = 0; d < ND; ++d)
+                    x.d[rr][d] &= drop_keep_mask(drop_word(drop, key, (uint32_t)(c0 >> 1) + d), thr_pair);
+            }
+        }
         // pairs of P -> LDS (wavefront-private region; LDS operations of one wavefront are ordered)
 #pragma unroll
         for (int t = 0; t < NPP; ++t) ppair[wave][lane + 64 * t] = x.plo[t] | (x.phi[t] << 16);
@@ -340,9 +366,9 @@ __global__ __launch_bounds__(64 * kGradWaves) __attribute__((amdgpu_waves_per_eu
     load_rows(xa, m_begin);
     for (int mb = m_begin; mb < m_end; mb += 32) {
         load_rows(xb, mb + 16);
-        consume(xa);
+        consume(xa, mb);
         load_rows(xa, mb + 32);
-        if (mb + 16 < m_end) consume(xb);
+        if (mb + 16 < m_end) consume(xb, mb + 16);
     }
 #pragma unroll
     for (int j = 0; j < R; ++j)
@@ -372,7 +398,7 @@ __global__ __launch_bounds__(256) void lora_grad_reduce_kernel(GradArgs ga) {
     const float* __restrict__ part = q.part;
     float* __restrict__ out = q.out;
     const int o_sr = q.o_sr, o_sc = q.o_sc, C = q.C, col_blocks = q.col_blocks, splits = q.splits;
-    const float alpha = ga.alpha;
+    const float alpha = ga.alpha * q.drop.scale;
     constexpr int CPT = 64 / R;
     constexpr int NACC = R * CPT;
     const int t = blockIdx.x * 256 + threadIdx.x;         // index into one split's tiles: [column block][a][lane]
@@ -394,6 +420,18 @@ __global__ __launch_bounds__(256) void lora_grad_reduce_kernel(GradArgs ga) {
     if (cc < C) out[(size_t)j * o_sr + (size_t)cc * o_sc] = alpha * v;
 }
 
+// keep[m, c] = 1 where dropout keeps element (m, c), else 0: the mask the kernels above regenerate, written out
+// for callers (and tests) that need to see it.
+__global__ __launch_bounds__(256) void dropout_keep_kernel(uint8_t* __restrict__ keep, int M, int C, DropArgs drop) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;              // one column pair per thread
+    const long pairs = (long)M * (C / 2);
+    if (i >= pairs) return;
+    const int m = (int)(i / (C / 2)), pr = (int)(i - (long)m * (C / 2));
+    const uint32_t w = drop_word(drop, drop_row_key(drop, (uint32_t)m), (uint32_t)pr);
+    keep[(size_t)m * C + 2 * pr] = (w & 0x7FFFu) >= drop.thr15;
+    keep[(size_t)m * C + 2 * pr + 1] = ((w >> 16) & 0x7FFFu) >= drop.thr15;
+}
+
 struct GradPlan { int col_blocks, splits, rows_per_wg; };
 inline GradPlan plan_grad(int M, int C, int R) {
     GradPlan g;
@@ -413,7 +451,7 @@ inline GradPlan plan_grad(int M, int C, int R) {
 
 template <int RB, int WL, bool F32, int RQ>
 static void launch_down_kernel(const q4::half_t* ip, const void* w, int w_sr, int w_sc, q4::half_t* op,
-                               int M, int C, int R, hipStream_t stream) {
+                               int M, int C, int R, const q4::DropArgs& drop, hipStream_t stream) {
     // rows of `in` per workgroup: 16 fill the MFMA operand, but with few rows that leaves compute units idle and
     // the kernel is bound by the latency of its single burst of loads, so smaller blocks spread it out
     static const int force_rows = getenv("Q4_LORA_DOWN_ROWS") ? atoi(getenv("Q4_LORA_DOWN_ROWS")) : 0;
@@ -421,50 +459,51 @@ static void launch_down_kernel(const q4::half_t* ip, const void* w, int w_sr, in
     while (rows > 4 && (M + rows - 1) / rows < 256) rows >>= 1;
     if (force_rows == 4 || force_rows == 8 || force_rows == 16) rows = force_rows;
     hipLaunchKernelGGL((q4::lora_down_kernel<RB, WL, F32, RQ>), dim3((M + rows - 1) / rows), dim3(64 * q4::kDownWaves), 0,
-                       stream, ip, w, w_sr, w_sc, op, M, C, R, rows);
+                       stream, ip, w, w_sr, w_sc, op, M, C, R, rows, drop);
 }
 
 template <int WL, bool F32>
 static void launch_down_rb(const q4::half_t* ip, const void* w, int w_sr, int w_sc, q4::half_t* op,
-                           int M, int C, int R, hipStream_t stream) {
+                           int M, int C, int R, const q4::DropArgs& drop, hipStream_t stream) {
     switch ((R + 15) / 16) {
-        case 1: launch_down_kernel<1, WL, F32, 0>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
-        case 2: launch_down_kernel<2, WL, F32, 0>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
-        case 3: launch_down_kernel<3, WL, F32, 0>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
-        default: launch_down_kernel<4, WL, F32, 0>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
+        case 1: launch_down_kernel<1, WL, F32, 0>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream); break;
+        case 2: launch_down_kernel<2, WL, F32, 0>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream); break;
+        case 3: launch_down_kernel<3, WL, F32, 0>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream); break;
+        default: launch_down_kernel<4, WL, F32, 0>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream); break;
     }
 }
 
 template <int WL, bool F32>
 static void launch_down_staged(const q4::half_t* ip, const void* w, int w_sr, int w_sc, q4::half_t* op,
-                             int M, int C, int R, hipStream_t stream) {
+                             int M, int C, int R, const q4::DropArgs& drop, hipStream_t stream) {
     switch ((R + 3) / 4) {
-        case 1: launch_down_kernel<1, WL, F32, 1>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
-        case 2: launch_down_kernel<1, WL, F32, 2>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
-        case 3: launch_down_kernel<1, WL, F32, 3>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
-        default: launch_down_kernel<1, WL, F32, 4>(ip, w, w_sr, w_sc, op, M, C, R, stream); break;
+        case 1: launch_down_kernel<1, WL, F32, 1>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream); break;
+        case 2: launch_down_kernel<1, WL, F32, 2>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream); break;
+        case 3: launch_down_kernel<1, WL, F32, 3>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream); break;
+        default: launch_down_kernel<1, WL, F32, 4>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream); break;
     }
 }
 
 extern "C" int q4_launch_lora_down(const void* in, const void* w, int w_sr, int w_sc, int w_is_f32, void* out,
-                                   int M, int C, int R, hipStream_t stream) {
+                                   int M, int C, int R, const q4::DropArgs* dropp, hipStream_t stream) {
     using namespace q4;
+    const DropArgs drop = dropp ? *dropp : DropArgs{0u, 0u, 0u, 1.0f};
     const half_t* ip = reinterpret_cast<const half_t*>(in);
     half_t* op = reinterpret_cast<half_t*>(out);
     const bool base16 = (reinterpret_cast<uintptr_t>(w) & 15u) == 0;
     const int vec = w_is_f32 ? 4 : 8;                       // elements per 16 bytes
     if (w_sc == 1 && base16 && w_sr % 4 == 0 && R <= 16) {
-        if (w_is_f32) launch_down_staged<kRowsT, true>(ip, w, w_sr, w_sc, op, M, C, R, stream);
-        else launch_down_staged<kRowsT, false>(ip, w, w_sr, w_sc, op, M, C, R, stream);
+        if (w_is_f32) launch_down_staged<kRowsT, true>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream);
+        else launch_down_staged<kRowsT, false>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream);
     } else if (w_sc == 1 && base16 && w_sr % vec == 0) {
-        if (w_is_f32) launch_down_rb<kRows, true>(ip, w, w_sr, w_sc, op, M, C, R, stream);
-        else launch_down_rb<kRows, false>(ip, w, w_sr, w_sc, op, M, C, R, stream);
+        if (w_is_f32) launch_down_rb<kRows, true>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream);
+        else launch_down_rb<kRows, false>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream);
     } else if (w_sr == 1 && base16 && w_sc % 4 == 0 && R % 4 == 0 && R <= 16 && w_sc >= R) {
-        if (w_is_f32) launch_down_staged<kCols, true>(ip, w, w_sr, w_sc, op, M, C, R, stream);
-        else launch_down_staged<kCols, false>(ip, w, w_sr, w_sc, op, M, C, R, stream);
+        if (w_is_f32) launch_down_staged<kCols, true>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream);
+        else launch_down_staged<kCols, false>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream);
     } else {
-        if (w_is_f32) launch_down_rb<kAny, true>(ip, w, w_sr, w_sc, op, M, C, R, stream);
-        else launch_down_rb<kAny, false>(ip, w, w_sr, w_sc, op, M, C, R, stream);
+        if (w_is_f32) launch_down_rb<kAny, true>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream);
+        else launch_down_rb<kAny, false>(ip, w, w_sr, w_sc, op, M, C, R, drop, stream);
     }
     return hipGetLastError() == hipSuccess ? 0 : -4;
 }
@@ -475,7 +514,7 @@ extern "C" size_t q4_lora_grad_workspace(int M, int C, int R) {
 }
 
 static q4::GradProb make_grad_prob(const void* P, const void* in, float* out, int o_sr, int o_sc, int M, int C, int R,
-                                   float* part) {
+                                   float* part, const q4::DropArgs* drop = nullptr) {
     const q4::GradPlan g = q4::plan_grad(M, C, R);
     q4::GradProb q;
     q.P = reinterpret_cast<const q4::half_t*>(P);
@@ -484,6 +523,7 @@ static q4::GradProb make_grad_prob(const void* P, const void* in, float* out, in
     q.part = part;
     q.o_sr = o_sr; q.o_sc = o_sc; q.C = C;
     q.col_blocks = g.col_blocks; q.splits = g.splits; q.rows_per_wg = g.rows_per_wg;
+    q.drop = drop ? *drop : q4::DropArgs{0u, 0u, 0u, 1.0f};
     return q;
 }
 
@@ -510,23 +550,30 @@ static int launch_grad(const q4::GradArgs& ga, int nprob, int R, hipStream_t str
 }
 
 extern "C" int q4_launch_lora_grad(const void* P, const void* in, float* out, int o_sr, int o_sc, float alpha,
-                                   int M, int C, int R, void* workspace, hipStream_t stream) {
+                                   int M, int C, int R, const q4::DropArgs* drop, void* workspace, hipStream_t stream) {
     q4::GradArgs ga;
-    ga.p[0] = make_grad_prob(P, in, out, o_sr, o_sc, M, C, R, reinterpret_cast<float*>(workspace));
+    ga.p[0] = make_grad_prob(P, in, out, o_sr, o_sc, M, C, R, reinterpret_cast<float*>(workspace), drop);
     ga.p[1] = ga.p[0];
     ga.alpha = alpha;
     ga.M = M;
     return launch_grad(ga, 1, R, stream);
 }
 
+extern "C" int q4_launch_dropout_keep(uint8_t* keep, int M, int C, const q4::DropArgs* drop, hipStream_t stream) {
+    const long pairs = (long)M * (C / 2);
+    hipLaunchKernelGGL(q4::dropout_keep_kernel, dim3((unsigned)((pairs + 255) / 256)), dim3(256), 0, stream, keep, M, C, *drop);
+    return hipGetLastError() == hipSuccess ? 0 : -4;
+}
+
 // Two gradients with the same M, R and alpha in one launch (plus one launch for both reductions); the workspace
 // holds the partial tiles of the first problem followed by those of the second.
 extern "C" int q4_launch_lora_grad_pair(const void* P1, const void* in1, float* out1, int o1_sr, int o1_sc, int C1,
                                         const void* P2, const void* in2, float* out2, int o2_sr, int o2_sc, int C2,
-                                        float alpha, int M, int R, void* workspace, hipStream_t stream) {
+                                        float alpha, int M, int R, const q4::DropArgs* drop1, void* workspace,
+                                        hipStream_t stream) {
     q4::GradArgs ga;
     float* ws = reinterpret_cast<float*>(workspace);
-    ga.p[0] = make_grad_prob(P1, in1, out1, o1_sr, o1_sc, M, C1, R, ws);
+    ga.p[0] = make_grad_prob(P1, in1, out1, o1_sr, o1_sc, M, C1, R, ws, drop1);      // the mask applies to in1 only
     ga.p[1] = make_grad_prob(P2, in2, out2, o2_sr, o2_sc, M, C2, R,
                              ws ? ws + q4_lora_grad_workspace(M, C1, R) / sizeof(float) : nullptr);
     ga.alpha = alpha;

@@ -122,9 +122,8 @@ class Linear4bitLt(Autograd4bitQuantLinear, LoraLayer):
         r = self.lora_A[name].weight.shape[0]
         if r % 8 != 0 or not (8 <= r <= 64):
             return None
-        drop = self.lora_dropout[name]
-        if isinstance(drop, nn.Dropout) and drop.p > 0.0 and self.training:
-            return None
+        if self._dropout_p(name) >= 1.0 or (self._dropout_p(name) > 0.0 and torch.cuda.is_current_stream_capturing()):
+            return None                                   # the mask's seed is a launch argument: a replayed graph would repeat it
         rows = x.numel() // x.shape[-1]
         if rows <= autograd_4bit.quant_hip.MAX_GEMV_ROWS:
             return None
@@ -133,6 +132,13 @@ class Linear4bitLt(Autograd4bitQuantLinear, LoraLayer):
         if not (torch.is_autocast_enabled('cuda') or x.dtype == torch.float16):
             return None
         return name
+
+    def _dropout_p(self, name):
+        """Probability of the adapter's dropout as it applies to this call (0 in eval mode / without dropout)."""
+        drop = self.lora_dropout[name]
+        if isinstance(drop, nn.Dropout) and drop.p > 0.0 and self.training:
+            return float(drop.p)
+        return 0.0
 
     def _decode_adapter(self, x):
         """Name of the single adapter for the short no-grad path (a handful of rows, eval mode), else None."""
@@ -180,9 +186,15 @@ class Linear4bitLt(Autograd4bitQuantLinear, LoraLayer):
                 bias = None
                 if not self.disable_bias and not autograd_4bit._is_all_zero(self.bias):
                     bias = self.bias if self.bias.dtype == torch.float16 else self.bias.half()
+                # dropout(x) in front of lora_A (models.py:63-66) stays inside the fused kernels: a counter-based mask
+                # keyed by a seed drawn here from torch's CPU generator (so torch.manual_seed and the RNG state
+                # that checkpointing restores for its recomputation reproduce it)
+                drop_p = self._dropout_p(name)
+                drop_seed = int(torch.randint(0, 2 ** 62, (1,)).item()) if drop_p > 0.0 else 0
                 return autograd_4bit.AutogradMatmul4bitLora.apply(
                     x, self.qweight, self.scales, self.qzeros, self.g_idx, bias,
-                    self.lora_A[name].weight, self.lora_B[name].weight, float(self.scaling[name]), self.groupsize)
+                    self.lora_A[name].weight, self.lora_B[name].weight, float(self.scaling[name]), self.groupsize,
+                    drop_p, drop_seed)
 
         # reference composition (models.py:51-69)
         result = super().forward(x)

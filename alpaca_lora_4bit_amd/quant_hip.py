@@ -14,6 +14,8 @@ Nothing here computes on the CPU: without the built library the import fails.
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from . import _lib
@@ -495,9 +497,53 @@ def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, 
     return out
 
 
+def _drop_arg(dropout):
+    """(seed, p) -> ctypes descriptor (kept alive by the caller for the duration of the call), or None."""
+    if dropout is None:
+        return None
+    seed, p = dropout
+    p = float(p)
+    _require(0.0 <= p < 1.0, "dropout probability must be in [0, 1)")
+    if p == 0.0:
+        return None
+    seed = int(seed)
+    return _lib.Dropout(seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF, p)
+
+
+def _drop_ref(d):
+    return None if d is None else ctypes.byref(d)
+
+
+def dropout_scale(p):
+    """What the kernels multiply the surviving elements by: 1 / (1 - round(p * 32768) / 32768)."""
+    return float(_lib.lib().q4_dropout_scale(float(p)))
+
+
+def dropout_keep_mask(M, C, seed, p, device="cuda"):
+    """uint8 [M, C]: 1 where the counter-based dropout of (seed, p) keeps element (m, c), the mask that lora_down,
+    lora_grad and gemm_bwd_dx regenerate internally when given dropout=(seed, p)."""
+    dev = torch.device(device)
+    keep = torch.empty((M, C), dtype=torch.uint8, device=dev)
+    seed = int(seed)
+    d = _lib.Dropout(seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF, float(p))
+    with _device_ctx(dev):
+        rc = _lib.lib().q4_dropout_keep_u8(keep.data_ptr(), M, C, ctypes.byref(d), _stream(dev))
+    _lib.check(rc, "q4_dropout_keep_u8")
+    return keep
+
+
+def masked_adapter_term(dyb, lora_a, lora_scale, dropout):
+    """fp16 [M, K]: mask/(1-p) * lora_scale * dyb @ lora_a under the counter-based mask of dropout=(seed, p):
+    the adapter's share of grad_input for the routes that do not run the fused backward kernel."""
+    M, K = dyb.shape[0], lora_a.shape[1]
+    term = torch.mm(dyb * (float(lora_scale) * dropout_scale(dropout[1])), lora_a.to(torch.float16))
+    return term.mul_(dropout_keep_mask(M, K, dropout[0], dropout[1], dyb.device))
+
+
 def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=None, lora_a=None, lora_scale=1.0,
-                out_shape=None):
-    """dx fp16 [M, K] = dy [M, N] @ W^T (+ lora_scale * dyb @ lora_a); lora_a is an [R, K] view."""
+                out_shape=None, dropout=None):
+    """dx fp16 [M, K] = dy [M, N] @ W^T (+ lora_scale * dyb @ lora_a); lora_a is an [R, K] view.
+    dropout=(seed, p): the adapter term is masked like dropout(x) (gradient of lora_B(lora_A(dropout(x))))."""
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     dy2 = _flat_half(dy, N, dev, "grad_output")
     M = dy2.shape[0]
@@ -507,6 +553,11 @@ def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=Non
     if plan is not None:
         # dx comes out in sorted row order and is scattered back; the adapter matrix [R, K] is gathered too
         perm, inv, qs, gs_sorted = plan
+        if dropout is not None and dyb is not None:
+            # the mask is indexed by the ORIGINAL column: add the masked adapter term after the scatter
+            dx_sorted = gemm_bwd_dx(dy2, qs, qzeros, scales, None, gs_sorted)
+            dx = dx_sorted.index_select(1, inv)
+            return dx.add_(masked_adapter_term(dyb, lora_a, lora_scale, dropout)).reshape(_out_shape(out_shape, M, K))
         la_sorted = None if lora_a is None else lora_a.index_select(1, perm)
         dx_sorted = gemm_bwd_dx(dy2, qs, qzeros, scales, None, gs_sorted, dyb=dyb, lora_a=la_sorted, lora_scale=lora_scale)
         return dx_sorted.index_select(1, inv).reshape(_out_shape(out_shape, M, K))
@@ -514,11 +565,12 @@ def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=Non
     gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
     out = torch.empty(_out_shape(out_shape, M, K), dtype=torch.float16, device=dev)
     L = _lib.lib()
+    drop = _drop_arg(dropout)
     with _device_ctx(dev):
         wp, wn = _gemm_scratch(L, dev, 0, M, K, N)
         rc = L.q4_gemm_bwd_dx_f16(dy2.data_ptr(), qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
                                   gp, gs, _ptr(dyb), _ptr(lora_a), sr, sc, f32, float(lora_scale), R,
-                                  out.data_ptr(), M, K, N, G, wp, wn, _stream(dev))
+                                  out.data_ptr(), M, K, N, G, _drop_ref(drop), wp, wn, _stream(dev))
     _lib.check(rc, "q4_gemm_bwd_dx_f16")
     return out
 
@@ -526,9 +578,10 @@ def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=Non
 LORA_GRAD_RANKS = (8, 16)
 
 
-def lora_down(inp, w):
+def lora_down(inp, w, dropout=None):
     """out fp16 [M, R] = inp fp16 [M, C] @ w^T for an adapter matrix view w [R, C] (fp16/fp32, any positive
-    strides): xa = x @ A^T with w = lora_A.weight, dyb = dy @ B with w = lora_B.weight.t()  (models.py:66)."""
+    strides): xa = x @ A^T with w = lora_A.weight, dyb = dy @ B with w = lora_B.weight.t()  (models.py:66).
+    dropout=(seed, p): out = dropout(inp) @ w^T with the counter-based mask of (seed, p)."""
     _require(inp.is_cuda and inp.dtype == torch.float16 and inp.dim() == 2 and inp.is_contiguous(),
              "inp must be a contiguous float16 [M, C] CUDA tensor")
     M, C = inp.shape
@@ -541,16 +594,18 @@ def lora_down(inp, w):
     sr, sc = w.stride()
     _require(sr >= 1 and sc >= 1, "w must have positive strides")
     out = torch.empty((M, R), dtype=torch.float16, device=inp.device)
+    drop = _drop_arg(dropout)
     with _device_ctx(inp.device):
         rc = _lib.lib().q4_lora_down_f16(inp.data_ptr(), w.data_ptr(), int(sr), int(sc), f32, out.data_ptr(),
-                                         M, C, R, _stream(inp.device))
+                                         M, C, R, _drop_ref(drop), _stream(inp.device))
     _lib.check(rc, "q4_lora_down_f16")
     return out
 
 
-def lora_grad(p, inp, alpha, transposed=False):
+def lora_grad(p, inp, alpha, transposed=False, dropout=None):
     """alpha * p^T @ inp in fp32 for p fp16 [M, R], inp fp16 [M, C], R in LORA_GRAD_RANKS.  Returns [R, C], or
-    with transposed=True the same values stored as a contiguous [C, R] tensor (lora_B.weight's layout)."""
+    with transposed=True the same values stored as a contiguous [C, R] tensor (lora_B.weight's layout).
+    dropout=(seed, p): inp is replaced by dropout(inp)."""
     _require(p.is_cuda and p.dtype == torch.float16 and p.dim() == 2 and p.is_contiguous(),
              "p must be a contiguous float16 [M, R] CUDA tensor")
     _require(inp.dtype == torch.float16 and inp.dim() == 2 and inp.is_contiguous() and inp.device == p.device
@@ -569,18 +624,20 @@ def lora_grad(p, inp, alpha, transposed=False):
         sr, sc = C, 1
     L = _lib.lib()
     nbytes = L.q4_lora_grad_workspace_bytes(M, C, R)
+    drop = _drop_arg(dropout)
     with _device_ctx(dev):
         ws = _scratch(dev, nbytes)
         rc = L.q4_lora_grad_f32(p.data_ptr(), inp.data_ptr(), out.data_ptr(), sr, sc, float(alpha), M, C, R,
-                                ws.data_ptr(), ws.numel(), _stream(dev))
+                                _drop_ref(drop), ws.data_ptr(), ws.numel(), _stream(dev))
     _lib.check(rc, "q4_lora_grad_f32")
     return out
 
 
-def lora_grad_pair(p1, inp1, p2, inp2, alpha):
+def lora_grad_pair(p1, inp1, p2, inp2, alpha, dropout=None):
     """Both adapter gradients of a layer in one launch: returns (alpha * p1^T @ inp1 as [R, C1],
     alpha * p2^T @ inp2 stored as a contiguous [C2, R] tensor) -- dA from (dyb, x) and dB in lora_B.weight's
-    layout from (xa, dy).  Same requirements as lora_grad; p1 and p2 share their shape."""
+    layout from (xa, dy).  Same requirements as lora_grad; p1 and p2 share their shape.
+    dropout=(seed, p): inp1 is replaced by dropout(inp1) (inp2 is left as it is)."""
     for p, inp in ((p1, inp1), (p2, inp2)):
         _require(p.is_cuda and p.dtype == torch.float16 and p.dim() == 2 and p.is_contiguous(),
                  "p must be a contiguous float16 [M, R] CUDA tensor")
@@ -597,11 +654,12 @@ def lora_grad_pair(p1, inp1, p2, inp2, alpha):
     out2 = torch.empty((C2, R), dtype=torch.float32, device=dev)
     L = _lib.lib()
     nbytes = L.q4_lora_grad_workspace_bytes(M, C1, R) + L.q4_lora_grad_workspace_bytes(M, C2, R)
+    drop = _drop_arg(dropout)
     with _device_ctx(dev):
         ws = _scratch(dev, nbytes)
         rc = L.q4_lora_grad_pair_f32(p1.data_ptr(), inp1.data_ptr(), out1.data_ptr(), C1, 1, C1,
                                      p2.data_ptr(), inp2.data_ptr(), out2.data_ptr(), 1, R, C2,
-                                     float(alpha), M, R, ws.data_ptr(), ws.numel(), _stream(dev))
+                                     float(alpha), M, R, _drop_ref(drop), ws.data_ptr(), ws.numel(), _stream(dev))
     _lib.check(rc, "q4_lora_grad_pair_f32")
     return out1, out2
 

@@ -185,19 +185,21 @@ def bench_dequant(K, N, act_order, reps, copies=6, seed=9):
     return dict(us=per * 1e6, gbs=b / per / 1e9, frac_hbm=b / per / 1e9 / HBM_PEAK_GBS, bytes=b, copies=copies)
 
 
-def bench_lora_step(reps, seed=5):
+def bench_lora_step(reps, seed=5, dropout=0.0):
     """Config 2: Linear4bitLt 4096->4096, r=8, alpha=16, 2048 tokens: forward + backward
-    (dx, dA, dB).  138.24 GFLOP of algorithmic work per step."""
+    (dx, dA, dB).  138.24 GFLOP of algorithmic work per step.  dropout > 0: the layer in training mode with that
+    adapter dropout (the mask's seed is a launch argument, so that variant is timed eagerly only)."""
     import torch
     from alpaca_lora_4bit_amd import models
     gen = torch.Generator(device="cuda").manual_seed(seed)
     K = N = 4096
     M, r = 2048, 8
     lay = make_layer_gpu(K, N, 128, gen)
-    m = models.Linear4bitLt("default", K, N, 128, False, r=r, lora_alpha=16).cuda()
+    m = models.Linear4bitLt("default", K, N, 128, False, r=r, lora_alpha=16, lora_dropout=dropout).cuda()
     m.qweight, m.qzeros, m.scales = lay["qweight"], lay["qzeros"], lay["scales"]
     m.g_idx = (torch.arange(K, device="cuda") // 128).to(torch.int32)
     m.bias = torch.zeros(N, dtype=torch.float16, device="cuda")
+    m.train(dropout > 0)
     with torch.no_grad():
         m.lora_B["default"].weight.normal_(0, 0.02, generator=gen)
     x = torch.randn((8, 256, K), device="cuda", generator=gen).half().requires_grad_(True)
@@ -223,6 +225,10 @@ def bench_lora_step(reps, seed=5):
     e1.record()
     torch.cuda.synchronize()
     eager = e0.elapsed_time(e1) * 1e-3 / reps
+    flop = 2 * 2 * M * K * N + (2 * M * K * r + 2 * M * r * N) + 2 * (2 * M * K * r + 2 * M * r * N)
+    if dropout > 0:
+        return dict(eager_ms=eager * 1e3, eager_tokens_per_s=M / eager, eager_tflops=flop / eager / 1e12,
+                    eager_frac_mfma=flop / eager / 1e12 / MFMA_FP16_PEAK_TFLOPS, dropout=dropout)
 
     # the same forward + backward captured once as a HIP graph and replayed (no Python between kernels)
     s = torch.cuda.Stream()
@@ -244,7 +250,6 @@ def bench_lora_step(reps, seed=5):
         e1.record(s)
         torch.cuda.synchronize()
     per = e0.elapsed_time(e1) * 1e-3 / reps
-    flop = 2 * 2 * M * K * N + (2 * M * K * r + 2 * M * r * N) + 2 * (2 * M * K * r + 2 * M * r * N)
     return dict(ms=per * 1e3, tokens_per_s=M / per, tflops=flop / per / 1e12,
                 frac_mfma=flop / per / 1e12 / MFMA_FP16_PEAK_TFLOPS, gflop_per_step=flop / 1e9,
                 eager_ms=eager * 1e3, eager_tokens_per_s=M / eager)
@@ -500,7 +505,9 @@ def main():
         return
     if args.lora_step_only:
         r = bench_lora_step(max(args.steps, 5))
-        print(json.dumps({"workload": "config2_lora_fwd_bwd_M2048", **{k: round(v, 4) for k, v in r.items()}}))
+        rd = bench_lora_step(max(args.steps, 5), dropout=0.05)
+        print(json.dumps({"workload": "config2_lora_fwd_bwd_M2048", **{k: round(v, 4) for k, v in r.items()},
+                          "with_dropout_0.05": {k: round(v, 4) for k, v in rd.items()}}))
         return
     if args.calibrate_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
@@ -571,6 +578,8 @@ def main():
             extra[name] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in dq.items()}
         lo = bench_lora_step(20)
         extra["config2_lora_fwd_bwd_M2048"] = {k: round(v, 4) for k, v in lo.items()}
+        lod = bench_lora_step(20, dropout=0.05)          # the reference's default --lora_dropout, fused path
+        extra["config2_lora_fwd_bwd_M2048_dropout0.05"] = {k: round(v, 4) for k, v in lod.items()}
         gm = bench_gemm_only(2048, 4096, 4096, False, 20)
         extra["config2_gemm_kernels"] = {k: {kk: round(vv, 4) for kk, vv in v.items()} for k, v in gm.items()}
         g3 = bench_gemm_only(512, 5120, 13824, True, 10)

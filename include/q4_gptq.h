@@ -143,6 +143,22 @@ int q4_gemv_v1_f16(const void *x, const int32_t *qweight, const void *scales, co
                    int accumulate, int M, int K, int N,
                    void *workspace, size_t workspace_bytes, void *stream);
 
+/* Dropout on the adapter input (the reference applies nn.Dropout to x in front of lora_A, models.py:63-66, default
+ * p = 0.05, arg_parser.py:48).  The mask is never stored: element (m, c) of the [M, C] adapter input is dropped iff
+ * a 15-bit draw that is a pure function of (seed_lo, seed_hi, m, c) is below round(p * 32768); what survives is
+ * multiplied by q4_dropout_scale(p) = 32768 / (32768 - round(p * 32768)).  Every entry point below that takes a
+ * `const q4_dropout_t *drop` (HOST pointer, read during the call; NULL or p == 0: no dropout) regenerates the same
+ * mask from the same descriptor, so forward and backward agree as long as the caller passes the same seed.
+ *   draw(m, c): w = ((m * 0x9E3779B1 + seed_lo) ^ ((c >> 1) * 0x85EBCA6B + seed_hi));  w ^= w >> 16;  w *= 0x7FEB352D;
+ *               w ^= w >> 15;  w *= 0x846CA68B;  w ^= w >> 16   (32-bit unsigned);   draw = (w >> 16 * (c & 1)) & 0x7FFF.
+ * 0 <= p < 1.  q4_dropout_keep_u8 writes the mask itself (1 = kept) for callers that want to see it; C even. */
+typedef struct q4_dropout {
+    uint32_t seed_lo, seed_hi;
+    float p;
+} q4_dropout_t;
+float q4_dropout_scale(float p);
+int q4_dropout_keep_u8(uint8_t *keep, int M, int C, const q4_dropout_t *drop, void *stream);
+
 /* Forward GEMM, any M >= 1:
  *   y fp16 [M, N] = x fp16 [M, K] @ W  (+ bias fp16 [N])  (+ lora_scale * xa fp16 [M, R] @ Bm [R, N])
  * with fp32 accumulation on MFMA; W tiles are dequantized in LDS and never written to HBM.
@@ -171,19 +187,22 @@ int q4_gemm_fwd_f16(const void *x, const int32_t *qweight, const int32_t *qzeros
  * Replaces vecquant4recons_v2 + torch.matmul(grad_output, buffer.T)
  * (matmul_utils_4bit.py:114-126 with transpose=True, called from autograd_4bit.py:53) and the
  * adapter's contribution to grad_input, with dyb = dy @ B and Am[r, k] = lora_a[r*lda_r + k*lda_k]
- * (lora_A.weight [R, K]: lda_r = K, lda_k = 1). */
+ * (lora_A.weight [R, K]: lda_r = K, lda_k = 1).
+ * With `drop` the adapter term of dx[m, k] is kept (and scaled) only where the dropout mask keeps x[m, k]: the
+ * gradient of lora_B(lora_A(dropout(x))) with respect to x. */
 int q4_gemm_bwd_dx_f16(const void *dy, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                        const int32_t *g_idx, int groupsize,
                        const void *dyb, const void *lora_a, int lda_r, int lda_k, int lora_is_f32, float lora_scale,
-                       int R, void *dx, int M, int K, int N, int G,
+                       int R, void *dx, int M, int K, int N, int G, const q4_dropout_t *drop,
                        void *workspace, size_t workspace_bytes, void *stream);
 
 /* Rank-R down projection of the adapter:  out fp16 [M, R] = in fp16 [M, C] @ Wm^T,
  * Wm[j, c] = w[j*w_sr + c*w_sc] (fp16, or fp32 when w_is_f32 != 0).  xa = x @ A^T (w = lora_A.weight,
  * w_sr = K, w_sc = 1) and dyb = dy @ B (w = lora_B.weight, w_sr = 1, w_sc = R): the two products that
- * lora_A(x) and the backward of lora_B perform in the reference (models.py:66).  C % 32 == 0, 1 <= R <= 64. */
+ * lora_A(x) and the backward of lora_B perform in the reference (models.py:66).  C % 32 == 0, 1 <= R <= 64.
+ * With `drop`: out = dropout(in) @ Wm^T, i.e. lora_A(dropout(x)). */
 int q4_lora_down_f16(const void *in, const void *w, int w_sr, int w_sc, int w_is_f32, void *out,
-                     int M, int C, int R, void *stream);
+                     int M, int C, int R, const q4_dropout_t *drop, void *stream);
 
 /* Gradient of an adapter matrix:  out fp32 [j*o_sr + c*o_sc] = alpha * sum_m p[m, j] * in[m, c]
  * with p fp16 [M, R] and in fp16 [M, C]:  dA = scaling * dyb^T @ x (out = [R, K], o_sr = K, o_sc = 1) and
@@ -191,19 +210,23 @@ int q4_lora_down_f16(const void *in, const void *w, int w_sr, int w_sc, int w_is
  * computes for the two adapter Linears of models.py:66.  R is 8 or 16, C % 8 == 0.
  * `workspace`: q4_lora_grad_workspace_bytes(M, C, R) bytes (0 for small M: then it may be NULL), 256-byte
  * aligned, contents irrelevant before and after the call: it carries fp32 partial sums of row blocks,
- * which a second kernel adds in a fixed order (bit-reproducible). */
+ * which a second kernel adds in a fixed order (bit-reproducible).  With `drop`, `in` is replaced by dropout(in)
+ * (dA of lora_A(dropout(x))). */
 size_t q4_lora_grad_workspace_bytes(int M, int C, int R);
 int q4_lora_grad_f32(const void *p, const void *in, float *out, int o_sr, int o_sc, float alpha,
-                     int M, int C, int R, void *workspace, size_t workspace_bytes, void *stream);
+                     int M, int C, int R, const q4_dropout_t *drop,
+                     void *workspace, size_t workspace_bytes, void *stream);
 
 /* Both adapter gradients of a layer in one launch (plus one for the two reductions): problem 1 and problem 2 as
  * for q4_lora_grad_f32, sharing M, R and alpha -- dA from (dyb, x, C1 = K) and dB from (xa, dy, C2 = N) in the
  * backward of models.py:66.  A single gradient is bound by the latency of its one burst of loads, so the pair
  * costs little more than one.  `workspace`: q4_lora_grad_workspace_bytes(M, C1, R) +
- * q4_lora_grad_workspace_bytes(M, C2, R) bytes, 256-byte aligned, contents irrelevant. */
+ * q4_lora_grad_workspace_bytes(M, C2, R) bytes, 256-byte aligned, contents irrelevant.  `drop1` applies to in1 only
+ * (x in dA; xa in dB already carries the mask). */
 int q4_lora_grad_pair_f32(const void *p1, const void *in1, float *out1, int o1_sr, int o1_sc, int C1,
                           const void *p2, const void *in2, float *out2, int o2_sr, int o2_sc, int C2,
-                          float alpha, int M, int R, void *workspace, size_t workspace_bytes, void *stream);
+                          float alpha, int M, int R, const q4_dropout_t *drop1,
+                          void *workspace, size_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

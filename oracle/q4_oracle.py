@@ -219,25 +219,29 @@ def gemv_v2_fp32(x, qweight, qzeros, scales, g_idx) -> np.ndarray:
 
 
 # --------------------------------------------------------------------------- LoRA
-def lora_forward(x, W, A, B, scaling, bias=None) -> np.ndarray:
-    """Linear4bitLt.forward (models.py:51-69) for one active adapter, dropout off:
-    result = x @ W (+ bias, autograd_4bit.py:206-207) + lora_B(lora_A(x)) * scaling,
+def lora_forward(x, W, A, B, scaling, bias=None, keep=None, drop_scale=1.0) -> np.ndarray:
+    """Linear4bitLt.forward (models.py:51-69) for one active adapter:
+    result = x @ W (+ bias, autograd_4bit.py:206-207) + lora_B(lora_A(dropout(x))) * scaling,
     with lora_A.weight = A [r, K], lora_B.weight = B [N, r].  float64 throughout.
+    `keep` [M, K] (0/1) and `drop_scale` = 1/(1-p) describe the dropout of models.py:63-66 as torch's nn.Dropout
+    applies it in training mode: dropout(x) = x * keep * drop_scale; keep=None is dropout off / eval mode.
     """
     x = np.asarray(x, dtype=np.float64)
     y = x @ np.asarray(W, dtype=np.float64)
     if bias is not None:
         y = y + np.asarray(bias, dtype=np.float64)
-    xa = x @ np.asarray(A, dtype=np.float64).T
+    xd = x if keep is None else x * np.asarray(keep, dtype=np.float64) * float(drop_scale)
+    xa = xd @ np.asarray(A, dtype=np.float64).T
     return y + (xa @ np.asarray(B, dtype=np.float64).T) * float(scaling)
 
 
-def lora_backward(x, dy, W, A, B, scaling):
+def lora_backward(x, dy, W, A, B, scaling, keep=None, drop_scale=1.0):
     """Gradients of lora_forward w.r.t. x, A, B (closed form of what torch autograd
-    computes over autograd_4bit.py:45-54 plus models.py:66).  float64.
-      dx = dy @ W.T + scaling * (dy @ B) @ A
-      dA = scaling * (dy @ B).T @ x          [r, K]
-      dB = scaling * dy.T @ (x @ A.T)        [N, r]
+    computes over autograd_4bit.py:45-54 plus models.py:66).  float64.  With xd = x * keep * drop_scale
+    (dropout in front of lora_A; keep=None: xd = x, mask = 1):
+      dx = dy @ W.T + keep * drop_scale * (scaling * (dy @ B) @ A)
+      dA = scaling * (dy @ B).T @ xd         [r, K]
+      dB = scaling * dy.T @ (xd @ A.T)       [N, r]
     """
     x = np.asarray(x, dtype=np.float64)
     dy = np.asarray(dy, dtype=np.float64)
@@ -245,11 +249,35 @@ def lora_backward(x, dy, W, A, B, scaling):
     A = np.asarray(A, dtype=np.float64)
     B = np.asarray(B, dtype=np.float64)
     s = float(scaling)
+    m = 1.0 if keep is None else np.asarray(keep, dtype=np.float64) * float(drop_scale)
+    xd = x * m
     dyB = dy @ B
-    dx = dy @ W.T + s * (dyB @ A)
-    dA = s * (dyB.T @ x)
-    dB = s * (dy.T @ (x @ A.T))
+    dx = dy @ W.T + m * (s * (dyB @ A))
+    dA = s * (dyB.T @ xd)
+    dB = s * (dy.T @ (xd @ A.T))
     return dx, dA, dB
+
+
+def dropout_keep_counter(M, C, seed, p):
+    """(keep uint8 [M, C], scale): the counter-based dropout mask the library documents in include/q4_gptq.h
+    (no reference counterpart: the reference's mask comes from torch's generator, models.py:63 -- any mask with
+    the right statistics is a valid nn.Dropout).  Restated here from the header's formula with numpy uint32
+    arithmetic: element (m, c) is kept iff its 15-bit draw >= round(p * 32768)."""
+    thr = min(int(np.float32(p) * np.float32(32768.0) + np.float32(0.5)), 32767)
+    seed_lo, seed_hi = np.uint32(seed & 0xFFFFFFFF), np.uint32((seed >> 32) & 0xFFFFFFFF)
+    with np.errstate(over="ignore"):
+        rows = np.arange(M, dtype=np.uint32)[:, None]
+        pairs = np.arange(C // 2, dtype=np.uint32)[None, :]
+        w = (rows * np.uint32(0x9E3779B1) + seed_lo) ^ (pairs * np.uint32(0x85EBCA6B) + seed_hi)
+        w ^= w >> np.uint32(16)
+        w = w * np.uint32(0x7FEB352D)
+        w ^= w >> np.uint32(15)
+        w = w * np.uint32(0x846CA68B)
+        w ^= w >> np.uint32(16)
+    keep = np.empty((M, C), dtype=np.uint8)
+    keep[:, 0::2] = (w & np.uint32(0x7FFF)) >= thr
+    keep[:, 1::2] = ((w >> np.uint32(16)) & np.uint32(0x7FFF)) >= thr
+    return keep, 32768.0 / (32768 - thr)
 
 
 # --------------------------------------------------------------------------- synthetic data

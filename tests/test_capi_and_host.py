@@ -60,7 +60,7 @@ def test_error_codes_and_validation_need_no_gpu():
     assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, None, 1, 8, 0, 1.0, 8, fake, 64, 256, 128, 2, None, 0, None) == -1
     assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, fake, 1, 12, 0, 1.0, 12, fake, 64, 256, 128, 2, None, 0, None) == -2
     assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, fake, fake, 0, 8, 1, 1.0, 8, fake, 64, 256, 128, 2, None, 0, None) == -2
-    assert L.q4_gemm_bwd_dx_f16(fake, fake, fake, fake, None, 32, None, None, 0, 0, 0, 1.0, 0, fake, 64, 256, 128, 8, None, 0, None) == -2
+    assert L.q4_gemm_bwd_dx_f16(fake, fake, fake, fake, None, 32, None, None, 0, 0, 0, 1.0, 0, fake, 64, 256, 128, 8, None, None, 0, None) == -2
     assert L.q4_gemm_fwd_f16(fake, fake, fake, fake, None, 128, None, None, None, 0, 0, 0, 1.0, 0, fake, 64, 256, 128, 2, ctypes.c_void_p(0x1010), 1 << 20, None) == -5
     assert L.q4_gemm_workspace_bytes(1, 2048, 4096, 4096) == 0            # enough tiles: no split
     assert L.q4_gemm_workspace_bytes(1, 64, 4096, 4096) == 8 * 64 * 4096 * 4    # 32 tiles -> 8 splits of fp32 partials
@@ -76,19 +76,19 @@ def test_error_codes_and_validation_need_no_gpu():
     assert L.q4_dequant2_f16(fake, fake, fake, None, 128, fake, 264, 128, 3, None) == -2     # K % 16
     assert L.q4_dequant2_f16(fake, fake, fake, None, 128, odd, 256, 128, 2, None) == -5
     # adapter helpers
-    assert L.q4_lora_down_f16(fake, None, 4096, 1, 1, fake, 64, 4096, 8, None) == -1
-    assert L.q4_lora_down_f16(fake, fake, 4096, 1, 1, fake, 64, 4100, 8, None) == -2        # C % 32
-    assert L.q4_lora_down_f16(fake, fake, 4096, 1, 1, fake, 64, 4096, 65, None) == -2       # R > 64
-    assert L.q4_lora_down_f16(fake, ctypes.c_void_p(0x1002), 4096, 1, 1, fake, 64, 4096, 8, None) == -5
+    assert L.q4_lora_down_f16(fake, None, 4096, 1, 1, fake, 64, 4096, 8, None, None) == -1
+    assert L.q4_lora_down_f16(fake, fake, 4096, 1, 1, fake, 64, 4100, 8, None, None) == -2        # C % 32
+    assert L.q4_lora_down_f16(fake, fake, 4096, 1, 1, fake, 64, 4096, 65, None, None) == -2       # R > 64
+    assert L.q4_lora_down_f16(fake, ctypes.c_void_p(0x1002), 4096, 1, 1, fake, 64, 4096, 8, None, None) == -5
     assert L.q4_lora_grad_workspace_bytes(64, 4096, 8) == 0            # one row block: no partial sums
     assert L.q4_lora_grad_workspace_bytes(2048, 4096, 8) == 32 * 8 * 64 * 64 * 4
     assert L.q4_lora_grad_workspace_bytes(2048, 4096, 12) == 0
-    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 64, 4096, 12, fake, 1 << 20, None) == -2   # R not 8/16
-    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 2048, 4096, 8, None, 0, None) == -3
-    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 2048, 4096, 8, fake, 1024, None) == -3
-    assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, None, 1, 8, 4096, 1.0, 2048, 8, fake, 1 << 24, None) == -1
-    assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, fake, 1, 8, 4100, 1.0, 2048, 8, fake, 1 << 24, None) == -2
-    assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, fake, 1, 8, 4096, 1.0, 2048, 8, fake, 1 << 22, None) == -3  # needs 2 x 4 MiB
+    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 64, 4096, 12, None, fake, 1 << 20, None) == -2   # R not 8/16
+    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 2048, 4096, 8, None, None, 0, None) == -3
+    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 2048, 4096, 8, None, fake, 1024, None) == -3
+    assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, None, 1, 8, 4096, 1.0, 2048, 8, None, fake, 1 << 24, None) == -1
+    assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, fake, 1, 8, 4100, 1.0, 2048, 8, None, fake, 1 << 24, None) == -2
+    assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, fake, 1, 8, 4096, 1.0, 2048, 8, None, fake, 1 << 22, None) == -3  # needs 2 x 4 MiB
     # allocation-free GEMV: validated like q4_gemv_f16, plus the size of the built-in accumulator array
     assert L.q4_gemv_noalloc_max_outputs() == 16 * 32768
     assert L.q4_gemv_noalloc_f16(fake, fake, fake, fake, None, 128, fake, 0, 16, 256, 32832, 2, None) == -6
@@ -111,6 +111,13 @@ def test_error_codes_and_validation_need_no_gpu():
     lay[1].N = 128
     lay[1].y = 0
     assert L.q4_gemv_grouped_f16(lay, 2, 128, 0, 1, 256, fake, 1 << 20, None) == -1
+    # dropout descriptor: p outside [0, 1) is rejected, the realized scale is 32768 / (32768 - round(p * 32768))
+    bad = _lib.Dropout(1, 2, 1.0)
+    assert L.q4_lora_down_f16(fake, fake, 4096, 1, 1, fake, 64, 4096, 8, ctypes.byref(bad), None) == -2
+    assert L.q4_dropout_keep_u8(fake, 4, 7, ctypes.byref(_lib.Dropout(1, 2, 0.5)), None) == -2       # C must be even
+    assert L.q4_dropout_keep_u8(None, 4, 8, ctypes.byref(_lib.Dropout(1, 2, 0.5)), None) == -1
+    assert abs(L.q4_dropout_scale(0.05) - 32768.0 / (32768 - 1638)) < 1e-6 and L.q4_dropout_scale(0.0) == 1.0
+    assert L.q4_dropout_scale(1.5) == 0.0
     assert L.q4_gemv_workspace_bytes(16, 4096, 11008) == 16 * 11008 * 8
     assert L.q4_gemv_workspace_bytes(0, 4096, 11008) == 0
 
