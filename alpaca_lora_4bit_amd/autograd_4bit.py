@@ -344,6 +344,8 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
         dyb = quant_hip.lora_down(dy, b.t())
         dropout = ctx.dropout
         dx = da = db = None
+        r = a.shape[0]
+        need_a, need_b = ctx.needs_input_grad[6], ctx.needs_input_grad[7]
         if ctx.needs_input_grad[0]:
             dx_shape = tuple(grad_output.shape[:-1]) + (qweight.shape[0] * 8,)
             if mm4b.use_dense_route(dy.shape[0]):
@@ -355,8 +357,6 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
             else:
                 dx = quant_hip.gemm_bwd_dx(dy, qweight, zeros, scales, g_idx, ctx.groupsize, dyb=dyb, lora_a=a,
                                            lora_scale=ctx.scaling, out_shape=dx_shape, dropout=dropout)
-        r = a.shape[0]
-        need_a, need_b = ctx.needs_input_grad[6], ctx.needs_input_grad[7]
         if need_a and need_b and r in quant_hip.LORA_GRAD_RANKS:
             da, db = quant_hip.lora_grad_pair(dyb, x2, xa, dy, ctx.scaling, dropout=dropout)   # one launch for both gradients
         else:

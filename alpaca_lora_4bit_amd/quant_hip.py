@@ -633,7 +633,7 @@ def lora_grad(p, inp, alpha, transposed=False, dropout=None):
     return out
 
 
-def lora_grad_pair(p1, inp1, p2, inp2, alpha, dropout=None):
+def lora_grad_pair(p1, inp1, p2, inp2, alpha, dropout=None, outs=None):
     """Both adapter gradients of a layer in one launch: returns (alpha * p1^T @ inp1 as [R, C1],
     alpha * p2^T @ inp2 stored as a contiguous [C2, R] tensor) -- dA from (dyb, x) and dB in lora_B.weight's
     layout from (xa, dy).  Same requirements as lora_grad; p1 and p2 share their shape.
@@ -650,8 +650,14 @@ def lora_grad_pair(p1, inp1, p2, inp2, alpha, dropout=None):
     dev = p1.device
     if M == 0:
         return (torch.zeros((R, C1), dtype=torch.float32, device=dev), torch.zeros((C2, R), dtype=torch.float32, device=dev))
-    out1 = torch.empty((R, C1), dtype=torch.float32, device=dev)
-    out2 = torch.empty((C2, R), dtype=torch.float32, device=dev)
+    if outs is None:
+        out1 = torch.empty((R, C1), dtype=torch.float32, device=dev)
+        out2 = torch.empty((C2, R), dtype=torch.float32, device=dev)
+    else:                                     # allocated by the caller (e.g. on another stream than the launch)
+        out1, out2 = outs
+        _require(out1.dtype == torch.float32 and tuple(out1.shape) == (R, C1) and out1.is_contiguous()
+                 and out2.dtype == torch.float32 and tuple(out2.shape) == (C2, R) and out2.is_contiguous()
+                 and out1.device == dev and out2.device == dev, "outs must be float32 [R, C1] and [C2, R] on the same device")
     L = _lib.lib()
     nbytes = L.q4_lora_grad_workspace_bytes(M, C1, R) + L.q4_lora_grad_workspace_bytes(M, C2, R)
     drop = _drop_arg(dropout)
