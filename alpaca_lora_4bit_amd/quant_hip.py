@@ -23,6 +23,17 @@ from ._lib import Q4Error  # noqa: F401  (re-exported)
 
 _lib.lib()  # fail at import time, loudly, if the HIP library is missing
 
+# Compiled host binding (csrc/host/q4_host.cpp, built by g++ next to the library): does the per-call checks, takes
+# torch's current stream, keeps the workspaces and calls the C ABI without going through ctypes.  The ctypes path
+# below stays as the fallback for a tree where only the library was built.
+try:
+    from . import _q4_host as _host
+    if _host.abi_version() != _lib.ABI_VERSION:
+        raise ImportError(f"_q4_host was built against ABI {_host.abi_version()}, the library has {_lib.ABI_VERSION}; rebuild")
+    _host.set_error_class(_lib.Q4Error)
+except ModuleNotFoundError:
+    _host = None
+
 MAX_GEMV_ROWS = 16
 MAX_GEMV_SORTED_ROWS = 3          # q4_gemv_sorted_f16 (x gathered inside the kernel) wins up to 3 rows, ties at 4
 _workspaces = {}
@@ -146,9 +157,9 @@ def scales_fit_fused_dequant(scales):
 def _gemm_gidx_arg(g_idx, groupsize, G, K, scales):
     """Like _gidx_arg for the GEMM kernels; layers with huge scales are routed to the
     per-row-group path, whose dequant has no range restriction."""
-    if scales_fit_fused_dequant(scales):
+    if scales_fit_fused_dequant(scales) and not (g_idx is None and int(groupsize) % 64 != 0):
         return _gidx_arg(g_idx, groupsize, G, need_multiple=64) + (g_idx,)
-    if g_idx is None:
+    if g_idx is None:            # sequential groups the tiled kernels do not take as such (group size not a multiple of 64)
         g_idx = (torch.arange(K, device=scales.device, dtype=torch.int32) // int(groupsize)).contiguous()
     return g_idx.data_ptr(), int(groupsize or 0), g_idx
 
@@ -188,6 +199,68 @@ def _actorder_plan(qweight, scales, g_idx, groupsize, G):
     return sorted_layer(qweight, g_idx, G)
 
 
+class _LayerInfo:
+    """What the content-dependent checks decided for one layer's tensors: how the GEMV and the GEMM kernels are to
+    be called (g_idx tensor or None for sequential groups, group size) and the sorted-rows plan of an act-order layer."""
+    __slots__ = ("dev", "K", "N", "G", "gemv_gidx", "gemv_gs", "gemm", "plan", "_src")
+
+    def gemm_args(self):
+        """(g_idx tensor or None, group size) for the tiled kernels; decided on the first product above 16 rows."""
+        if self.gemm is None:
+            g_idx, groupsize, scales = self._src
+            gp, gs, keep = _gemm_gidx_arg(g_idx, groupsize, self.G, self.K, scales)
+            self.gemm = (None if gp == 0 else keep, gs)
+        return self.gemm
+
+
+def _layer_info(qweight, qzeros, scales, g_idx, groupsize):
+    """_LayerInfo of these tensors.  Kept on the qweight tensor object and reused while the very same tensor objects
+    come back with unchanged in-place version counters: a handful of identity and integer comparisons per call.
+    (Writes through `.data` do not bump the counters: call `invalidate` after such a write.)"""
+    gver = -1 if g_idx is None else g_idx._version
+    c = getattr(qweight, "_q4_info", None)
+    if (c is not None and c[0] is qzeros and c[1] is scales and c[2] is g_idx and c[3] == groupsize
+            and c[4] == qweight._version and c[5] == qzeros._version and c[6] == scales._version and c[7] == gver
+            and c[8] == actorder_repack):
+        return c[9]
+    info = _LayerInfo()
+    info.dev, info.K, info.N, info.G = _check_layer_uncached(qweight, qzeros, scales, g_idx, groupsize)
+    info.plan = _actorder_plan(qweight, scales, g_idx, groupsize, info.G)
+    info._src = (g_idx, groupsize, scales)
+    info.gemm = None
+    if info.plan is not None:
+        info.gemv_gidx, info.gemv_gs = None, info.plan[3]
+        info.gemm = (None, info.plan[3])
+    else:
+        gp, gs = _gidx_arg(g_idx, groupsize, info.G)
+        info.gemv_gidx, info.gemv_gs = (None if gp == 0 else g_idx), gs
+    try:
+        qweight._q4_info = (qzeros, scales, g_idx, groupsize, qweight._version, qzeros._version, scales._version, gver,
+                            actorder_repack, info)
+    except AttributeError:          # tensor subclasses without a __dict__
+        pass
+    return info
+
+
+def invalidate(*tensors_or_modules):
+    """Forget what was cached about these tensors (or about every tensor of these modules): the layer verdicts,
+    the g_idx classification, the scale-range check and the sorted copy of an act-order layer.  Needed only after
+    writing packed tensors through `.data` (which does not bump the version counter the caches are keyed on)."""
+    for obj in tensors_or_modules:
+        items = [obj] if isinstance(obj, torch.Tensor) else [t for _, t in obj.named_buffers()] + list(obj.parameters())
+        for t in items:
+            for name in ("_q4_info", "_q4_layer", "_q4_kind", "_q4_small", "_q4_sorted", "_q4_zero"):
+                if hasattr(t, name):
+                    try:
+                        delattr(t, name)
+                    except AttributeError:
+                        pass
+
+
+def _shape_arg(out_shape):
+    return None if out_shape is None else [int(d) for d in out_shape]
+
+
 def _gidx_arg(g_idx, groupsize, G, need_multiple=32):
     """Returns (pointer-or-0, groupsize) to hand to the C ABI."""
     if g_idx is None:
@@ -206,6 +279,22 @@ def _workspace(device, nbytes):
         ws = torch.zeros(max(nbytes, 1 << 22), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
+
+
+def workspaces_are_zero():
+    """True when the GEMV's split-K accumulators cached for every (device, stream) are all zero, as every completed
+    call leaves them (synchronises; for tests and debugging).  `Q4_CHECK_WORKSPACE=1` in the environment makes the
+    compiled host binding check this on entry of every GEMV."""
+    ok = all(int(ws.view(torch.int32).abs().max()) == 0 for ws in _workspaces.values())
+    return ok and (_host is None or _host.workspaces_are_zero())
+
+
+def reset_workspaces():
+    """Zeroes the cached GEMV accumulators (after a run that was cut short inside a GEMV)."""
+    for ws in _workspaces.values():
+        ws.zero_()
+    if _host is not None:
+        _host.reset_workspaces()
 
 
 def _scratch(device, nbytes):
@@ -252,11 +341,13 @@ def _flat_half(x, K, dev, what):
 def dequant(qweight, qzeros, scales, g_idx=None, groupsize=None, out=None):
     """W fp16 [K, N], bit-exact with vecquant4recons_v2 (quant_cuda_kernel.cu:1127-1153)."""
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
+    gp, gs = _gidx_arg(g_idx, groupsize, G, need_multiple=8)
+    if _host is not None:
+        return _host.dequant(qweight, qzeros, scales, None if gp == 0 else g_idx, gs, out)
     if out is None:
         out = torch.empty((K, N), dtype=torch.float16, device=dev)
     _require(out.dtype == torch.float16 and tuple(out.shape) == (K, N) and out.is_contiguous() and out.device == dev,
              "out must be a contiguous float16 [K, N] tensor on the same device")
-    gp, gs = _gidx_arg(g_idx, groupsize, G, need_multiple=8)
     with _device_ctx(dev):
         rc = _lib.lib().q4_dequant_f16(qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), gp, gs,
                                        out.data_ptr(), K, N, G, _stream(dev))
@@ -353,6 +444,11 @@ def dequant2(qweight, qzeros, scales, g_idx=None, groupsize=None, out=None):
 def gemv(x, qweight, qzeros, scales, g_idx=None, groupsize=None, out=None, accumulate=False, out_shape=None):
     """y fp16 [M, N] = x [M, K] @ W for M <= 16 (decode).  `out_shape` (same number of elements)
     lets the result be allocated with the caller's leading dimensions instead of being a view."""
+    if _host is not None:
+        info = _layer_info(qweight, qzeros, scales, g_idx, groupsize)
+        if info.plan is None:
+            return _host.gemv(x, qweight, qzeros, scales, info.gemv_gidx, info.gemv_gs, out, bool(accumulate),
+                              _shape_arg(out_shape))
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     x2 = _flat_half(x, K, dev, "x")
     M = x2.shape[0]
@@ -403,6 +499,12 @@ def gemv_grouped(xs, layers, groupsize, outs=None, accumulate=False):
     if isinstance(xs, torch.Tensor):
         xs = [xs] * n
     _require(len(xs) == n, "one activation tensor per layer (or a single shared one)")
+    if _host is not None:
+        for lay in layers:
+            info = _layer_info(lay[0], lay[1], lay[2], lay[3] if len(lay) > 3 else None, groupsize)
+            _require(info.plan is None and info.gemv_gidx is None, "gemv_grouped needs sequential groups (no act-order)")
+        return _host.gemv_grouped(list(xs), [(lay[0], lay[1], lay[2]) for lay in layers], int(groupsize),
+                                  None if outs is None else list(outs), bool(accumulate))
     dev = K = M = None
     desc = (_lib.GemvLayer * n)()
     keep, shapes = [], []
@@ -470,6 +572,12 @@ def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, 
              lora_scale=1.0, out_shape=None):
     """y fp16 [M, N] = x @ W (+ bias) (+ lora_scale * xa @ lora_bt), W dequantized tile by tile in LDS.
     `lora_bt` is the adapter matrix as an [R, N] fp16/fp32 view with any strides (e.g. `lora_B.weight.t()`)."""
+    if _host is not None:
+        info = _layer_info(qweight, qzeros, scales, g_idx, groupsize)
+        if info.plan is None:
+            gi, gs = info.gemm_args()
+            return _host.gemm_fwd(x, qweight, qzeros, scales, gi, gs, bias, xa, lora_bt,
+                                  float(lora_scale), _shape_arg(out_shape))
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     x2 = _flat_half(x, K, dev, "x")
     M = x2.shape[0]
@@ -544,6 +652,13 @@ def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=Non
                 out_shape=None, dropout=None):
     """dx fp16 [M, K] = dy [M, N] @ W^T (+ lora_scale * dyb @ lora_a); lora_a is an [R, K] view.
     dropout=(seed, p): the adapter term is masked like dropout(x) (gradient of lora_B(lora_A(dropout(x))))."""
+    if _host is not None:
+        info = _layer_info(qweight, qzeros, scales, g_idx, groupsize)
+        if info.plan is None:
+            gi, gs = info.gemm_args()
+            return _host.gemm_bwd_dx(dy, qweight, qzeros, scales, gi, gs, dyb, lora_a,
+                                     float(lora_scale), _shape_arg(out_shape),
+                                     None if dropout is None else (int(dropout[0]), float(dropout[1])))
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     dy2 = _flat_half(dy, N, dev, "grad_output")
     M = dy2.shape[0]
@@ -582,6 +697,8 @@ def lora_down(inp, w, dropout=None):
     """out fp16 [M, R] = inp fp16 [M, C] @ w^T for an adapter matrix view w [R, C] (fp16/fp32, any positive
     strides): xa = x @ A^T with w = lora_A.weight, dyb = dy @ B with w = lora_B.weight.t()  (models.py:66).
     dropout=(seed, p): out = dropout(inp) @ w^T with the counter-based mask of (seed, p)."""
+    if _host is not None:
+        return _host.lora_down(inp, w, None if dropout is None else (int(dropout[0]), float(dropout[1])))
     _require(inp.is_cuda and inp.dtype == torch.float16 and inp.dim() == 2 and inp.is_contiguous(),
              "inp must be a contiguous float16 [M, C] CUDA tensor")
     M, C = inp.shape
@@ -638,6 +755,9 @@ def lora_grad_pair(p1, inp1, p2, inp2, alpha, dropout=None, outs=None):
     alpha * p2^T @ inp2 stored as a contiguous [C2, R] tensor) -- dA from (dyb, x) and dB in lora_B.weight's
     layout from (xa, dy).  Same requirements as lora_grad; p1 and p2 share their shape.
     dropout=(seed, p): inp1 is replaced by dropout(inp1) (inp2 is left as it is)."""
+    if _host is not None and outs is None:
+        return _host.lora_grad_pair(p1, inp1, p2, inp2, float(alpha),
+                                    None if dropout is None else (int(dropout[0]), float(dropout[1])))
     for p, inp in ((p1, inp1), (p2, inp2)):
         _require(p.is_cuda and p.dtype == torch.float16 and p.dim() == 2 and p.is_contiguous(),
                  "p must be a contiguous float16 [M, R] CUDA tensor")

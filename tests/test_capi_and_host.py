@@ -122,6 +122,25 @@ def test_error_codes_and_validation_need_no_gpu():
     assert L.q4_gemv_workspace_bytes(0, 4096, 11008) == 0
 
 
+def test_compiled_host_binding_is_built_and_matches_the_library():
+    """The pybind11 host module (csrc/host/q4_host.cpp) sits next to the library, was built against the same ABI
+    version, and quant_hip routes its operators through it.  Its argument checks run without a GPU."""
+    import torch
+    from alpaca_lora_4bit_amd import _lib, quant_hip
+    host = quant_hip._host
+    assert host is not None and host.abi_version() == _lib.ABI_VERSION
+    for name in ("dequant", "gemv", "gemv_grouped", "gemm_fwd", "gemm_bwd_dx", "lora_down", "lora_grad_pair",
+                 "reset_workspaces", "workspaces_are_zero"):
+        assert callable(getattr(host, name))
+    qw = torch.zeros((32, 128), dtype=torch.int32)
+    qz = torch.zeros((2, 16), dtype=torch.int32)
+    sc = torch.zeros((2, 128), dtype=torch.float16)
+    with pytest.raises(ValueError, match="GPU"):                      # CPU tensors are refused, nothing is computed on the host
+        host.gemv(torch.zeros((1, 256), dtype=torch.float16), qw, qz, sc, None, 128)
+    with pytest.raises(ValueError):
+        host.lora_down(torch.zeros((4, 64), dtype=torch.float16), torch.zeros((8, 64)))
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     from alpaca_lora_4bit_amd import _lib
     monkeypatch.setattr(_lib, "_lib", None)

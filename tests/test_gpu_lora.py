@@ -77,8 +77,7 @@ def test_lora_grad_does_not_disturb_gemv_workspace(oracle):
     quant_hip.lora_grad(pd, xd, 1.0)
     y1 = quant_hip.gemv(x, q, z, sc, None, 128)
     assert torch.equal(y0, y1)
-    for ws in quant_hip._workspaces.values():
-        assert int(ws.count_nonzero()) == 0
+    assert quant_hip.workspaces_are_zero()
 
 
 def test_fused_lora_function_against_oracle_fp32_adapters(oracle):
