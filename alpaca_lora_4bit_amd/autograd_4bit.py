@@ -179,6 +179,17 @@ class Autograd4bitQuantLinear(nn.Module):
         self.register_buffer('qweight', torch.empty((in_features * bits // 32, out_features), dtype=torch.int32))
 
     def forward(self, x):
+        if (self.bits == 4 and not self.is_v1_model and x.dtype == torch.float16 and backend == 'cuda'
+                and not torch.is_grad_enabled() and mm4b.use_new and mm4b.auto_switch):
+            # decode: the same call matmul4bit -> _matmul4bit_v2 would end in, without the stops on the way
+            rows = x.numel() // self.in_features if self.in_features else 0
+            if 1 <= rows <= min(int(mm4b.auto_switch_thd), quant_hip.MAX_GEMV_ROWS) and x.shape[-1] == self.in_features:
+                scales = self.scales
+                out = quant_hip.gemv(x, self.qweight, self.qzeros, scales if scales.dtype == torch.float16 else scales.half(),
+                                     self.g_idx, self.groupsize, out_shape=x.shape[:-1] + (self.out_features,))
+                if not self.disable_bias and not _is_all_zero(self.bias):
+                    out += self.bias
+                return out
         zeros = self.zeros if self.is_v1_model else self.qzeros
         if self.bits == 4:
             if torch.is_grad_enabled():
