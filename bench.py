@@ -25,10 +25,11 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, GB/s
 MFMA_FP16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 MFMA
-# HBM bytes per launch of the headline GEMV kernel, measured in two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE),
-# each scaled by what the same counter reads for a 256 MiB copy (--calibrate-copy): 23 587 KiB read + 432 KiB written.
-GEMV_TRAFFIC_BYTES = 24594000
-GEMV_TRAFFIC_SOURCE = "profiles/gemv_seq_mlp_decode_M1_hbm_traffic.md"
+# HBM bytes per launch of the headline kernel (the grouped gate|up GEMV), measured in two rocprofv3 --pmc runs
+# (FETCH_SIZE, WRITE_SIZE), each scaled by what the same counter reads for a 256 MiB copy (--calibrate-copy):
+# 2 x 23 470.3 KiB read + 903.0 KiB written.  Not re-measured by a bench run: the file named below holds the commands.
+GEMV_TRAFFIC_BYTES = 48991000
+GEMV_TRAFFIC_SOURCE = "profiles/gemv_mlp_decode_M1_gate_up_grouped_and_down.md"
 
 
 def gemv_bytes(M, K, N, G, act_order=False):
