@@ -246,6 +246,8 @@ def fuse_quant_linears(layers):
 def _cast_quant_buffers(model, dtype):
     for _, m in model.named_modules():
         if isinstance(m, Autograd4bitQuantLinear):
+            if gptq_backend_loaded:
+                quant_hip.invalidate(m)                    # whatever was cached about the old buffers goes with them
             if m.is_v1_model:
                 m.zeros = m.zeros.to(dtype)
             m.scales = m.scales.to(dtype)

@@ -114,7 +114,10 @@ def _matmul4bit_v2_recons(x, qweight, scales, zeros, g_idx, transpose=False, gro
         assert qweight.shape[1] == x.shape[-1]
     gs = _groupsize_of(qweight, scales, groupsize)
     lead = tuple(x.shape[:-1])
-    if use_dense_route(_rows(x)) and x.is_cuda:
+    # layers whose in / out features are not multiples of 128 are outside the tiled kernels: they take the dense route
+    # at every size (the dequantization needs only K % 32 == 0 and N % 64 == 0), as the reference does for every layer
+    odd_shape = (qweight.shape[0] * 8) % 128 != 0 or qweight.shape[1] % 128 != 0
+    if (use_dense_route(_rows(x)) or odd_shape) and x.is_cuda:
         return _dense_matmul(x, dense_weight(qweight, scales, zeros, g_idx, gs), transpose)
     if not transpose:
         return quant_hip.gemm_fwd(x, qweight, zeros, _half_scales(scales), g_idx, gs,

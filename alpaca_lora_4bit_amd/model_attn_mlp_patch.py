@@ -27,34 +27,39 @@ class FusedProjectionSlice(nn.Module):
     """Stands where one projection of a fused group stood; returns its columns of the fused output.
     The fused layer itself is registered once, on the parent module; the slices only point to it."""
 
-    def __init__(self, group, start, stop, last):
+    def __init__(self, group, start, stop):
         super().__init__()
         object.__setattr__(self, "_group", group)          # not a registered submodule: no duplicate state
         self.in_features = group.layer.in_features
         self.out_features = stop - start
-        self._start, self._stop, self._last = start, stop, last
+        self._start, self._stop = start, stop
 
     def forward(self, x):
-        y = self._group.run(x, release=self._last)
+        y = self._group.run(x)
         return y[..., self._start:self._stop]
 
 
 class _FusedGroup:
-    """Runs the fused layer once per input tensor and hands the result to every slice."""
+    """Runs the fused layer once per input tensor and hands the result to every slice.  The result is kept for as
+    long as the same tensor object comes back unmodified (identity and in-place version counter), whatever the order
+    in which the host block calls its projections; a forward hook on the block (installed by _fuse_children) drops
+    it when the block returns, so nothing stays pinned between forwards."""
 
     def __init__(self, layer):
         self.layer = layer
         self._x = None
+        self._version = -1
         self._y = None
 
-    def run(self, x, release):
-        if self._x is not x:
+    def run(self, x):
+        if self._x is not x or self._version != x._version:
             self._y = self.layer(x)
-            self._x = x
-        y = self._y
-        if release:                                          # the last projection of the group has been served
-            self._x = self._y = None
-        return y
+            self._x, self._version = x, x._version
+        return self._y
+
+    def clear(self, *unused):
+        self._x = self._y = None
+        self._version = -1
 
 
 def _fusable(mods):
@@ -72,16 +77,19 @@ def _fuse_children(parent, names, fused_name):
     fused = fuse_quant_linears(mods)
     group = _FusedGroup(fused)
     setattr(parent, fused_name, fused)
+    parent.register_forward_hook(group.clear)
     start = 0
     for i, (n, m) in enumerate(zip(names, mods)):
-        setattr(parent, n, FusedProjectionSlice(group, start, start + m.out_features, last=i == len(names) - 1))
+        setattr(parent, n, FusedProjectionSlice(group, start, start + m.out_features))
         start += m.out_features
     return True
 
 
 def make_quant_attn(model, is_v1_model=False):
     """Fuse q_proj / k_proj / v_proj of every attention block (model_attn_mlp_patch.py:73-160).
-    Returns the number of blocks fused.  Like the reference it turns the dense-buffer cache off."""
+    Returns the number of blocks fused.  Like the reference (model_attn_mlp_patch.py:78) it turns the shared dense
+    buffer off -- process-wide: above matmul_utils_4bit.dense_switch_rows rows every product then allocates its own
+    dense buffer; set matmul_utils_4bit.cache_buffer = True again if prefill batches of that size matter."""
     if is_v1_model:
         raise NotImplementedError("v1 (fp zeros) layers are not fused")
     matmul_utils_4bit.cache_buffer = False

@@ -10,7 +10,6 @@ lora_alpha / r); peft itself could not be imported where this was written, so eq
 peft's internals is not verified -- the adapter arithmetic (models.py:58-66) is.
 """
 import math
-import warnings
 
 import torch
 import torch.nn as nn
@@ -173,7 +172,7 @@ class Linear4bitLt(Autograd4bitQuantLinear, LoraLayer):
                 # decode: base product (GEMV), x @ A^T with the adapter read in place, one rank-r update in place:
                 # three launches instead of the seven of the composition below, same values up to fp16 rounding
                 result = Autograd4bitQuantLinear.forward(self, x)
-                xa = autograd_4bit.quant_hip.lora_down(x.reshape(-1, x.shape[-1]).to(torch.float16),
+                xa = autograd_4bit.quant_hip.lora_down(x.reshape(-1, x.shape[-1]).to(torch.float16).contiguous(),
                                                        self.lora_A[name].weight)
                 out2 = result.view(-1, result.shape[-1])
                 if out2.dtype == torch.float16:
@@ -243,62 +242,31 @@ def _move_adapters(new_module, device):
 
 
 if HAVE_PEFT:  # pragma: no cover - peft is not available where the tests run
-    from peft.tuners.lora import Linear as _PeftLinear
-    from transformers.pytorch_utils import Conv1D
+    # peft's own hooks, taken before replace_peft_model_with_int4_lora_model() redirects them: every target that is
+    # not a 4-bit layer is handed on to them unchanged
+    _peft_create_new_module = _peft_lora.LoraModel.__dict__["_create_new_module"].__func__
+    _peft_replace_module = _peft_lora.LoraModel.__dict__["_replace_module"]
+    _peft_replace_module = getattr(_peft_replace_module, "__func__", _peft_replace_module)
 
     class GPTQLoraModel(_peft_lora.LoraModel):
         """peft LoraModel that builds Linear4bitLt for 4-bit targets (models.py:79-163)."""
 
         @staticmethod
         def _create_new_module(lora_config, adapter_name, target, **kwargs):
-            bias = kwargs.pop("bias", False)
             if isinstance(target, Autograd4bitQuantLinear):
+                bias = kwargs.pop("bias", False)
                 return Linear4bitLt(adapter_name, target.in_features, target.out_features, target.groupsize,
                                     target.is_v1_model, bias=bias, **kwargs)
-            if isinstance(target, torch.nn.Linear):
-                in_features, out_features = target.in_features, target.out_features
-                if kwargs["fan_in_fan_out"]:
-                    warnings.warn("fan_in_fan_out is set to True but the target module is `torch.nn.Linear`. "
-                                  "Setting fan_in_fan_out to False.")
-                    kwargs["fan_in_fan_out"] = lora_config.fan_in_fan_out = False
-            elif isinstance(target, Conv1D):
-                in_features, out_features = (target.weight.ds_shape if hasattr(target.weight, "ds_shape")
-                                             else target.weight.shape)
-                kwargs["is_target_conv_1d_layer"] = True
-                if not kwargs["fan_in_fan_out"]:
-                    warnings.warn("fan_in_fan_out is set to False but the target module is `Conv1D`. "
-                                  "Setting fan_in_fan_out to True.")
-                    kwargs["fan_in_fan_out"] = lora_config.fan_in_fan_out = True
-            else:
-                raise ValueError(f"Target module {target} is not supported. "
-                                 f"Currently, only `torch.nn.Linear` and `Conv1D` are supported.")
-            return _PeftLinear(adapter_name, in_features, out_features, bias=bias, **kwargs)
+            return _peft_create_new_module(lora_config, adapter_name, target, **kwargs)
 
         @staticmethod
         def _replace_module(parent, child_name, new_module, child):
-            setattr(parent, child_name, new_module)
             if isinstance(child, Autograd4bitQuantLinear) and isinstance(new_module, Linear4bitLt):
+                setattr(parent, child_name, new_module)
                 _share_quant_tensors(new_module, child)
-                if getattr(child, "state", None) is not None:
-                    new_module.state = child.state
-                    new_module.to(child.qweight.device)
                 _move_adapters(new_module, child.qweight.device)
                 return
-            if hasattr(child, "base_layer"):
-                child = child.base_layer
-            elif hasattr(child, "quant_linear_module"):
-                child = child.quant_linear_module
-            if not hasattr(new_module, "base_layer"):
-                new_module.weight = child.weight
-                if hasattr(child, "bias"):
-                    new_module.bias = child.bias
-            if getattr(child, "state", None) is not None:
-                if hasattr(new_module, "base_layer"):
-                    new_module.base_layer.state = child.state
-                else:
-                    new_module.state = child.state
-                new_module.to(child.weight.device)
-            _move_adapters(new_module, child.weight.device)
+            return _peft_replace_module(parent, child_name, new_module, child)
 else:
     class GPTQLoraModel:
         """Without peft there is no LoraModel to derive from; the two hooks the monkeypatch

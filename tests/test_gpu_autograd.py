@@ -319,3 +319,59 @@ def test_empty_batches(oracle, shape):
         assert xg.grad is not None and xg.grad.shape == x.shape
     for w in (lora.lora_A["default"].weight, lora.lora_B["default"].weight):
         assert w.grad is not None and float(w.grad.abs().max()) == 0.0
+
+
+def test_layers_outside_the_tiled_kernels_take_the_dense_route(oracle):
+    """in / out features that are not multiples of 128 (here 160 -> 192): above 16 rows the tiled kernels do not
+    apply, the layer then runs dense dequantization + a library GEMM, forward and backward, like every layer of the
+    reference (matmul_utils_4bit.py:114-127); up to 16 rows it takes the GEMV."""
+    import torch
+    from alpaca_lora_4bit_amd import models
+    from alpaca_lora_4bit_amd.autograd_4bit import Autograd4bitQuantLinear
+    K, N = 160, 192
+    layer = oracle.make_layer(K, N, 32, seed=31)
+    m = _fill(Autograd4bitQuantLinear(K, N, groupsize=32), layer)
+    for rows in (1, 16, 17, 200):
+        x = oracle.make_activations(rows, K, seed=rows)
+        dy = oracle.make_activations(rows, N, seed=rows + 1)
+        ref = oracle.matmul_recons(x, layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
+        refx = oracle.matmul_recons_t(dy, layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
+        xt = torch.from_numpy(x).cuda().requires_grad_(True)
+        y = m(xt)
+        y.backward(torch.from_numpy(dy).cuda())
+        assert rel_err(y.detach().cpu().numpy(), ref) <= TOL
+        assert rel_err(xt.grad.cpu().numpy(), refx) <= TOL
+        with torch.no_grad():
+            assert rel_err(m(torch.from_numpy(x).cuda()).cpu().numpy(), ref) <= TOL
+    # with an adapter: the reference composition on top of the same route
+    A, B = oracle.make_lora(K, N, 8, seed=3)
+    lt = models.Linear4bitLt("default", K, N, 32, False, r=8, lora_alpha=16).cuda()
+    _fill(lt, layer)
+    lt.lora_A["default"].weight.data = torch.from_numpy(A).cuda()
+    lt.lora_B["default"].weight.data = torch.from_numpy(B).cuda()
+    x = oracle.make_activations(64, K, seed=9)
+    W = oracle.dequant_v2(layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"]).astype(np.float64)
+    with torch.amp.autocast(device_type="cuda"):
+        y = lt(torch.from_numpy(x).cuda())
+    assert rel_err(y.detach().float().cpu().numpy(), oracle.lora_forward(x, W, A, B, 2.0)) <= TOL
+
+
+def test_decode_with_adapter_takes_a_strided_last_token_view(oracle):
+    """h[:, -1:, :] of a batch is not contiguous: the short adapter path must accept it."""
+    import torch
+    from alpaca_lora_4bit_amd import models
+    K, N, r = 256, 128, 8
+    layer = oracle.make_layer(K, N, 128, seed=37)
+    A, B = oracle.make_lora(K, N, r, seed=37)
+    m = models.Linear4bitLt("default", K, N, 128, False, r=r, lora_alpha=16).cuda().eval()
+    _fill(m, layer)
+    m.lora_A["default"].weight.data = torch.from_numpy(A).cuda()
+    m.lora_B["default"].weight.data = torch.from_numpy(B).cuda()
+    h = torch.from_numpy(oracle.make_activations(3 * 5, K, seed=6)).cuda().view(3, 5, K)
+    last = h[:, -1:, :]
+    assert not last.is_contiguous()
+    with torch.no_grad():
+        y = m(last)
+    W = oracle.dequant_v2(layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"]).astype(np.float64)
+    ref = oracle.lora_forward(last.reshape(3, K).cpu().numpy(), W, A, B, 2.0)
+    assert y.shape == (3, 1, N) and rel_err(y.reshape(3, N).cpu().numpy(), ref) <= TOL

@@ -111,6 +111,23 @@ def test_fused_qkv_and_gate_up_keep_the_logits(tmp_path, oracle):
     for a, b in ((after, before), (after1, before1)):
         assert (a - b).abs().max().item() <= 2e-3 * b.abs().max().item()
     assert make_quant_attn(model) == 0                       # idempotent: nothing left to fuse
+    # the slices in any order, one fused launch per input; an in-place change of the input is noticed; nothing stays
+    # cached once the block has returned
+    attn = layer0.self_attn
+    calls = []
+    handle = attn.qkv_proj.register_forward_hook(lambda m, i, o: calls.append(1))
+    x = torch.randn(1, 3, 256, device="cuda", dtype=torch.float16)
+    with torch.no_grad():
+        v, q, k = attn.v_proj(x), attn.q_proj(x), attn.k_proj(x)
+        assert len(calls) == 1
+        full = attn.qkv_proj(x)
+        assert torch.equal(torch.cat([q, k, v], dim=-1), full)
+        x.mul_(2.0)
+        q2 = attn.q_proj(x)
+        assert len(calls) == 3 and not torch.equal(q2, q)
+        model(ids[:, :1])
+    handle.remove()
+    assert attn.q_proj._group._x is None and attn.q_proj._group._y is None
 
 
 @pytest.mark.gpu
