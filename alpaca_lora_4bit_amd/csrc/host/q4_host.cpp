@@ -346,7 +346,7 @@ std::pair<at::Tensor, at::Tensor> lora_grad_pair(const at::Tensor& p1, const at:
     }
     TORCH_CHECK_VALUE(p1.sizes() == p2.sizes() && p1.device() == p2.device(), "the two rank-R operands must share shape and device");
     const int64_t M = p1.size(0), R = p1.size(1), C1 = in1.size(1), C2 = in2.size(1);
-    TORCH_CHECK_VALUE((R == 8 || R == 16) && C1 % 8 == 0 && C2 % 8 == 0, "lora_grad needs R in (8, 16) and C % 8 == 0");
+    TORCH_CHECK_VALUE(R >= 2 && R <= 32 && R % 2 == 0 && C1 % 8 == 0 && C2 % 8 == 0, "lora_grad needs an even R in 2..32 and C % 8 == 0");
     const auto opt = at::TensorOptions().dtype(at::kFloat).device(p1.device());
     if (M == 0) return {at::zeros({R, C1}, opt), at::zeros({C2, R}, opt)};
     at::Tensor o1 = at::empty({R, C1}, opt), o2 = at::empty({C2, R}, opt);

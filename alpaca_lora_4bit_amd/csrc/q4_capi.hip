@@ -283,7 +283,7 @@ extern "C" int q4_lora_down_f16(const void* in, const void* w, int w_sr, int w_s
 }
 
 extern "C" size_t q4_lora_grad_workspace_bytes(int M, int C, int R) {
-    if (M < 1 || C < 8 || (R != 8 && R != 16)) return 0;
+    if (M < 1 || C < 8 || R < 2 || R > 32 || (R & 1)) return 0;
     return q4_lora_grad_workspace(M, C, R);
 }
 
@@ -294,7 +294,7 @@ extern "C" int q4_lora_grad_f32(const void* p, const void* in, float* out, int o
     q4_drop_args da;
     const q4_drop_args* dp;
     if (!make_drop(drop, &da, &dp)) return Q4_ERR_BAD_SHAPE;
-    if (M < 1 || C < 8 || (C % 8) != 0 || (R != 8 && R != 16) || o_sr < 1 || o_sc < 1) return Q4_ERR_BAD_SHAPE;
+    if (M < 1 || C < 8 || (C % 8) != 0 || R < 2 || R > 32 || (R & 1) || o_sr < 1 || o_sc < 1) return Q4_ERR_BAD_SHAPE;
     if ((long long)M * C * 2 >= 0x70000000ll || C > (1 << 20)) return Q4_ERR_BAD_SHAPE;     /* 32-bit buffer offsets */
     if (misaligned(p) || misaligned(in) || (reinterpret_cast<uintptr_t>(out) & 3u)) return Q4_ERR_MISALIGNED;
     const size_t need = q4_lora_grad_workspace(M, C, R);
@@ -313,7 +313,7 @@ extern "C" int q4_lora_grad_pair_f32(const void* p1, const void* in1, float* out
     q4_drop_args da;
     const q4_drop_args* dp;
     if (!make_drop(drop1, &da, &dp)) return Q4_ERR_BAD_SHAPE;
-    if (M < 1 || (R != 8 && R != 16)) return Q4_ERR_BAD_SHAPE;
+    if (M < 1 || R < 2 || R > 32 || (R & 1)) return Q4_ERR_BAD_SHAPE;
     const int Cs[2] = {C1, C2};
     const int strides[4] = {o1_sr, o1_sc, o2_sr, o2_sc};
     for (int i = 0; i < 2; ++i) {

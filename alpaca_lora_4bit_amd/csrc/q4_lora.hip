@@ -227,31 +227,27 @@ __global__ __launch_bounds__(64 * kDownWaves) void lora_down_kernel(const half_t
     }
 }
 
-// ---- gradient of an adapter matrix -------------------------------------------------------
-// out[j, c] = alpha * sum_m P[m, j] * in[m, c].  A thread owns CPT = 64/R adjacent columns (R is 8
-// or 16: 8 or 4 columns) and R x CPT fp32 accumulators; the 4 wavefronts of a workgroup share a
-// block of 64*CPT columns and split its rows 16 at a time; gridDim.y workgroups share a column
-// block.  Two rows are multiplied per instruction with v_dot2_f32_f16: rows (2i, 2i+1) of `in` are
-// interleaved in registers with two byte permutes per dword, the matching pairs of P come from
-// LDS as broadcasts.  The sum over wavefronts goes through LDS; the sum over workgroups goes
-// through fp32 partial tiles in the workspace that a second small kernel adds in a fixed order
-// (bit-reproducible, no atomics, nothing to pre-clear).
-// Partial tile layout: part[split][column block][a = j*CPT + e][lane], i.e. exactly the order the
-// workgroup produces, so both kernels read and write it fully coalesced; only the final, small
-// output goes through the caller's strides.
-constexpr int kGradWaves = 4;
-
-template <int ND, int NPP>
-struct RowRegs { uint32_t d[16][ND]; uint32_t plo[NPP], phi[NPP]; };
+// ---- gradient of an adapter matrix --------------------------------------------------------
+// out[j, c] = alpha * sum_m P[m, j] * in[m, c] as v_mfma_f32_16x16x32_f16 products whose reduction index is the ROW m:
+//   A operand  P^T: lane (j = l % 16, kk = l / 16) holds P[mb + 8*kk .. + 7][j]   (rows j >= R are zero)
+//   B operand  in:  lane (cg = l % 16, kk) holds in[mb + 8*kk .. + 7][col]         for ONE column per MFMA
+// A lane loads eight 16-byte pieces, rows mb + 8*kk + e (e = 0..7) x columns c0 + 8*cg .. + 7 (256 contiguous bytes
+// per 16 lanes and row), and turns the 8 x 8 block around in registers with 32 byte permutes; MFMA i of the eight
+// then multiplies column c0 + 8*cg + i.  A wavefront so consumes a block of 32 rows x 128 columns (8 KB) with 8
+// loads, 32 permutes and 8 MFMAs per 16 adapter rows; the kernel is bound by its loads.  P for the block (32 x R
+// values, R even and at most 32) is fetched with 4-byte loads and transposed through a wavefront-private LDS tile.
+// Workgroup = 4 wavefronts on one 128-column strip and `rows_per_wg` rows (wavefront w takes the 32-row blocks
+// w, w + 4, ...); the sum over wavefronts goes through LDS, the sum over the gridDim.y workgroups of a strip through
+// fp32 partial tiles [split][strip][R][128] that lora_grad_reduce_kernel adds in a fixed order (bit-reproducible).
+constexpr int kG2Waves = 4, kG2Cols = 128, kG2PadRows = 40;
 
 // One or two gradients per launch (blockIdx.z): the two adapter gradients of a layer share M, R and alpha and are
-// independent, and since a single one is bound by the latency of its burst of loads, running them side by side
-// costs little more than one.  Workgroups beyond a problem's own grid leave at once.
+// independent, so they go out side by side.  Workgroups beyond a problem's own grid leave at once.
 struct GradProb {
     const half_t* P;          // [M, R]
     const half_t* in;         // [M, C]
     float* out;               // through o_sr, o_sc
-    float* part;              // partial tiles [splits][col_blocks][NACC][64]
+    float* part;              // partial tiles [splits][col_blocks][R][128]
     int o_sr, o_sc, C, col_blocks, splits, rows_per_wg;
     DropArgs drop;            // dropout mask applied to `in` (thr15 == 0: none); the result carries drop.scale
 };
@@ -261,163 +257,165 @@ struct GradArgs {
     int M;
 };
 
-template <int R>
-__global__ __launch_bounds__(64 * kGradWaves) __attribute__((amdgpu_waves_per_eu(2, 2))) void lora_grad_kernel(GradArgs ga) {
+
+template <int NPL>
+struct G2Regs { uint4_t d[8]; uint32_t p[NPL]; };
+
+template <bool DROP, int RB>    // RB = ceil(R / 16) A operands (1 or 2); R is even
+__global__ __launch_bounds__(64 * kG2Waves) void lora_grad_kernel(GradArgs ga, int R) {
     const GradProb& q = ga.p[blockIdx.z];
     if ((int)blockIdx.x >= q.col_blocks || (int)blockIdx.y >= q.splits) return;       // uniform over the workgroup
-    const half_t* __restrict__ P = q.P;
-    const half_t* __restrict__ in = q.in;
-    float* __restrict__ out = q.out;
-    float* __restrict__ part = q.part;
-    const int o_sr = q.o_sr, o_sc = q.o_sc, C = q.C, rows_per_wg = q.rows_per_wg, M = ga.M;
-    const float alpha = ga.alpha * q.drop.scale;
-    const DropArgs drop = q.drop;
-    const uint32_t thr_pair = drop.thr15 | (drop.thr15 << 16);
-    constexpr int CPT = 64 / R;                  // columns per thread: 8 (R = 8) or 4 (R = 16)
-    constexpr int ND = CPT / 2;                  // dwords per thread and row
-    constexpr int NPP = 8 * R / 64;              // pairs of P staged per lane and 16-row block
-    constexpr int NACC = R * CPT;                // 64
-    __shared__ float red[kGradWaves][NACC][64];  // 64 KB
-    __shared__ __attribute__((aligned(16))) uint32_t ppair[kGradWaves][8 * R];
+    constexpr int NPL = 4 * RB;                                                       // 4-byte loads of P per lane and block
+    __shared__ float red[kG2Waves][16][kG2Cols];                                      // 32 KB
+    __shared__ __attribute__((aligned(16))) half_t pt[kG2Waves][16 * RB][kG2PadRows]; // P^T of the current block
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int c0 = (blockIdx.x * 64 + lane) * CPT;
-    // lanes past the last column get an offset beyond the buffer: their loads return zero
-    const int voff = c0 < C ? c0 * 2 : kFarOffset;
+    const int cg = lane & 15, kk = lane >> 4;
+    const int C = q.C, M = ga.M;
     const int row_bytes = C * 2;
-    const int rows_per_wave = rows_per_wg / kGradWaves;           // a multiple of 16
-    const int m_begin = blockIdx.y * rows_per_wg + wave * rows_per_wave;
-    const int m_end = min(m_begin + rows_per_wave, M);
-    // both buffers end at this wavefront's last row: rows past it read as zero
-    const rsrc_t rs_in = make_rsrc(in, (unsigned)max(m_end, 0) * (unsigned)row_bytes);
-    const rsrc_t rs_p = make_rsrc(P, (unsigned)max(m_end, 0) * (unsigned)(R * 2));
-    float acc[R][CPT];
+    const int c0 = blockIdx.x * kG2Cols + 8 * cg;
+    const int m_wg = blockIdx.y * q.rows_per_wg;
+    const int m_end = min(m_wg + q.rows_per_wg, M);
+    const rsrc_t rs_in = make_rsrc(q.in, (unsigned)m_end * (unsigned)row_bytes);       // rows past m_end read as zero
+    const rsrc_t rs_p = make_rsrc(q.P, (unsigned)m_end * (unsigned)(R * 2));
+    int voff[8];
 #pragma unroll
-    for (int j = 0; j < R; ++j)
+    for (int e = 0; e < 8; ++e) voff[e] = c0 < C ? (8 * kk + e) * row_bytes + c0 * 2 : kFarOffset;
+    // this lane's share of a block of P: the pairs i = lane, lane + 64, ... of the 32 x R block
+    // (row i / (R/2), columns 2 * (i % (R/2)) and the next)
+    const int hr = R >> 1;
+    int pvoff[NPL], pdst[NPL];
 #pragma unroll
-        for (int e = 0; e < CPT; ++e) acc[j][e] = 0.f;
+    for (int t = 0; t < NPL; ++t) {
+        const int i = lane + 64 * t, m = i / hr, j = 2 * (i - m * hr);
+        pvoff[t] = i < 32 * hr ? i * 4 : kFarOffset;
+        pdst[t] = i < 32 * hr ? j * kG2PadRows + m : -1;
+    }
+    half_t* const ptw = &pt[wave][0][0];
+    for (int i = lane; i < 16 * RB * kG2PadRows; i += 64) ptw[i] = (half_t)0.f;   // rows j >= R stay zero
+    const DropArgs drop = q.drop;
+    const uint32_t thr_pair = drop.thr15 | (drop.thr15 << 16);
 
-    // Loads of one 16-row block: first the pairs (P[2i][j], P[2i+1][j]) this lane will stage in LDS,
-    // then the 16 rows of `in`.  No branches: a block past the end is fetched from kFarOffset.
-    auto load_rows = [&](RowRegs<ND, NPP>& x, int mb) {
+    float4_t acc[RB][8];
+#pragma unroll
+    for (int b = 0; b < RB; ++b)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[b][i] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    auto load_block = [&](G2Regs<NPL>& x, int mb) {
         const bool live = mb < m_end;
+        const int soff = live ? mb * row_bytes : kFarOffset;
         const int soff_p = live ? mb * R * 2 : kFarOffset;
-        const int soff_x = live ? mb * row_bytes : kFarOffset;
 #pragma unroll
-        for (int t = 0; t < NPP; ++t) {
-            const int i = lane + 64 * t, pi = i / R, j = i - pi * R;
-            x.plo[t] = buf_load16(rs_p, (2 * pi * R + j) * 2, soff_p);
-            x.phi[t] = buf_load16(rs_p, ((2 * pi + 1) * R + j) * 2, soff_p);
-        }
+        for (int t = 0; t < NPL; ++t) x.p[t] = buf_load32(rs_p, pvoff[t], soff_p);
 #pragma unroll
-        for (int rr = 0; rr < 16; ++rr) {
-            const int soff = soff_x + rr * row_bytes;
-            if constexpr (ND == 4) {
-                const uint4_t v = buf_load128(rs_in, voff, soff);
-                x.d[rr][0] = v.x; x.d[rr][1] = v.y; x.d[rr][2] = v.z; x.d[rr][3] = v.w;
-            } else {
-                const uint2_t v = buf_load64(rs_in, voff, soff);
-                x.d[rr][0] = v.x; x.d[rr][1] = v.y;
-            }
-        }
+        for (int e = 0; e < 8; ++e) x.d[e] = buf_load128(rs_in, voff[e], soff);
     };
-    auto consume = [&](RowRegs<ND, NPP>& x, int mb) {
-        if (drop.thr15) {                         // uniform: rows mb .. mb+15, this thread's column pairs c0/2 .. + ND-1
+    auto consume = [&](G2Regs<NPL>& x, int mb) {
+        if (DROP && drop.thr15) {                 // uniform: the mask belongs to one problem of a pair
 #pragma unroll
-            for (int rr = 0; rr < 16; ++rr) {
-                const uint32_t key = drop_row_key(drop, (uint32_t)(mb + rr));
-#pragma unroll
-                for (int d = 0; d < ND; ++d)
-                    x.d[rr][d] &= drop_keep_mask(drop_word(drop, key, (uint32_t)(c0 >> 1) + d), thr_pair);
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t key = drop_row_key(drop, (uint32_t)(mb + 8 * kk + e));
+                const uint32_t pr = (uint32_t)(c0 >> 1);
+                x.d[e].x &= drop_keep_mask(drop_word(drop, key, pr), thr_pair);
+                x.d[e].y &= drop_keep_mask(drop_word(drop, key, pr + 1), thr_pair);
+                x.d[e].z &= drop_keep_mask(drop_word(drop, key, pr + 2), thr_pair);
+                x.d[e].w &= drop_keep_mask(drop_word(drop, key, pr + 3), thr_pair);
             }
         }
-        // pairs of P -> LDS (wavefront-private region; LDS operations of one wavefront are ordered)
 #pragma unroll
-        for (int t = 0; t < NPP; ++t) ppair[wave][lane + 64 * t] = x.plo[t] | (x.phi[t] << 16);
+        for (int t = 0; t < NPL; ++t)
+            if (pdst[t] >= 0) {
+                ptw[pdst[t]] = __builtin_bit_cast(half_t, (uint16_t)(x.p[t] & 0xFFFFu));
+                ptw[pdst[t] + kG2PadRows] = __builtin_bit_cast(half_t, (uint16_t)(x.p[t] >> 16));
+            }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        half8_t aop[RB];
 #pragma unroll
-        for (int pi = 0; pi < 8; ++pi) {
-            if constexpr (R > 8) __builtin_amdgcn_sched_barrier(0);   // bounds the live LDS reads (register pressure)
-            uint32_t p2[R];
+        for (int b = 0; b < RB; ++b) aop[b] = *reinterpret_cast<const half8_t*>(ptw + (16 * b + cg) * kG2PadRows + 8 * kk);
+        __builtin_amdgcn_wave_barrier();
+        // 8 x 8 turn: tr[c][q] = (row 2q, row 2q + 1) of column c of this lane's block
+        uint32_t tr[8][4];
 #pragma unroll
-            for (int j = 0; j < R; j += 4) {
-                const uint4_t pv = *reinterpret_cast<const uint4_t*>(&ppair[wave][pi * R + j]);
-                p2[j] = pv.x; p2[j + 1] = pv.y; p2[j + 2] = pv.z; p2[j + 3] = pv.w;
-            }
+        for (int qq = 0; qq < 4; ++qq) {
+            const uint4_t r0 = x.d[2 * qq], r1 = x.d[2 * qq + 1];
+            const uint32_t a0[4] = {r0.x, r0.y, r0.z, r0.w}, a1[4] = {r1.x, r1.y, r1.z, r1.w};
 #pragma unroll
-            for (int d = 0; d < ND; ++d) {
-                const uint32_t r0 = x.d[2 * pi][d], r1 = x.d[2 * pi + 1][d];
-                const half2_t xlo = as_half2(__builtin_amdgcn_perm(r1, r0, 0x05040100u));   // column 2d of both rows
-                const half2_t xhi = as_half2(__builtin_amdgcn_perm(r1, r0, 0x07060302u));   // column 2d+1
-#pragma unroll
-                for (int j = 0; j < R; ++j) {
-                    acc[j][2 * d] = __builtin_amdgcn_fdot2(as_half2(p2[j]), xlo, acc[j][2 * d], false);
-                    acc[j][2 * d + 1] = __builtin_amdgcn_fdot2(as_half2(p2[j]), xhi, acc[j][2 * d + 1], false);
-                }
+            for (int p = 0; p < 4; ++p) {
+                tr[2 * p][qq] = __builtin_amdgcn_perm(a1[p], a0[p], 0x05040100u);
+                tr[2 * p + 1][qq] = __builtin_amdgcn_perm(a1[p], a0[p], 0x07060302u);
             }
         }
-        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint4_t bq = {tr[i][0], tr[i][1], tr[i][2], tr[i][3]};
+#pragma unroll
+            for (int b = 0; b < RB; ++b)
+                acc[b][i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(aop[b], __builtin_bit_cast(half8_t, bq), acc[b][i], 0, 0, 0);
+        }
     };
 
-    // rows in blocks of 16, the next block's loads in flight while the current one is consumed
-    RowRegs<ND, NPP> xa, xb;
-    load_rows(xa, m_begin);
-    for (int mb = m_begin; mb < m_end; mb += 32) {
-        load_rows(xb, mb + 16);
+    // blocks w, w + 4, ... of the workgroup's rows; the next block's loads are in flight while one is consumed
+    const int step = 32 * kG2Waves;
+    G2Regs<NPL> xa, xb;
+    int mb = m_wg + 32 * wave;
+    load_block(xa, mb);
+    for (; mb < m_end; mb += 2 * step) {
+        load_block(xb, mb + step);
         consume(xa, mb);
-        load_rows(xa, mb + 32);
-        if (mb + 16 < m_end) consume(xb, mb + 16);
+        load_block(xa, mb + 2 * step);
+        if (mb + step < m_end) consume(xb, mb + step);
     }
-#pragma unroll
-    for (int j = 0; j < R; ++j)
-#pragma unroll
-        for (int e = 0; e < CPT; ++e) red[wave][j * CPT + e][lane] = acc[j][e];
-    __syncthreads();
     const bool direct = q.splits == 1;
-    float* tile = part + ((size_t)blockIdx.y * q.col_blocks + blockIdx.x) * (NACC * 64);
-    for (int o = threadIdx.x; o < NACC * 64; o += 64 * kGradWaves) {
-        const int a = o >> 6, ln = o & 63;
-        float v = 0.f;
+    const float alpha = ga.alpha * drop.scale;
+    float* tile = q.part + ((size_t)blockIdx.y * q.col_blocks + blockIdx.x) * (size_t)(R * kG2Cols);
 #pragma unroll
-        for (int wv = 0; wv < kGradWaves; ++wv) v += red[wv][a][ln];
-        if (direct) {
-            const int j = a / CPT, cc = (blockIdx.x * 64 + ln) * CPT + (a - j * CPT);
-            if (cc < C) out[(size_t)j * o_sr + (size_t)cc * o_sc] = alpha * v;
-        } else {
-            tile[o] = v;
+    for (int b = 0; b < RB; ++b) {
+        if (b > 0) __syncthreads();
+        // acc[b][i][r]: adapter row j = 16*b + 4*kk + r, column 8*cg + i of the strip
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float* dst = &red[wave][4 * kk + r][8 * cg];
+            *reinterpret_cast<float4_t*>(dst) = float4_t{acc[b][0][r], acc[b][1][r], acc[b][2][r], acc[b][3][r]};
+            *reinterpret_cast<float4_t*>(dst + 4) = float4_t{acc[b][4][r], acc[b][5][r], acc[b][6][r], acc[b][7][r]};
+        }
+        __syncthreads();
+        const int nj = min(16, R - 16 * b);
+        for (int o = threadIdx.x; o < nj * kG2Cols; o += 64 * kG2Waves) {
+            const int jl = o >> 7, cl = o & (kG2Cols - 1), j = 16 * b + jl;
+            const float v = (red[0][jl][cl] + red[1][jl][cl]) + (red[2][jl][cl] + red[3][jl][cl]);
+            if (direct) {
+                const int cc = blockIdx.x * kG2Cols + cl;
+                if (cc < C) q.out[(size_t)j * q.o_sr + (size_t)cc * q.o_sc] = alpha * v;
+            } else {
+                tile[j * kG2Cols + cl] = v;
+            }
         }
     }
 }
 
-// Adds the `splits` partial tiles of every column block in order and writes the scaled result.
-template <int R>
-__global__ __launch_bounds__(256) void lora_grad_reduce_kernel(GradArgs ga) {
+// Adds the `splits` partial tiles of every strip in order and writes the scaled result through the caller's strides.
+__global__ __launch_bounds__(256) void lora_grad_reduce_kernel(GradArgs ga, int R) {
     const GradProb& q = ga.p[blockIdx.y];
+    const int total = q.col_blocks * R * kG2Cols;              // one split's tiles: [strip][j][column]
+    const int t = blockIdx.x * 256 + threadIdx.x;
+    if (q.splits <= 1 || t >= total) return;                   // a single split was written directly
     const float* __restrict__ part = q.part;
-    float* __restrict__ out = q.out;
-    const int o_sr = q.o_sr, o_sc = q.o_sc, C = q.C, col_blocks = q.col_blocks, splits = q.splits;
-    const float alpha = ga.alpha * q.drop.scale;
-    constexpr int CPT = 64 / R;
-    constexpr int NACC = R * CPT;
-    const int t = blockIdx.x * 256 + threadIdx.x;         // index into one split's tiles: [column block][a][lane]
-    const int total = col_blocks * NACC * 64;
-    if (splits <= 1 || t >= total) return;                // a single split was written directly
     float v = 0.f;
     int s = 0;
-    for (; s + 8 <= splits; s += 8) {
+    for (; s + 8 <= q.splits; s += 8) {
         float u[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) u[i] = part[(size_t)(s + i) * total + t];
 #pragma unroll
         for (int i = 0; i < 8; ++i) v += u[i];
     }
-    for (; s < splits; ++s) v += part[(size_t)s * total + t];
-    const int bx = t / (NACC * 64), o = t - bx * (NACC * 64);
-    const int a = o >> 6, ln = o & 63;
-    const int j = a / CPT, cc = (bx * 64 + ln) * CPT + (a - j * CPT);
-    if (cc < C) out[(size_t)j * o_sr + (size_t)cc * o_sc] = alpha * v;
+    for (; s < q.splits; ++s) v += part[(size_t)s * total + t];
+    const int bx = t / (R * kG2Cols), o = t - bx * (R * kG2Cols);
+    const int j = o >> 7, cc = bx * kG2Cols + (o & (kG2Cols - 1));
+    if (cc < q.C) q.out[(size_t)j * q.o_sr + (size_t)cc * q.o_sc] = ga.alpha * q.drop.scale * v;
 }
 
 // keep[m, c] = 1 where dropout keeps element (m, c), else 0: the mask the kernels above regenerate, written out
@@ -432,16 +430,17 @@ __global__ __launch_bounds__(256) void dropout_keep_kernel(uint8_t* __restrict__
     keep[(size_t)m * C + 2 * pr + 1] = ((w >> 16) & 0x7FFFu) >= drop.thr15;
 }
 
+// 128-column strips; enough row splits for about two workgroups per CU over both problems of a pair (their partial
+// tiles cost 2 * splits * R * C * 4 bytes of traffic); rows per workgroup a multiple of 128 (4 wavefronts x 32 rows).
 struct GradPlan { int col_blocks, splits, rows_per_wg; };
-inline GradPlan plan_grad(int M, int C, int R) {
+inline GradPlan plan_grad(int M, int C) {
+    static const int env_wgs = getenv("Q4_LORA_GRAD_WGS") ? atoi(getenv("Q4_LORA_GRAD_WGS")) : 384;
     GradPlan g;
-    const int cpt = 64 / R;
-    g.col_blocks = (C + 64 * cpt - 1) / (64 * cpt);
-    // rows per workgroup: a multiple of 64 (4 wavefronts x 16 rows); about one workgroup for each of
-    // the 256 CUs, at most 32 row splits (their partial tiles cost 2*splits*R*C*4 bytes of traffic)
-    int splits = (256 + g.col_blocks - 1) / g.col_blocks;
-    if (splits > 32) splits = 32;
-    const int unit = 16 * kGradWaves;
+    g.col_blocks = (C + kG2Cols - 1) / kG2Cols;
+    int splits = (env_wgs + g.col_blocks - 1) / g.col_blocks;
+    if (splits > 64) splits = 64;
+    if (splits < 1) splits = 1;
+    const int unit = 32 * kG2Waves;
     g.rows_per_wg = ((M + splits - 1) / splits + unit - 1) / unit * unit;
     g.splits = (M + g.rows_per_wg - 1) / g.rows_per_wg;
     return g;
@@ -509,13 +508,13 @@ extern "C" int q4_launch_lora_down(const void* in, const void* w, int w_sr, int 
 }
 
 extern "C" size_t q4_lora_grad_workspace(int M, int C, int R) {
-    const q4::GradPlan g = q4::plan_grad(M, C, R);
-    return g.splits == 1 ? 0 : (size_t)g.splits * g.col_blocks * 64 * 64 * sizeof(float);
+    const q4::GradPlan g = q4::plan_grad(M, C);
+    return g.splits == 1 ? 0 : (size_t)g.splits * g.col_blocks * R * q4::kG2Cols * sizeof(float);
 }
 
 static q4::GradProb make_grad_prob(const void* P, const void* in, float* out, int o_sr, int o_sc, int M, int C, int R,
                                    float* part, const q4::DropArgs* drop = nullptr) {
-    const q4::GradPlan g = q4::plan_grad(M, C, R);
+    const q4::GradPlan g = q4::plan_grad(M, C);
     q4::GradProb q;
     q.P = reinterpret_cast<const q4::half_t*>(P);
     q.in = reinterpret_cast<const q4::half_t*>(in);
@@ -530,22 +529,24 @@ static q4::GradProb make_grad_prob(const void* P, const void* in, float* out, in
 static int launch_grad(const q4::GradArgs& ga, int nprob, int R, hipStream_t stream) {
     using namespace q4;
     int gx = 0, gy = 0, rx = 0;
-    bool any_split = false;
+    bool any_split = false, any_drop = false;
     for (int i = 0; i < nprob; ++i) {
         gx = ga.p[i].col_blocks > gx ? ga.p[i].col_blocks : gx;
         gy = ga.p[i].splits > gy ? ga.p[i].splits : gy;
-        const int rb = (ga.p[i].col_blocks * 64 * 64 + 255) / 256;
+        const int rb = (ga.p[i].col_blocks * R * kG2Cols + 255) / 256;
         rx = rb > rx ? rb : rx;
         any_split = any_split || ga.p[i].splits > 1;
+        any_drop = any_drop || ga.p[i].drop.thr15 != 0;
     }
-    const dim3 grid(gx, gy, nprob), block(64 * kGradWaves);
-    if (R == 8) {
-        hipLaunchKernelGGL(lora_grad_kernel<8>, grid, block, 0, stream, ga);
-        if (any_split) hipLaunchKernelGGL(lora_grad_reduce_kernel<8>, dim3(rx, nprob), dim3(256), 0, stream, ga);
+    const dim3 grid(gx, gy, nprob), block(64 * kG2Waves);
+    if (R <= 16) {
+        if (any_drop) hipLaunchKernelGGL((lora_grad_kernel<true, 1>), grid, block, 0, stream, ga, R);
+        else hipLaunchKernelGGL((lora_grad_kernel<false, 1>), grid, block, 0, stream, ga, R);
     } else {
-        hipLaunchKernelGGL(lora_grad_kernel<16>, grid, block, 0, stream, ga);
-        if (any_split) hipLaunchKernelGGL(lora_grad_reduce_kernel<16>, dim3(rx, nprob), dim3(256), 0, stream, ga);
+        if (any_drop) hipLaunchKernelGGL((lora_grad_kernel<true, 2>), grid, block, 0, stream, ga, R);
+        else hipLaunchKernelGGL((lora_grad_kernel<false, 2>), grid, block, 0, stream, ga, R);
     }
+    if (any_split) hipLaunchKernelGGL(lora_grad_reduce_kernel, dim3(rx, nprob), dim3(256), 0, stream, ga, R);
     return hipGetLastError() == hipSuccess ? 0 : -4;
 }
 

@@ -690,7 +690,7 @@ def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=Non
     return out
 
 
-LORA_GRAD_RANKS = (8, 16)
+LORA_GRAD_RANKS = tuple(range(2, 33, 2))
 
 
 def lora_down(inp, w, dropout=None):
@@ -729,7 +729,7 @@ def lora_grad(p, inp, alpha, transposed=False, dropout=None):
              and inp.shape[0] == p.shape[0], "inp must be a contiguous float16 [M, C] tensor on the same device")
     M, R = p.shape
     C = inp.shape[1]
-    _require(R in LORA_GRAD_RANKS and C % 8 == 0, "lora_grad needs R in (8, 16) and C % 8 == 0")
+    _require(R in LORA_GRAD_RANKS and C % 8 == 0, "lora_grad needs an even R in 2..32 and C % 8 == 0")
     dev = p.device
     if M == 0:                                               # empty batch: the gradient is zero
         return torch.zeros((C, R) if transposed else (R, C), dtype=torch.float32, device=dev)
@@ -766,7 +766,7 @@ def lora_grad_pair(p1, inp1, p2, inp2, alpha, dropout=None, outs=None):
     _require(p1.shape == p2.shape and p1.device == p2.device, "the two rank-R operands must share shape and device")
     M, R = p1.shape
     C1, C2 = inp1.shape[1], inp2.shape[1]
-    _require(R in LORA_GRAD_RANKS and C1 % 8 == 0 and C2 % 8 == 0, "lora_grad needs R in (8, 16) and C % 8 == 0")
+    _require(R in LORA_GRAD_RANKS and C1 % 8 == 0 and C2 % 8 == 0, "lora_grad needs an even R in 2..32 and C % 8 == 0")
     dev = p1.device
     if M == 0:
         return (torch.zeros((R, C1), dtype=torch.float32, device=dev), torch.zeros((C2, R), dtype=torch.float32, device=dev))

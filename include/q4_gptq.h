@@ -207,7 +207,7 @@ int q4_lora_down_f16(const void *in, const void *w, int w_sr, int w_sc, int w_is
 /* Gradient of an adapter matrix:  out fp32 [j*o_sr + c*o_sc] = alpha * sum_m p[m, j] * in[m, c]
  * with p fp16 [M, R] and in fp16 [M, C]:  dA = scaling * dyb^T @ x (out = [R, K], o_sr = K, o_sc = 1) and
  * dB = scaling * dy^T @ xa (out = lora_B.weight.grad [N, R], o_sr = 1, o_sc = R) -- what torch autograd
- * computes for the two adapter Linears of models.py:66.  R is 8 or 16, C % 8 == 0.
+ * computes for the two adapter Linears of models.py:66.  R even, 2 <= R <= 32; C % 8 == 0.
  * `workspace`: q4_lora_grad_workspace_bytes(M, C, R) bytes (0 for small M: then it may be NULL), 256-byte
  * aligned, contents irrelevant before and after the call: it carries fp32 partial sums of row blocks,
  * which a second kernel adds in a fixed order (bit-reproducible).  With `drop`, `in` is replaced by dropout(in)
@@ -219,8 +219,7 @@ int q4_lora_grad_f32(const void *p, const void *in, float *out, int o_sr, int o_
 
 /* Both adapter gradients of a layer in one launch (plus one for the two reductions): problem 1 and problem 2 as
  * for q4_lora_grad_f32, sharing M, R and alpha -- dA from (dyb, x, C1 = K) and dB from (xa, dy, C2 = N) in the
- * backward of models.py:66.  A single gradient is bound by the latency of its one burst of loads, so the pair
- * costs little more than one.  `workspace`: q4_lora_grad_workspace_bytes(M, C1, R) +
+ * backward of models.py:66.  `workspace`: q4_lora_grad_workspace_bytes(M, C1, R) +
  * q4_lora_grad_workspace_bytes(M, C2, R) bytes, 256-byte aligned, contents irrelevant.  `drop1` applies to in1 only
  * (x in dA; xa in dB already carries the mask). */
 int q4_lora_grad_pair_f32(const void *p1, const void *in1, float *out1, int o1_sr, int o1_sc, int C1,

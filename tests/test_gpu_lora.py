@@ -42,7 +42,8 @@ def test_lora_down_both_layouts(M, C, R, wdtype):
 
 
 @pytest.mark.parametrize("M,C,R", [(2048, 4096, 8), (2048, 11008, 8), (2048, 4096, 16), (77, 64, 8),
-                                   (1, 8, 16), (1000, 520, 8), (5000, 128, 16)])
+                                   (1, 8, 16), (1000, 520, 8), (5000, 128, 16), (513, 4096, 4), (300, 264, 2),
+                                   (1024, 4096, 32), (129, 136, 24), (40000, 128, 12)])
 def test_lora_grad_matches_fp32_product(M, C, R):
     from alpaca_lora_4bit_amd import quant_hip
     rng = np.random.default_rng(M + C * 3 + R)
@@ -110,7 +111,8 @@ def test_fused_lora_function_against_oracle_fp32_adapters(oracle):
     assert Ad.grad.dtype == torch.float32 and Bd.grad.dtype == torch.float32
 
 
-@pytest.mark.parametrize("M,C1,C2,R", [(2048, 4096, 4096, 8), (300, 1408, 512, 16), (50, 512, 11008, 8), (1000, 11008, 4096, 16)])
+@pytest.mark.parametrize("M,C1,C2,R", [(2048, 4096, 4096, 8), (300, 1408, 512, 16), (50, 512, 11008, 8), (1000, 11008, 4096, 16),
+                                       (700, 4096, 1024, 32), (2048, 128, 4096, 6)])
 def test_lora_grad_pair_equals_the_two_single_launches(M, C1, C2, R):
     """Both gradients in one launch (different column counts, hence different grids and split counts) give the
     bits of the two separate launches."""
