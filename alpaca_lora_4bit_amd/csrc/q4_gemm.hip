@@ -724,6 +724,10 @@ int q4_skinny_applicable(int M, int K, int N, int groupsize, int has_gidx);
 size_t q4_skinny_workspace(int M, int K, int N);
 int q4_launch_skinny(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales, int groupsize,
                      const void* bias, void* y, int M, int K, int N, int G, void* workspace, hipStream_t stream);
+int q4_skinny_dx_applicable(int M, int K, int N, int groupsize, int has_gidx);
+size_t q4_skinny_dx_workspace(int M, int K, int N);
+int q4_launch_skinny_dx(const void* dy, const int32_t* qweight, const int32_t* qzeros, const void* scales, int groupsize,
+                        void* dx, int M, int K, int N, int G, void* workspace, hipStream_t stream);
 }
 
 extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, const int32_t* qzeros,
@@ -756,6 +760,10 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     if (fwd && a.R == 0 && q4_skinny_applicable(M, K, N, groupsize, gidx) && workspace &&
         workspace_bytes >= q4_skinny_workspace(M, K, N))
         return q4_launch_skinny(act, qweight, qzeros, scales, groupsize, bias, out, M, K, N, G, workspace, stream);
+    // 17..48 rows, grad-input, no adapter: its transposed counterpart
+    if (!fwd && a.R == 0 && q4_skinny_dx_applicable(M, K, N, groupsize, gidx) && workspace &&
+        workspace_bytes >= q4_skinny_dx_workspace(M, K, N))
+        return q4_launch_skinny_dx(act, qweight, qzeros, scales, groupsize, out, M, K, N, G, workspace, stream);
     // tile configuration: 256-row tiles once they still give every CU a workgroup; split-K for few tiles
     const GemmPlan p = plan_gemm(M, fwd ? K : N, nout, workspace ? workspace_bytes : 0);
     a.part = reinterpret_cast<float*>(workspace);
@@ -774,6 +782,10 @@ extern "C" size_t q4_gemm_plan_workspace(int fwd, int M, int K, int N) {
     if (p.tail_cols > 0) need = (size_t)p.tail_splits * (size_t)M * (size_t)p.tail_cols * BN * sizeof(float);
     if (fwd && M > 16 && M <= 64) {               // the skinny kernel's partial rows (it may or may not apply)
         const size_t sk = q4_skinny_workspace(M, K, N);
+        if (sk > need) need = sk;
+    }
+    if (!fwd && M > 16 && M <= 48) {
+        const size_t sk = q4_skinny_dx_workspace(M, K, N);
         if (sk > need) need = sk;
     }
     return need;

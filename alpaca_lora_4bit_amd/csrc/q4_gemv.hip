@@ -3,6 +3,7 @@
 //   gemv_seq_perm_kernel  1 <= M <= 4, act-order layer with rows sorted by group: gathers x through the permutation
 //   gemv_gidx_kernel      1 <= M <= 16, act-order with per-row groups read through g_idx
 //   skinny_seq_kernel     17 <= M <= 64, sequential groups (fp32 partial rows + ordered reduction)
+//   skinny_dx_kernel      17 <= M <= 48, the transposed product dy @ W^T (grad-input), sequential groups
 //
 // Work split.  A workgroup owns a strip of 64 columns; its W wavefronts (W = blockDim.x / 64)
 // take consecutive chunks of 32*NSTEP rows, and gridDim.y workgroups share one strip when K is
@@ -37,6 +38,7 @@
 // memory round trip, with no fences and no spinning.
 #include "q4_common.hpp"
 #include <stdlib.h>
+#include <type_traits>
 
 namespace q4 {
 
@@ -609,6 +611,228 @@ void skinny_seq_kernel(SkinnyArgs a) {
     }
 }
 
+// ------------------------------------------------------------------ grad-input, 17 <= M <= 48 (sequential groups)
+// dx[M, K] = dy[M, N] @ W^T with the same streaming scheme: the reduction runs over the columns n of W, the outputs
+// are its rows k.  A packed word holds 8 consecutive rows k of one column n, so the 8 words of columns n .. n+7
+// (two 128-bit loads of lane (i = l % 16, kk = l / 16): word-row k8 + i, columns n0 + 32*t + 8*kk .. + 7) hold an
+// 8 x 8 block of codes, and nibble j of those 8 words is exactly the 8-deep slice of the reduction that lane l
+// feeds to MFMA j as B operand for output row 8*(k8 + i) + j: eight MFMAs per step of 32 columns produce 16
+// word-rows = 128 outputs, one quantization group when groupsize % 128 == 0.  Within a group the scale and the zero
+// depend on n only, so they move to the A side:
+//   dx[m, k] = sum_n (dy[m, n] * s[g, n]) * (1024 + q[k, n])  -  sum_n (dy[m, n] * s[g, n]) * (1025 + z[g, n])
+// (codes enter as fp16 1024 + q by OR-ing them into the mantissa; the second sum is one more MFMA per step whose
+// B operand is the same for all columns).  A wavefront owns one chunk of 128 columns n: it keeps that chunk of
+// all dy rows as A operands in registers and walks over `strips_per_wg` neighbouring output blocks of 128 rows k,
+// the words of the next two steps in flight while it multiplies.  The eight wavefronts of a workgroup (eight
+// chunks) are summed through LDS, 64 outputs at a time; the gridDim.y workgroups of a block leave fp32 partial rows
+// [gridDim.y][M][K] that gemm_splitk_reduce_kernel adds in order (bit-reproducible).
+// Mathematically sum_n dy * W[k, n] (src/alpaca_lora_4bit/autograd_4bit.py:45-54 through
+// matmul_utils_4bit.py:125-126); the scale is applied to dy before the product instead of to the weight, within
+// the tolerance of the path.
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for_dx(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for_dx<I + 1, N>(f);
+    }
+}
+
+struct SkinnyDxArgs {
+    const half_t* dy;
+    const uint32_t* qweight;
+    const uint32_t* qzeros;
+    const half_t* scales;
+    int groupsize;
+    half_t* dx;               // written directly when gridDim.y == 1
+    float* part;              // [gridDim.y][M][K]
+    int M, K, N, G;
+    int strips_per_wg;
+};
+
+template <int RB, int SS>      // SS: steps of 32 columns per pipeline stage (2; 1 where registers are short)
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2)))
+void skinny_dx_kernel(SkinnyDxArgs a) {
+    constexpr int NSTEP = 4, NW = 8, NH = NSTEP / SS;
+    constexpr int kFar = 0x70000000;
+    __shared__ __attribute__((aligned(16))) float red[RB][NW][16 * 64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kk = lane >> 4, c = lane & 15;
+    const int nblocks = a.K >> 7;
+    const int strip0 = blockIdx.x * a.strips_per_wg;
+    const int nl = min(a.strips_per_wg, nblocks - strip0);
+    const int n0 = (blockIdx.y * NW + wave) * 128;
+    const int dead = n0 < a.N ? 0 : kFar;          // wave-uniform
+    const int S = gridDim.y;
+    const int G = a.G;
+
+    const rsrc_t rw = make_rsrc(a.qweight, (unsigned)((size_t)(a.K >> 3) * a.N * 4));
+    const rsrc_t rs = make_rsrc(a.scales, (unsigned)((size_t)G * a.N * 2));
+    const rsrc_t rz = make_rsrc(a.qzeros, (unsigned)((size_t)G * (a.N >> 3) * 4));
+    const rsrc_t rdy = make_rsrc(a.dy, (unsigned)((size_t)a.M * a.N * 2));
+    const int vw = dead ? 0 : (c * a.N + n0 + 8 * kk) * 4;
+    const int vs = dead ? 0 : (n0 + 8 * kk) * 2;
+    const int vz = dead ? 0 : ((n0 >> 3) + kk) * 4;
+    const int wblock = 16 * a.N * 4;               // bytes between two output blocks (16 word-rows)
+
+    // the chunk of dy as A operands: row-contiguous loads turned through this wavefront's own LDS (as in
+    // skinny_seq_kernel); natural order, unit (4t + kk) of row c = dy[c][n0 + 32t + 8kk .. + 7]
+    half8_t av[RB][NSTEP];
+    {
+        uint4_t xv[RB][NSTEP];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int i = 0; i < NSTEP; ++i) {
+                const int vx = (min(16 * rb + 4 * i + kk, a.M - 1) * a.N + 8 * c) * 2;
+                xv[rb][i] = buf_load128(rdy, vx, dead + n0 * 2);
+            }
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            uint4_t* stage = reinterpret_cast<uint4_t*>(&red[rb][wave][0]);
+#pragma unroll
+            for (int i = 0; i < NSTEP; ++i) stage[(4 * i + kk) * 16 + (c ^ (4 * i + kk))] = xv[rb][i];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const uint4_t* stage = reinterpret_cast<const uint4_t*>(&red[rb][wave][0]);
+#pragma unroll
+            for (int t = 0; t < NSTEP; ++t) av[rb][t] = __builtin_bit_cast(half8_t, stage[c * 16 + ((4 * t + kk) ^ c)]);
+        }
+    }
+    __syncthreads();                               // red is reused by the sums below
+
+    // one pipeline stage = SS steps of one output block
+    struct Stage { uint4_t w[SS][2]; uint4_t s[SS]; uint32_t z[SS]; };
+    auto load_stage = [&](Stage& st, int it) {     // it = NH * block + part, beyond the end: no traffic
+        const int l = it / NH, h = it % NH;
+        const int off = (dead || l >= nl) ? kFar : 0;
+        const int blk = strip0 + l;
+        const int g = off ? 0 : (blk << 7) / a.groupsize;
+#pragma unroll
+        for (int u = 0; u < SS; ++u) {
+            const int t = SS * h + u;
+            st.s[u] = buf_load128(rs, vs, off + g * a.N * 2 + t * 64);
+            st.z[u] = buf_load32(rz, vz, off + g * (a.N >> 3) * 4 + t * 16);
+        }
+#pragma unroll
+        for (int u = 0; u < SS; ++u) {
+            const int t = SS * h + u;
+            st.w[u][0] = buf_load128(rw, vw, off + blk * wblock + t * 128);
+            st.w[u][1] = buf_load128(rw, vw, off + blk * wblock + t * 128 + 16);
+        }
+    };
+
+    float4_t acc[RB][8], corr[RB];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            corr[rb] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[rb][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    auto multiply = [&](const Stage& st, auto htag) {
+        constexpr int h = decltype(htag)::value;
+#pragma unroll
+        for (int u = 0; u < SS; ++u) {
+            constexpr int tbase = SS * h;
+            const half8_t s8 = __builtin_bit_cast(half8_t, st.s[u]);
+            half8_t as[RB];
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) as[rb] = av[rb][tbase + u] * s8;
+            // B operand of the zero term: 1025 + z for this lane's eight columns
+            const uint32_t zlo = st.z[u] & 0x0F0F0F0Fu, zhi = (st.z[u] >> 4) & 0x0F0F0F0Fu;
+            const half2_t one2 = {(half_t)1.f, (half_t)1.f};
+            uint32_t zb[4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p)
+                zb[p] = as_u32(as_half2(__builtin_amdgcn_perm(zhi, zlo, 0x0c040c00u + 0x00010001u * p) | kMagic) + one2);
+            const half8_t zB = make_half8(zb[0], zb[1], zb[2], zb[3]);
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) corr[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as[rb], zB, corr[rb], 0, 0, 0);
+            // code operands: byte b of a word holds the codes of rows 2b (low nibble) and 2b + 1
+            const uint32_t wd[8] = {st.w[u][0].x, st.w[u][0].y, st.w[u][0].z, st.w[u][0].w,
+                                    st.w[u][1].x, st.w[u][1].y, st.w[u][1].z, st.w[u][1].w};
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                uint32_t ev[4], od[4];
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    const uint32_t sel = 0x0c000c00u | ((4u + b) << 16) | (uint32_t)b;
+                    const uint32_t pb = __builtin_amdgcn_perm(wd[2 * p + 1], wd[2 * p], sel);   // byte b of columns 2p, 2p+1
+                    ev[p] = (pb & 0x000F000Fu) | kMagic;
+                    od[p] = ((pb >> 4) & 0x000F000Fu) | kMagic;
+                }
+                const half8_t be = make_half8(ev[0], ev[1], ev[2], ev[3]), bo = make_half8(od[0], od[1], od[2], od[3]);
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) {
+                    acc[rb][2 * b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as[rb], be, acc[rb][2 * b], 0, 0, 0);
+                    acc[rb][2 * b + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as[rb], bo, acc[rb][2 * b + 1], 0, 0, 0);
+                }
+            }
+        }
+    };
+    // sums 64 outputs of the block over the wavefronts: local column lc = 4c + jj stands for output
+    // 128*blk + 8*(lc / 4) + 4*hf + lc % 4; acc[rb][4*hf + jj][r] is row 16*rb + 4*kk + r
+    auto finish_half = [&](int blk, int hf) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float4_t v;
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) v[jj] = acc[rb][4 * hf + jj][r] - corr[rb][r];
+                *reinterpret_cast<float4_t*>(&red[rb][wave][((4 * kk + r) << 6) + 4 * c]) = v;
+            }
+        __syncthreads();
+        {
+            const int e = 2 * threadIdx.x;
+            const int row = e >> 6, lc = e & 63;
+            const int cc = (blk << 7) + 8 * (lc >> 2) + 4 * hf + (lc & 3);
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) {
+                    const float* rp = &red[rb][w][e];
+                    v0 += rp[0];
+                    v1 += rp[1];
+                }
+                const int m = 16 * rb + row;
+                if (m < a.M) {
+                    if (S == 1) {
+                        const half2_t hv = {(half_t)v0, (half_t)v1};
+                        *reinterpret_cast<half2_t*>(a.dx + (size_t)m * a.K + cc) = hv;
+                    } else {
+                        float* pp = a.part + ((size_t)blockIdx.y * a.M + m) * a.K + cc;
+                        pp[0] = v0;
+                        pp[1] = v1;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    };
+
+    Stage buf[2];
+    load_stage(buf[0], 0);
+    for (int l = 0; l < nl; ++l) {
+        clear_acc();
+        static_for_dx<0, NH>([&](auto hc) {
+            constexpr int h = decltype(hc)::value;
+            load_stage(buf[(h + 1) & 1], NH * l + h + 1);      // NH is even: stage NH*l + h sits in buf[h & 1]
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(buf[h & 1], hc);
+        });
+        finish_half(strip0 + l, 0);
+        finish_half(strip0 + l, 1);
+    }
+}
+
 // ------------------------------------------------------------------ act-order (per-row groups)
 template <int NSTEP>
 __global__ __launch_bounds__(512) void gemv_gidx_kernel(GemvArgs a) {
@@ -941,6 +1165,50 @@ extern "C" int q4_launch_skinny(const void* x, const int32_t* qweight, const int
     else hipLaunchKernelGGL(skinny_seq_kernel<4>, grid, block, 0, stream, a);
     if (hipGetLastError() != hipSuccess) return -4;
     if (S > 1) return q4_launch_splitk_reduce(a.part, y, (long)M * N, S, stream);
+    return 0;
+}
+
+// Shapes the streaming grad-input kernel takes: 17..48 rows, sequential groups that are multiples of 128 rows.
+extern "C" int q4_skinny_dx_applicable(int M, int K, int N, int groupsize, int has_gidx) {
+    static const int max_rows = getenv("Q4_SKINNY_DX_MAX_ROWS") ? atoi(getenv("Q4_SKINNY_DX_MAX_ROWS")) : 48;
+    return M > 16 && M <= max_rows && M <= 48 && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 &&
+           N % 128 == 0;
+}
+
+static int skinny_dx_splits(int N) {
+    return (N / 128 + 7) / 8;                     // 8 wavefronts per workgroup, one chunk of 128 columns each
+}
+
+extern "C" size_t q4_skinny_dx_workspace(int M, int K, int N) {
+    const int S = skinny_dx_splits(N);
+    return S > 1 ? (size_t)S * (size_t)M * (size_t)K * sizeof(float) : 0;
+}
+
+extern "C" int q4_launch_skinny_dx(const void* dy, const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                                   int groupsize, void* dx, int M, int K, int N, int G, void* workspace,
+                                   hipStream_t stream) {
+    using namespace q4;
+    SkinnyDxArgs a;
+    a.dy = reinterpret_cast<const half_t*>(dy);
+    a.qweight = reinterpret_cast<const uint32_t*>(qweight);
+    a.qzeros = reinterpret_cast<const uint32_t*>(qzeros);
+    a.scales = reinterpret_cast<const half_t*>(scales);
+    a.groupsize = groupsize;
+    a.dx = reinterpret_cast<half_t*>(dx);
+    a.part = reinterpret_cast<float*>(workspace);
+    a.M = M; a.K = K; a.N = N; a.G = G;
+    const int S = skinny_dx_splits(N);
+    const int blocks = K / 128;
+    static const int force_l = getenv("Q4_SKINNY_DX_STRIPS") ? atoi(getenv("Q4_SKINNY_DX_STRIPS")) : 0;
+    const int slots = 256;                        // one workgroup per compute unit (register budget)
+    int L = force_l > 0 ? force_l : (blocks * S + slots - 1) / slots;
+    L = L < 1 ? 1 : (L > 4 ? 4 : L);
+    a.strips_per_wg = L;
+    const dim3 grid((blocks + L - 1) / L, S), block(512);     // wavefronts past the end of N read zeros
+    if (M <= 32) hipLaunchKernelGGL((skinny_dx_kernel<2, 2>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((skinny_dx_kernel<3, 1>), grid, block, 0, stream, a);   // a fourth row block would not fit the registers
+    if (hipGetLastError() != hipSuccess) return -4;
+    if (S > 1) return q4_launch_splitk_reduce(a.part, dx, (long)M * K, S, stream);
     return 0;
 }
 

@@ -47,6 +47,29 @@ def test_gemm_backward_dx(oracle, K, N, gs, act, M):
     assert rel_err(dx.cpu().numpy(), ref) <= 2e-3
 
 
+@pytest.mark.parametrize("K,N,gs", [(4096, 11008, 128), (11008, 4096, 128), (4096, 4096, 256), (1408, 384, 256), (128, 128, 128)])
+@pytest.mark.parametrize("M", [17, 24, 32, 33, 48])
+def test_streaming_grad_input_17_to_48_rows(oracle, K, N, gs, M):
+    """The weight-streaming grad-input kernel (17..48 rows, sequential groups of a multiple of 128 rows) against the
+    float64 product of dy with the bit-exact dense W, and against the tiled kernel that takes 49 rows and more."""
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    layer = oracle.make_layer(K, N, gs, act_order=False, seed=K + N + M)
+    t = to_cuda_layer(layer)
+    dy = _t(oracle.make_activations(M, N, seed=M + 9))
+    W = quant_hip.dequant(t["qweight"], t["qzeros"], t["scales"], t["g_idx"], gs)
+    ref = dy.double() @ W.double().t()
+    dx = quant_hip.gemm_bwd_dx(dy, t["qweight"], t["qzeros"], t["scales"], None, gs)
+    assert dx.shape == (M, K)
+    err = float((dx.double() - ref).abs().max() / ref.abs().max())
+    assert err <= TOL and err <= 2e-3, err
+    again = quant_hip.gemm_bwd_dx(dy, t["qweight"], t["qzeros"], t["scales"], None, gs)
+    assert torch.equal(dx, again)                                   # ordered partial sums: bit-reproducible
+    big = torch.cat([dy, torch.zeros(49 - M, N, dtype=dy.dtype, device=dy.device)])     # 49 rows: the tiled kernel
+    tiled = quant_hip.gemm_bwd_dx(big, t["qweight"], t["qzeros"], t["scales"], None, gs)[:M]
+    assert float((dx.float() - tiled.float()).abs().max() / ref.abs().max()) <= 2e-3
+
+
 def test_gemm_equals_dense_matmul_of_dequantized_weight(oracle):
     """The fused kernels hold the same fp16 W in LDS that the dense dequant writes: against
     torch.matmul(x, W_hip) the only difference is fp32 summation order."""
