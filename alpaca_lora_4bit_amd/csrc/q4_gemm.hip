@@ -55,7 +55,7 @@ struct GemmArgs {
     int R;
     half_t* out;              // fwd: y [M,N]      bwd: dx [M,K]
     int M, K, N, G;
-    int phase_step;           // rotation of the reduction loop per row tile, in steps of 64
+    int phase_step;           // bits 0-7: rotation of the reduction loop per row tile, in steps of 64; bits 8+: row tiles per group of the tile order
     float* part;              // split-K: fp32 partial outputs [gridDim.z][M][part_cols] (gridDim.z > 1 only)
     int col_tile0;            // first column tile of this launch (a launch may cover a range of column tiles)
     int part_cols;            // columns held by `part`: those of this launch's column tiles
@@ -64,9 +64,11 @@ struct GemmArgs {
 
 // Which output tile a workgroup computes, and where in the reduction it starts.
 //  * Workgroups are handed to the 8 XCDs round-robin in dispatch order.  The ids are permuted so that one
-//    XCD owns a contiguous range of tiles in column-major order: a few column tiles for all row tiles.
-//    Its L2 then holds few columns of W, spread over several L2 channels, and each slab of activations
-//    is fetched once per XCD and shared by its column tiles.
+//    XCD owns a contiguous range of tiles, ordered in groups of `rg` row tiles: all column tiles of a group,
+//    then the next group.  The 32 workgroups an XCD runs at a time then share 2 slabs of activations and 16
+//    column tiles of W (about 4 MB each at K = 4096, what its L2 holds) instead of every row tile of a few
+//    columns: with many row tiles the activations would otherwise stream from HBM once per column tile
+//    (8192 x 4096 x 4096: 306 -> 260 us; no shape slower).
 //  * Activation rows of a power-of-two pitch (K = 4096: 8 KB) put one reduction slab of ALL rows into
 //    a single L2 channel; workgroups marching through the reduction in lockstep then queue on that one
 //    channel.  Row tile r therefore starts its (cyclic) reduction loop phase_step * r steps later.
@@ -78,8 +80,19 @@ __device__ __forceinline__ TileMap map_tile(int phase_step, int nsteps, int col_
     int id = blockIdx.y * nc + blockIdx.x;
     if (total % 8 == 0) id = (id % 8) * (total / 8) + id / 8;
     TileMap m;
-    m.tile_c = id / nr;
-    m.tile_r = id - m.tile_c * nr;
+    const int rg = phase_step >> 8;                   // row tiles per group (0: column-major over all row tiles)
+    phase_step &= 0xff;
+    const int grouped = rg > 0 ? (nr / rg) * rg * nc : 0;
+    if (id < grouped) {
+        // groups of rg row tiles: all column tiles of a group, then the next group
+        const int gi = id / (rg * nc), rem = id - gi * rg * nc;
+        m.tile_c = rem / rg;
+        m.tile_r = gi * rg + (rem - m.tile_c * rg);
+    } else {
+        const int left = rg > 0 ? nr % rg : nr, base = nr - left, rem = id - grouped;
+        m.tile_c = rem / left;
+        m.tile_r = base + (rem - m.tile_c * left);
+    }
     m.tile_c += col_tile0;
     m.phase = (m.tile_r * phase_step) % nsteps;
     return m;
@@ -754,6 +767,8 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     a.M = M; a.K = K; a.N = N; a.G = G;
     static const int env_phase = getenv("Q4_GEMM_PHASE") ? atoi(getenv("Q4_GEMM_PHASE")) : 2;
     a.phase_step = env_phase < 0 ? 0 : env_phase;
+    static const int env_order = getenv("Q4_GEMM_ORDER") ? atoi(getenv("Q4_GEMM_ORDER")) : 2;   // row tiles per group
+    if (env_order > 0) a.phase_step |= (env_order > 64 ? 64 : env_order) << 8;
     const int nout = fwd ? N : K;
     const bool gidx = g_idx != nullptr;
     // 17..64 rows, forward, no adapter: the weight-streaming kernel (one pass over the packed weights)
