@@ -188,8 +188,18 @@ struct FwdSlab {
     __device__ __forceinline__ void load(const GemmArgs& a, const SlabRsrc& r, int, int kred0) {
         static_for<0, kLoads>([&](auto ic) { load_part<decltype(ic)::value>(a, r, kred0); });
     }
+    // what the slices of a step need of (scale, zero) of the step's group, computed once per group change
+    struct Prep { half2_t s2, zero2, s1024; };
+    __device__ __forceinline__ Prep make_prep(int n0) const {
+        Prep pr;
+        pr.s2 = as_half2(s_raw | (s_raw << 16));
+        const uint32_t z_cur = (z_raw >> (((n0 + col) & 7) * 4)) & 0xFu;
+        pr.zero2 = zero_term(pr.s2, z_cur, z_cur);
+        pr.s1024 = pr.s2 * half2_t{(half_t)1024.f, (half_t)1024.f};
+        return pr;
+    }
     template <int I>
-    __device__ __forceinline__ void store_slice(const GemmArgs& a, int n0, int kred0, half_t* sB) {
+    __device__ __forceinline__ void store_slice(const GemmArgs& a, int n0, int kred0, half_t* sB, const Prep& pr) {
         const int n = n0 + col;
         if constexpr (GIDX) {
             if constexpr (I == 0) {
@@ -216,18 +226,15 @@ struct FwdSlab {
             }
         } else {
             constexpr int i = I / 4, p = I % 4;
-            const half2_t s2 = as_half2(s_raw | (s_raw << 16));
-            const uint32_t z_cur = (z_raw >> ((n & 7) * 4)) & 0xFu;
-            const half2_t zero2 = zero_term(s2, z_cur, z_cur);
-            const half2_t s1024 = s2 * half2_t{(half_t)1024.f, (half_t)1024.f};
             const uint32_t lo = w[i] & 0x0F0F0F0Fu;          // bytes e0 e2 e4 e6
             const uint32_t hi = (w[i] >> 4) & 0x0F0F0F0Fu;   // bytes e1 e3 e5 e7
             const uint32_t codes = __builtin_amdgcn_perm(hi, lo, 0x0c040c00u + 0x00010001u * p) | kMagic;
-            o[p] = as_u32(dequant_pair_magic(codes, s2, s1024, zero2));
+            o[p] = as_u32(dequant_pair_magic(codes, pr.s2, pr.s1024, pr.zero2));
             if constexpr (p == 3)
                 *reinterpret_cast<uint4_t*>(sB + col * LDS_STRIDE + 8 * (wr0 + WSTEP * i)) = uint4_t{o[0], o[1], o[2], o[3]};
         }
     }
+    __device__ __forceinline__ void fetch_tab(const unsigned char*, int) {}
     // LoRA step: B operand = adapter matrix [R, N]; LDS row = column n, minor = r (zero padded to 64).
     __device__ __forceinline__ void store_lora(const GemmArgs& a, int n0, half_t* sB, int t) const {
         for (int idx = t; idx < BN * BK; idx += NT) {
@@ -244,13 +251,17 @@ struct FwdSlab {
 // With 512 threads two threads share a load and split the word-row's 8 rows 4 + 4.
 // Piece I dequantizes columns (0,1) [I even] or (2,3) [I odd] of the thread's row I/2; the
 // 8-byte row segment goes to LDS with the odd piece.
-template <bool GIDX, int NT>
+// TAB: the scales and the zero terms rn16(s * (z + 1)) of the tile's group sit in an LDS table for every column n,
+// per column pair as (s_a, s_b, zero_a, zero_b) (filled once per workgroup), and come from there: one 16-byte LDS
+// read per step instead of two more global loads and the zero-term arithmetic of every step.
+template <bool GIDX, int NT, bool TAB = false>
 struct BwdSlab {
     static constexpr int RPT = 8 * 256 / NT;      // rows of the word-row handled by one thread (8 or 4)
     static constexpr int kSlices = 2 * RPT;
     uint4_t w;
     uint2_t sv;
     uint32_t zw, o01;
+    uint4_t tv;                                   // TAB: (s01, zero01, s23, zero23) of this thread's four columns
     int wr, n4, e0;
     int voff_w, voff_s, voff_z;
     __device__ __forceinline__ void init(int t, const GemmArgs& a, int kout0) {
@@ -260,7 +271,12 @@ struct BwdSlab {
         voff_s = (g * a.N + 4 * n4) * 2;
         voff_z = (g * (a.N >> 3) + (n4 >> 1)) * 4;
     }
-    static constexpr int kLoads = GIDX ? 1 : 3;
+    static constexpr int kLoads = (GIDX || TAB) ? 1 : 3;
+    __device__ __forceinline__ void fetch_tab(const unsigned char* tab, int nred0) {
+        tv = *reinterpret_cast<const uint4_t*>(tab + (nred0 + 4 * n4) * 4);
+    }
+    struct Prep {};
+    __device__ __forceinline__ Prep make_prep(int) const { return Prep{}; }
     template <int I>
     __device__ __forceinline__ void load_part(const GemmArgs&, const SlabRsrc& r, int nred0) {
         if constexpr (I == 0) w = buf_load128(r.w, voff_w, nred0 * 4);
@@ -271,7 +287,7 @@ struct BwdSlab {
         static_for<0, kLoads>([&](auto ic) { load_part<decltype(ic)::value>(a, r, nred0); });
     }
     template <int I>
-    __device__ __forceinline__ void store_slice(const GemmArgs& a, int kout0, int nred0, half_t* sB) {
+    __device__ __forceinline__ void store_slice(const GemmArgs& a, int kout0, int nred0, half_t* sB, const Prep&) {
         const int n = nred0 + 4 * n4;
         const int zsh = (n4 & 1) * 16;
         const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
@@ -312,8 +328,14 @@ struct BwdSlab {
             const uint32_t na = (el & 1) ? ((wa >> 4) & 0x0F0F0F0Fu) : (wa & 0x0F0F0F0Fu);
             const uint32_t nb = (el & 1) ? ((wb >> 4) & 0x0F0F0F0Fu) : (wb & 0x0F0F0F0Fu);
             const uint32_t codes = __builtin_amdgcn_perm(nb, na, sel) | kMagic;  // (code of column a, of column b) of row e
-            const half2_t s2 = as_half2(h ? sv.y : sv.x);
-            const half2_t zero2 = zero_term(s2, (z4 >> (8 * h)) & 0xFu, (z4 >> (8 * h + 4)) & 0xFu);
+            half2_t s2, zero2;
+            if constexpr (TAB) {
+                s2 = as_half2(h ? tv.z : tv.x);
+                zero2 = as_half2(h ? tv.w : tv.y);
+            } else {
+                s2 = as_half2(h ? sv.y : sv.x);
+                zero2 = zero_term(s2, (z4 >> (8 * h)) & 0xFu, (z4 >> (8 * h + 4)) & 0xFu);
+            }
             const uint32_t r = as_u32(dequant_pair_magic(codes, s2, s2 * k1024, zero2));
             if constexpr (h == 0) o01 = r;
             else *reinterpret_cast<uint2_t*>(sB + (8 * wr + e) * LDS_STRIDE + 4 * n4) = uint2_t{o01, r};
@@ -331,8 +353,17 @@ struct BwdSlab {
 
 // FWD: out[M, NOUT=N], reduction length RED=K.   BWD: out[M, NOUT=K], reduction length RED=N.
 // WGM = wavefronts along M (2 or 4); the workgroup has 2*WGM wavefronts = NT threads.
-template <int BM, int WGM, bool FWD, bool GIDX>
+// SZ: how the sequential-group kernels get scale and zero (fewer vector-memory and vector-ALU instructions in the
+// main loop; 1.5-2.5 % of the kernel):
+//   0  loaded with every step (any group size, any split)
+//   1  forward: loaded with the even steps only; needs groups of a multiple of 128 rows and a step order in which
+//      steps 2i and 2i+1 of a workgroup lie in one group (host: even split starts, lengths and rotation)
+//   2  backward: from an LDS table of the tile's group, filled once (needs the 128 output rows of a tile in one
+//      group and room for 4 bytes per column n in dynamic LDS)
+template <int BM, int WGM, bool FWD, bool GIDX, int SZ = 0>
 __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
+    static_assert(SZ == 0 || (!GIDX && ((FWD && SZ == 1) || (!FWD && SZ == 2))), "unsupported scale/zero mode");
+    extern __shared__ __attribute__((aligned(16))) unsigned char sz_tab[];
     // four distinct LDS objects (not one carved-up array): the compiler can then prove that the
     // writes into one buffer do not alias the reads of the other and is free to interleave them
     __shared__ __attribute__((aligned(16))) half_t sA0[BM * LDS_STRIDE];
@@ -381,11 +412,12 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
             *reinterpret_cast<uint4_t*>(dst + (arow + APASS * i) * LDS_STRIDE + acol) = src[i];
     };
 
-    using Slab = typename std::conditional<FWD, FwdSlab<GIDX, NT>, BwdSlab<GIDX, NT>>::type;
+    using Slab = typename std::conditional<FWD, FwdSlab<GIDX, NT>, BwdSlab<GIDX, NT, SZ == 2>>::type;
     constexpr int NSL = Slab::kSlices;
     Slab slab[2];
     slab[0].init(t, a, c0);
     slab[1].init(t, a, c0);
+    typename Slab::Prep prep;
 
     // bias of this lane's two output columns, requested before everything else: its latency hides under the
     // prologue instead of sitting in the epilogue
@@ -424,13 +456,14 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     auto step = [&](int s, auto cur_tag) {
         constexpr int CUR = decltype(cur_tag)::value;
         constexpr int NM = TM * 2 * KS;                        // MFMAs per step
-        constexpr int BAR = NM - 3;                            // MFMA index after which the barrier sits (NM-2 .. NM-5 measured: within 3 %)
+        constexpr int BAR = NM - 3;                   // MFMA index after which the barrier sits (NM-2 .. NM-5 measured: within 3 %)
         // Side work of a step: NL global loads (stage s+2 -> register set CUR) and NC consumer items
         // (stage s+1: register set CUR^1 -> LDS[CUR^1]; NSL dequantization slices with the NA activation
         // stores spread evenly among them).  One load per MFMA slot from slot 0 on (never a burst: eight
         // wavefronts issuing ten loads each at once stall on the address unit), the consumers spread over
         // slots 0..BAR-2 so that the last LDS stores have two MFMAs to drain before the barrier.
-        constexpr int NLS = Slab::kLoads, NL = NLS + NA, NC = NSL + NA;
+        constexpr int NLS = (SZ == 1 && CUR == 1) ? Slab::kLoads - 2 : Slab::kLoads;   // SZ 1: odd steps load no scale / zero
+        constexpr int NL = NLS + NA, NC = NSL + NA;
         constexpr int SLOTS = BAR - 1;
         static_assert(SLOTS >= 1, "too few MFMAs per step");
         // fragment set 0 is reloaded right after the barrier: every MFMA of sub-step KS-2 (its last
@@ -448,13 +481,16 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
             if constexpr (r == 0 && ks + 1 < KS)
                 read_frags(af[(ks + 1) & 1], bf[(ks + 1) & 1], a_cur, b_cur, ks + 1);
             acc[ti][tj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[ks & 1][ti], bf[ks & 1][tj], acc[ti][tj], 0, 0, 0);
-            // loads l with l*SLOTS/NL == i, consumers q with q*SLOTS/NC == i
-            constexpr int l_lo = i < SLOTS ? (i * NL + SLOTS - 1) / SLOTS : NL;
-            constexpr int l_hi = i < SLOTS ? ((i + 1) * NL + SLOTS - 1) / SLOTS : NL;
-            static_for<l_lo, l_hi>([&](auto lc) {
+            // (scale, zero) terms of the stage dequantized in this step, in the shadow of the step's first MFMA;
+            // SZ 1: the odd stage (CUR == 0) shares the group of the even stage before it
+            if constexpr (i == 0 && (SZ != 1 || CUR == 1)) prep = slab[CUR ^ 1].make_prep(c0);
+            // load l goes out in slot l*SLOTS/NL (rounded down), consumer q in slot q*SLOTS/NC (rounded up)
+            static_for<0, NL>([&](auto lc) {
                 constexpr int l = decltype(lc)::value;
-                if constexpr (l < NLS) slab[CUR].template load_part<l>(a, rs, red_next2);
-                else areg[CUR][l - NLS] = buf_load128(rs_a, voff_a + (l - NLS) * astride, red_next2 * 2);
+                if constexpr (l * SLOTS / NL == i) {
+                    if constexpr (l < NLS) slab[CUR].template load_part<l>(a, rs, red_next2);
+                    else areg[CUR][l - NLS] = buf_load128(rs_a, voff_a + (l - NLS) * astride, red_next2 * 2);
+                }
             });
             constexpr int q_lo = i < SLOTS ? (i * NC + SLOTS - 1) / SLOTS : NC;
             constexpr int q_hi = i < SLOTS ? ((i + 1) * NC + SLOTS - 1) / SLOTS : NC;
@@ -465,13 +501,14 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
                 if constexpr (is_a)
                     *reinterpret_cast<uint4_t*>(a_nxt + (arow + APASS * na_before) * LDS_STRIDE + acol) = areg[CUR ^ 1][na_before];
                 else
-                    slab[CUR ^ 1].template store_slice<q - na_before>(a, c0, red_next1, b_nxt);
+                    slab[CUR ^ 1].template store_slice<q - na_before>(a, c0, red_next1, b_nxt, prep);
             });
             if constexpr (i == BAR) {
                 // every wavefront has finished reading LDS[CUR] (the last fragments were fetched at
                 // sub-step KS-2) and has written its share of LDS[CUR^1]
                 __syncthreads();
                 read_frags(af[0], bf[0], a_nxt, b_nxt, 0);
+                if constexpr (SZ == 2) slab[CUR].fetch_tab(sz_tab, red_next2);   // for the slices of the next step
             }
             __builtin_amdgcn_sched_barrier(0);
         });
@@ -503,10 +540,34 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     const bool lora_masked = lora_here && a.drop.thr15 != 0;              // uniform
 
     const int red0 = red_of(0, sr, tm.phase), red1 = red_of(1, sr, tm.phase);
-    load_a(areg[0], red0);
+    // Same order as inside a step (weights, scale, zero, then the activations): the compiler's wait counts at the
+    // head of the main loop are the merge of this path and the loop's own, and with the activations of stage 1
+    // requested BEFORE its weights that merge makes every even step wait for ALL loads of the step before it.
     slab[0].load(a, rs, c0, red0);
-    load_a(areg[1], red1);
+    load_a(areg[0], red0);
     slab[1].load(a, rs, c0, red1);
+    load_a(areg[1], red1);
+    if constexpr (SZ == 2) {
+        // table of the tile's group: per unit of 8 columns one 16-byte load of scales and one zero word in, four
+        // (s_a, s_b, zero_a, zero_b) entries out
+        const int g = c0 / a.groupsize;
+        for (int u = t; u < (a.N >> 3); u += NT) {
+            const uint4_t s8 = buf_load128(rs.s, u * 16, g * a.N * 2);
+            const uint32_t z8 = buf_load32(rs.z, u * 4, g * (a.N >> 3) * 4);
+            const uint32_t sw[4] = {s8.x, s8.y, s8.z, s8.w};
+            uint32_t e[8];
+#pragma unroll
+            for (int pp = 0; pp < 4; ++pp) {
+                e[2 * pp] = sw[pp];
+                e[2 * pp + 1] = as_u32(zero_term(as_half2(sw[pp]), (z8 >> (8 * pp)) & 0xFu, (z8 >> (8 * pp + 4)) & 0xFu));
+            }
+            *reinterpret_cast<uint4_t*>(sz_tab + u * 32) = uint4_t{e[0], e[1], e[2], e[3]};
+            *reinterpret_cast<uint4_t*>(sz_tab + u * 32 + 16) = uint4_t{e[4], e[5], e[6], e[7]};
+        }
+        __syncthreads();
+        slab[0].fetch_tab(sz_tab, red0);
+        slab[1].fetch_tab(sz_tab, red1);
+    }
     if (lora_masked) {
         // Dropout on the adapter input: the adapter's share of out[m, c] exists only where the mask keeps (m, c).
         // So the adapter step runs FIRST, into the zeroed accumulators (through the second pair of LDS buffers,
@@ -528,7 +589,8 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
             }
     }
     store_a(areg[0], sA0);
-    static_for<0, NSL>([&](auto jc) { slab[0].template store_slice<decltype(jc)::value>(a, c0, red0, sB0); });
+    prep = slab[0].make_prep(c0);
+    static_for<0, NSL>([&](auto jc) { slab[0].template store_slice<decltype(jc)::value>(a, c0, red0, sB0, prep); });
     __syncthreads();
     read_frags(af[0], bf[0], sA0, sB0, 0);
     for (int s = 0; s + 1 < sr.cnt; s += 2) {
@@ -620,6 +682,34 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_cols_kernel(const floa
     *reinterpret_cast<half4_t*>(out + m * out_cols + col0 + c) = h;
 }
 
+// One grid of tiles, with the cheapest way of feeding scale and zero that the problem allows (see gemm_kernel).
+constexpr size_t kSzTableMax = 48 * 1024;     // dynamic LDS left beside the 108 KB of tile buffers
+template <int BM, int WGM, bool FWD, bool GIDX>
+static void launch_tiles(const GemmArgs& a, dim3 grid, hipStream_t stream) {
+    static const int env_sz = getenv("Q4_GEMM_SZ") ? atoi(getenv("Q4_GEMM_SZ")) : 1;
+    const dim3 block(128 * WGM);
+    if constexpr (!GIDX) {
+        if (env_sz && a.groupsize % 128 == 0) {
+            if constexpr (FWD) {
+                const int nsteps = a.K / BK, S = (int)grid.z;
+                if (nsteps % (2 * S) == 0 && ((a.phase_step & 0xff) % 2) == 0) {
+                    hipLaunchKernelGGL((gemm_kernel<BM, WGM, FWD, GIDX, 1>), grid, block, 0, stream, a);
+                    return;
+                }
+            } else {
+                const size_t tab = (size_t)a.N * 4;
+                static const bool attr_ok = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_kernel<BM, WGM, FWD, GIDX, 2>),
+                                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSzTableMax) == hipSuccess;
+                if (attr_ok && tab <= kSzTableMax) {
+                    hipLaunchKernelGGL((gemm_kernel<BM, WGM, FWD, GIDX, 2>), grid, block, tab, stream, a);
+                    return;
+                }
+            }
+        }
+    }
+    hipLaunchKernelGGL((gemm_kernel<BM, WGM, FWD, GIDX, 0>), grid, block, 0, stream, a);
+}
+
 // tail_cols > 0: the last tail_cols column tiles run as a second launch with the reduction split tail_splits ways
 // (the main launch then covers whole rounds of the CUs, and the remainder does not cost a whole round).
 template <int BM, int WGM, bool FWD, bool GIDX>
@@ -627,7 +717,7 @@ static hipError_t launch_gemm(GemmArgs a, int nout, int splits, int tail_cols, i
     const int nc = nout / BN, nr = (a.M + BM - 1) / BM;
     a.col_tile0 = 0;
     a.part_cols = nout;
-    hipLaunchKernelGGL((gemm_kernel<BM, WGM, FWD, GIDX>), dim3(nc - tail_cols, nr, splits), dim3(128 * WGM), 0, stream, a);
+    launch_tiles<BM, WGM, FWD, GIDX>(a, dim3(nc - tail_cols, nr, splits), stream);
     if (splits > 1) {
         const long total = (long)a.M * nout;
         hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream,
@@ -636,7 +726,7 @@ static hipError_t launch_gemm(GemmArgs a, int nout, int splits, int tail_cols, i
     if (tail_cols > 0) {
         a.col_tile0 = nc - tail_cols;
         a.part_cols = tail_cols * BN;
-        hipLaunchKernelGGL((gemm_kernel<BM, WGM, FWD, GIDX>), dim3(tail_cols, nr, tail_splits), dim3(128 * WGM), 0, stream, a);
+        launch_tiles<BM, WGM, FWD, GIDX>(a, dim3(tail_cols, nr, tail_splits), stream);
         const long total = (long)a.M * a.part_cols;
         hipLaunchKernelGGL(gemm_splitk_reduce_cols_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream,
                            a.part, a.out, a.M, a.part_cols, nout, a.col_tile0 * BN, tail_splits);
