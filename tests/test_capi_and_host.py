@@ -81,14 +81,16 @@ def test_error_codes_and_validation_need_no_gpu():
     assert L.q4_lora_down_f16(fake, fake, 4096, 1, 1, fake, 64, 4096, 65, None, None) == -2       # R > 64
     assert L.q4_lora_down_f16(fake, ctypes.c_void_p(0x1002), 4096, 1, 1, fake, 64, 4096, 8, None, None) == -5
     assert L.q4_lora_grad_workspace_bytes(64, 4096, 8) == 0            # one row block: no partial sums
-    assert L.q4_lora_grad_workspace_bytes(2048, 4096, 8) == 32 * 8 * 64 * 64 * 4
-    assert L.q4_lora_grad_workspace_bytes(2048, 4096, 12) == 0
-    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 64, 4096, 12, None, fake, 1 << 20, None) == -2   # R not 8/16
+    assert L.q4_lora_grad_workspace_bytes(2048, 4096, 8) == 8 * 32 * 8 * 128 * 4      # 8 row blocks x 32 strips of [R, 128] fp32
+    assert L.q4_lora_grad_workspace_bytes(2048, 4096, 12) == 8 * 32 * 12 * 128 * 4
+    assert L.q4_lora_grad_workspace_bytes(2048, 4096, 7) == 0 and L.q4_lora_grad_workspace_bytes(2048, 4096, 34) == 0
+    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 64, 4096, 7, None, fake, 1 << 20, None) == -2    # odd R
+    assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 64, 4096, 34, None, fake, 1 << 20, None) == -2   # R > 32
     assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 2048, 4096, 8, None, None, 0, None) == -3
     assert L.q4_lora_grad_f32(fake, fake, fake, 4096, 1, 1.0, 2048, 4096, 8, None, fake, 1024, None) == -3
     assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, None, 1, 8, 4096, 1.0, 2048, 8, None, fake, 1 << 24, None) == -1
     assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, fake, 1, 8, 4100, 1.0, 2048, 8, None, fake, 1 << 24, None) == -2
-    assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, fake, 1, 8, 4096, 1.0, 2048, 8, None, fake, 1 << 22, None) == -3  # needs 2 x 4 MiB
+    assert L.q4_lora_grad_pair_f32(fake, fake, fake, 4096, 1, 4096, fake, fake, fake, 1, 8, 4096, 1.0, 2048, 8, None, fake, 1 << 20, None) == -3  # needs 2 x 1 MiB
     # allocation-free GEMV: validated like q4_gemv_f16, plus the size of the built-in accumulator array
     assert L.q4_gemv_noalloc_max_outputs() == 16 * 32768
     assert L.q4_gemv_noalloc_f16(fake, fake, fake, fake, None, 128, fake, 0, 16, 256, 32832, 2, None) == -6
