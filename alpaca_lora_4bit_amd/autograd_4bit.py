@@ -294,7 +294,7 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
     with fp32 accumulation, like the reference under autocast).  fp32 / fp16 adapter matrices are
     read in place by the kernels through strides: no cast, transposed or pre-scaled copies.
 
-    Above matmul_utils_4bit.dense_switch_rows rows the same sums run as dense dequantization + library GEMMs
+    With matmul_utils_4bit.dense_switch_rows set, above that many rows the same sums run as dense dequantization + library GEMMs
     (the rank-r product writes the output once, the big product accumulates onto it).
 
     Dropout in front of lora_A (models.py:63-66; the reference's default is p = 0.05, arg_parser.py:48) stays

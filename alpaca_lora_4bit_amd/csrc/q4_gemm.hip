@@ -154,10 +154,10 @@ struct SlabRsrc {
 // Forward: slab = 64 rows (k) x 128 columns (n); LDS row = column n, minor = k.
 // A thread owns ONE column for the whole kernel and 4 packed words (32 rows) per step;
 // piece I handles pair I%4 of word I/4 and the word goes to LDS with its last piece.
-template <bool GIDX, int NT>
+template <bool GIDX, int NT, int BNT = 128>
 struct FwdSlab {
-    static constexpr int NW = 1024 / NT;          // packed words per thread per step (4 or 2)
-    static constexpr int WSTEP = NT / 128;        // word-row distance between a thread's words
+    static constexpr int NW = 8 * BNT / NT;       // packed words per thread per step (4 or 2)
+    static constexpr int WSTEP = NT / BNT;        // word-row distance between a thread's words
     static constexpr int kSlices = 4 * NW;
     uint32_t w[NW];
     uint32_t s_raw;  // fp16 bits of the scale of (current group, own column); decoded in the slices
@@ -166,7 +166,7 @@ struct FwdSlab {
     int col, wr0;    // column 0..127 of the tile; first word-row within the slab, then +WSTEP per word
     int voff_w, voff_s, voff_z, wstride;
     __device__ __forceinline__ void init(int t, const GemmArgs& a, int n0) {
-        col = t & 127; wr0 = t >> 7;
+        col = t % BNT; wr0 = t / BNT;
         wstride = WSTEP * a.N * 4;
         voff_w = (wr0 * a.N + n0 + col) * 4;
         voff_s = (n0 + col) * 2;
@@ -237,8 +237,8 @@ struct FwdSlab {
     __device__ __forceinline__ void fetch_tab(const unsigned char*, int) {}
     // LoRA step: B operand = adapter matrix [R, N]; LDS row = column n, minor = r (zero padded to 64).
     __device__ __forceinline__ void store_lora(const GemmArgs& a, int n0, half_t* sB, int t) const {
-        for (int idx = t; idx < BN * BK; idx += NT) {
-            const int r = idx >> 7, c = idx & 127;
+        for (int idx = t; idx < BNT * BK; idx += NT) {
+            const int r = idx / BNT, c = idx % BNT;
             sB[c * LDS_STRIDE + r] = (r < a.R) ? (half_t)(a.lb_scale * adapter_at(a, (size_t)r * a.lb_sr + (size_t)(n0 + c) * a.lb_sc))
                                                : (half_t)0.f;
         }
@@ -254,9 +254,9 @@ struct FwdSlab {
 // TAB: the scales and the zero terms rn16(s * (z + 1)) of the tile's group sit in an LDS table for every column n,
 // per column pair as (s_a, s_b, zero_a, zero_b) (filled once per workgroup), and come from there: one 16-byte LDS
 // read per step instead of two more global loads and the zero-term arithmetic of every step.
-template <bool GIDX, int NT, bool TAB = false>
+template <bool GIDX, int NT, bool TAB = false, int BNT = 128>
 struct BwdSlab {
-    static constexpr int RPT = 8 * 256 / NT;      // rows of the word-row handled by one thread (8 or 4)
+    static constexpr int RPT = 16 * BNT / NT;     // rows of the word-row handled by one thread (8 or 4)
     static constexpr int kSlices = 2 * RPT;
     uint4_t w;
     uint2_t sv;
@@ -265,7 +265,7 @@ struct BwdSlab {
     int wr, n4, e0;
     int voff_w, voff_s, voff_z;
     __device__ __forceinline__ void init(int t, const GemmArgs& a, int kout0) {
-        wr = (t & 255) >> 4; n4 = t & 15; e0 = (t >> 8) * RPT;
+        wr = (t % (2 * BNT)) >> 4; n4 = t & 15; e0 = (t / (2 * BNT)) * RPT;
         const int g = GIDX ? 0 : (kout0 + 8 * wr) / a.groupsize;      // fixed for the whole kernel
         voff_w = (((kout0 >> 3) + wr) * a.N + 4 * n4) * 4;
         voff_s = (g * a.N + 4 * n4) * 2;
@@ -343,8 +343,8 @@ struct BwdSlab {
     }
     // LoRA step: B operand = adapter matrix [R, K]; LDS row = k, minor = r.
     __device__ __forceinline__ void store_lora(const GemmArgs& a, int kout0, half_t* sB, int t) const {
-        for (int idx = t; idx < BN * BK; idx += NT) {
-            const int r = idx >> 7, c = idx & 127;
+        for (int idx = t; idx < BNT * BK; idx += NT) {
+            const int r = idx / BNT, c = idx % BNT;
             sB[c * LDS_STRIDE + r] = (r < a.R) ? (half_t)(a.lb_scale * adapter_at(a, (size_t)r * a.lb_sr + (size_t)(kout0 + c) * a.lb_sc))
                                                : (half_t)0.f;
         }
@@ -360,17 +360,19 @@ struct BwdSlab {
 //      steps 2i and 2i+1 of a workgroup lie in one group (host: even split starts, lengths and rotation)
 //   2  backward: from an LDS table of the tile's group, filled once (needs the 128 output rows of a tile in one
 //      group and room for 4 bytes per column n in dynamic LDS)
-template <int BM, int WGM, bool FWD, bool GIDX, int SZ = 0>
-__global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
+// WGN: wavefronts along N (2 or 4), each 64 columns wide: the tile is BM x 64*WGN.
+template <int BM, int WGM, bool FWD, bool GIDX, int SZ = 0, int WGN = 2>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_kernel(GemmArgs a) {
+    constexpr int BNT = 64 * WGN;                     // columns of the tile
     static_assert(SZ == 0 || (!GIDX && ((FWD && SZ == 1) || (!FWD && SZ == 2))), "unsupported scale/zero mode");
     extern __shared__ __attribute__((aligned(16))) unsigned char sz_tab[];
     // four distinct LDS objects (not one carved-up array): the compiler can then prove that the
     // writes into one buffer do not alias the reads of the other and is free to interleave them
     __shared__ __attribute__((aligned(16))) half_t sA0[BM * LDS_STRIDE];
     __shared__ __attribute__((aligned(16))) half_t sA1[BM * LDS_STRIDE];
-    __shared__ __attribute__((aligned(16))) half_t sB0[BN * LDS_STRIDE];
-    __shared__ __attribute__((aligned(16))) half_t sB1[BN * LDS_STRIDE];
-    constexpr int NT = 128 * WGM;                     // threads per workgroup
+    __shared__ __attribute__((aligned(16))) half_t sB0[BNT * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) half_t sB1[BNT * LDS_STRIDE];
+    constexpr int NT = 64 * WGM * WGN;                // threads per workgroup
     constexpr int WROWS = BM / WGM;                   // output rows per wavefront
     constexpr int TM = WROWS / 32;                    // 32-row accumulator tiles per wavefront
     constexpr int NA = BM * 8 / NT;                   // 16-byte activation loads per thread per step
@@ -379,13 +381,13 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
 
     const int t = threadIdx.x;
     const int lane = t & 63, wave = t >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / WGN, wn = wave % WGN;
     const int NOUT = FWD ? a.N : a.K;
     const int RED = FWD ? a.K : a.N;
     const StepRange sr = split_steps(RED / BK);
     const TileMap tm = map_tile(a.phase_step, sr.cnt, a.col_tile0);
     const int m0 = tm.tile_r * BM;
-    const int c0 = tm.tile_c * BN;           // first output column of the tile
+    const int c0 = tm.tile_c * BNT;          // first output column of the tile
     const int rows_valid = min(BM, a.M - m0);
 
     // buffer descriptors: activations of this workgroup's rows (rows beyond M read as zero), weights
@@ -412,7 +414,7 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
             *reinterpret_cast<uint4_t*>(dst + (arow + APASS * i) * LDS_STRIDE + acol) = src[i];
     };
 
-    using Slab = typename std::conditional<FWD, FwdSlab<GIDX, NT>, BwdSlab<GIDX, NT, SZ == 2>>::type;
+    using Slab = typename std::conditional<FWD, FwdSlab<GIDX, NT, BNT>, BwdSlab<GIDX, NT, SZ == 2, BNT>>::type;
     constexpr int NSL = Slab::kSlices;
     Slab slab[2];
     slab[0].init(t, a, c0);
@@ -424,7 +426,7 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     float bias_v[2] = {0.f, 0.f};
     if (FWD && a.bias) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) bias_v[j] = (float)a.bias[c0 + (wave & 1) * 64 + 32 * j + (lane & 31)];
+        for (int j = 0; j < 2; ++j) bias_v[j] = (float)a.bias[c0 + wn * 64 + 32 * j + (lane & 31)];
     }
 
     float16_t acc[TM][2];
@@ -607,7 +609,7 @@ __global__ __launch_bounds__(128 * WGM) void gemm_kernel(GemmArgs a) {
     if (gridDim.z > 1) {
         // split-K: fp32 partial sums straight from the accumulators (32 lanes cover one 128-byte row segment);
         // the bias rides with split 0, the reduction kernel adds the splits in order and rounds once
-        float* const pz = a.part + (size_t)blockIdx.z * a.M * a.part_cols - (size_t)a.col_tile0 * BN;
+        float* const pz = a.part + (size_t)blockIdx.z * a.M * a.part_cols - (size_t)a.col_tile0 * BNT;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -710,6 +712,24 @@ static void launch_tiles(const GemmArgs& a, dim3 grid, hipStream_t stream) {
     hipLaunchKernelGGL((gemm_kernel<BM, WGM, FWD, GIDX, 0>), grid, block, 0, stream, a);
 }
 
+// 256 x 256 tiles (8 wavefronts of 128 x 64): half the activation traffic and 30 % less LDS traffic per MFMA than the
+// 256 x 128 tile; for outputs with enough such tiles to fill the CUs.  No split, no second launch; the tile buffers
+// take 144 KB of LDS, so the grad-input kernel keeps its per-step scale / zero loads.
+template <bool FWD, bool GIDX>
+static hipError_t launch_gemm_wide(GemmArgs a, int nout, hipStream_t stream) {
+    const dim3 grid(nout / 256, (a.M + 255) / 256, 1), block(512);
+    a.col_tile0 = 0;
+    a.part_cols = nout;
+    if constexpr (FWD && !GIDX) {
+        if (a.groupsize % 128 == 0 && (a.K / BK) % 2 == 0 && ((a.phase_step & 0xff) % 2) == 0) {
+            hipLaunchKernelGGL((gemm_kernel<256, 2, FWD, GIDX, 1, 4>), grid, block, 0, stream, a);
+            return hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((gemm_kernel<256, 2, FWD, GIDX, 0, 4>), grid, block, 0, stream, a);
+    return hipGetLastError();
+}
+
 // tail_cols > 0: the last tail_cols column tiles run as a second launch with the reduction split tail_splits ways
 // (the main launch then covers whole rounds of the CUs, and the remainder does not cost a whole round).
 template <int BM, int WGM, bool FWD, bool GIDX>
@@ -744,6 +764,7 @@ static hipError_t launch_gemm_cfg(const GemmPlan& p, const GemmArgs& a, int nout
     switch (p.cfg) {
         case 0: return launch_gemm<128, 2, FWD, GIDX>(a, nout, p.splits, 0, 1, stream);    // 128 x 128, 4 wavefronts of 64 x 64
         case 1: return launch_gemm<256, 2, FWD, GIDX>(a, nout, p.splits, 0, 1, stream);    // 256 x 128, 4 wavefronts of 128 x 64
+        case 3: return launch_gemm_wide<FWD, GIDX>(a, nout, stream);                        // 256 x 256, 8 wavefronts of 128 x 64
         default: return launch_gemm<256, 4, FWD, GIDX>(a, nout, p.splits, p.tail_cols, p.tail_splits, stream);   // 256 x 128, 8 wavefronts of 64 x 64
     }
 }
@@ -765,6 +786,17 @@ static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
     // empty round costs more than the split gains).
     const long t256 = (long)(nout / BN) * ((M + 255) / 256);
     int splits = 1;
+    // 256 x 256 tiles from 144 of them on (a workgroup does the work of two 256 x 128 ones in about 1.7 times their
+    // time), unless their last round would leave more than a fifth of the CUs' slots empty where the narrower tiles
+    // fill theirs better: 3072 x (4096 -> 11008) has 516 wide tiles = 3 rounds for 2.02 rounds of work and stays
+    // with the narrow ones (270 against 294 us), 4096 rows have 688 (313 against 356 us).
+    const long twide = (nout % 256 == 0) ? (long)(nout / 256) * ((M + 255) / 256) : 0;
+    static const int env_wide = getenv("Q4_GEMM_WIDE") ? atoi(getenv("Q4_GEMM_WIDE")) : 1;
+    if (env_wide && env_cfg < 0 && env_splits == 0 && twide >= 144 &&
+        (twide <= 256 || 5 * twide >= 4 * 256 * ((twide + 255) / 256))) {
+        p.cfg = 3; p.splits = 1;
+        return p;
+    }
     if (t256 > 128 && M > 128) {
         p.cfg = 2;
         // More tiles than CUs and a last round that fills at most half of them: the column tiles of that
@@ -796,7 +828,11 @@ static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
             if (splits > nsteps / 4) splits = nsteps / 4;      // at least four steps per workgroup
         }
     }
-    if (env_cfg >= 0 && env_cfg != p.cfg) {                    // experiments: forced tile shape, splits as before
+    if (env_cfg == 3 && nout % 256 == 0 && M > 256) {          // experiments: wide tiles wherever they apply
+        p.cfg = 3; p.splits = 1; p.tail_cols = 0; p.tail_splits = 1;
+        return p;
+    }
+    if (env_cfg >= 0 && env_cfg != 3 && env_cfg != p.cfg) {    // experiments: forced tile shape, splits as before
         p.cfg = env_cfg;
         p.tail_cols = 0;
         const int bm = p.cfg == 0 ? 128 : 256;

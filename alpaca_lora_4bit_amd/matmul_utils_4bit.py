@@ -7,11 +7,12 @@ What changed underneath (none of it visible in the signatures):
   that reads the packed weights once for all rows; the reference launches one grid slice per row
   and switches to recons + matmul above 8 rows (matmul_utils_4bit.py:15,164-167).
 * larger inputs go to the fused dequant + MFMA GEMM, which needs no dense [K, N] buffer.
-* above `dense_switch_rows` rows (default 2048) the reference's own scheme is faster again on this GPU and is
-  used: dense dequantization (one launch at 70 % of HBM bandwidth) into a buffer from `get_buffer`, then a
-  library GEMM.  The dequantization is then a small fraction of the product, and the library's GEMM has no
-  dequantization competing with its matrix instructions for issue slots.  `cache_buffer` keeps its meaning
-  (one process-global buffer per shape, or a fresh one per call when False).
+* the reference's own scheme (dense dequantization into a buffer from `get_buffer`, then a library GEMM) is kept
+  behind `dense_switch_rows`: rows above that value take it.  The default is None (never): with 256 x 256 tiles for
+  large outputs the fused kernel is level with dequantization + library GEMM from 2560 rows up (a 7B decoder
+  layer's seven products, forward + grad-input: 5 % faster at 4096 rows, 4 % slower at 8192) and needs no dense
+  buffer.  Layers whose in / out features are not multiples of 128 always take the dense route.  `cache_buffer`
+  keeps its meaning (one process-global buffer per shape, or a fresh one per call when False).
 * `act_order` and `faster_mode` no longer select kernels: whether `g_idx` is a real
   permutation is detected per tensor (quant_hip.classify_g_idx).  The reference's default
   kernel ignores g_idx unless the user sets `act_order = True` by hand (:75-87); here a
@@ -38,7 +39,7 @@ faster_mode = 'old_faster'
 valid_faster_mode = ('faster', 'old_faster')
 act_order = False
 cache_buffer = True
-dense_switch_rows = 2048          # rows above this: dense dequant + library GEMM; 0 or None: always the fused GEMM
+dense_switch_rows = None          # rows above this: dense dequant + library GEMM; 0 or None: always the fused GEMM
 
 
 def get_buffer(shape_of_qweight, dtype=torch.float16, device='cuda', bits=4, zero=True):

@@ -233,13 +233,15 @@ def test_backend_switch_and_errors():
 
 @pytest.mark.parametrize("act", [False, True])
 def test_dense_route_above_the_row_switch(oracle, act):
-    """Above matmul_utils_4bit.dense_switch_rows rows the product runs as dense dequantization + library GEMM (the
-    reference's recons scheme, matmul_utils_4bit.py:114-127): same values as the fused GEMM for the plain layer
-    (no-grad and autograd, with bias) and for the LoRA layer (y, dx, dA, dB), and the fused kernels are not called."""
+    """With matmul_utils_4bit.dense_switch_rows set, products above that many rows run as dense dequantization +
+    library GEMM (the reference's recons scheme, matmul_utils_4bit.py:114-127; off by default): same values as the
+    fused GEMM for the plain layer (no-grad and autograd, with bias) and for the LoRA layer (y, dx, dA, dB), and the
+    fused kernels are not called."""
     import torch
     from alpaca_lora_4bit_amd import autograd_4bit, matmul_utils_4bit as mm4b, models, quant_hip
     K, N, r, rows = 256, 384, 8, 2304
-    assert mm4b.dense_switch_rows == 2048
+    assert not mm4b.dense_switch_rows                      # default: the fused kernels at every size
+    mm4b.dense_switch_rows = 2048
     layer = oracle.make_layer(K, N, 128, act_order=act, seed=31)
     A, B = oracle.make_lora(K, N, r, seed=31)
     x = oracle.make_activations(rows, K, seed=61)
@@ -291,6 +293,7 @@ def test_dense_route_above_the_row_switch(oracle, act):
             mm4b.dense_switch_rows = 2048
         assert fused_calls == ["fwd"]
     finally:
+        mm4b.dense_switch_rows = None
         quant_hip.gemm_fwd, quant_hip.gemm_bwd_dx = real_fwd, real_bwd
 
 

@@ -127,6 +127,51 @@ def test_gemm_lora_steps(oracle, M, K, N, r, act):
     assert rel_err(y0.cpu().numpy(), yref) > rel_err(y.cpu().numpy(), yref)
 
 
+@pytest.mark.parametrize("M,K,N,gs,act,r", [(9300, 1024, 1024, 128, False, 8), (9217, 1024, 1024, 128, True, 0),
+                                            (9300, 1024, 1024, 64, False, 16), (2350, 4096, 4096, 128, False, 8),
+                                            (2305, 512, 4096, 256, False, 0)])
+def test_wide_tiles_256x256(oracle, M, K, N, gs, act, r):
+    """Outputs with at least 144 tiles of 256 x 256 run the eight-wavefront wide tile (forward and grad-input, with
+    bias, adapter step and the masked adapter term): against fp32 products with the bit-exact dense W on the GPU."""
+    import torch
+    from alpaca_lora_4bit_amd import _lib, quant_hip
+    layer = oracle.make_layer(K, N, gs, act_order=act, seed=M + K)
+    t = to_cuda_layer(layer)
+    g = torch.Generator(device="cuda").manual_seed(M)
+    x = torch.randn((M, K), device="cuda", generator=g).half()
+    dy = torch.randn((M, N), device="cuda", generator=g).half()
+    bias = (torch.randn(N, device="cuda", generator=g) * 0.1).half()
+    W = quant_hip.dequant(t["qweight"], t["qzeros"], t["scales"], t["g_idx"], gs).float()
+    gi = t["g_idx"] if (act or gs % 64) else None
+    kw_f, kw_b = {}, {}
+    yref = x.float() @ W + bias.float()
+    dxref = dy.float() @ W.t()
+    if r:
+        A = (torch.randn((r, K), device="cuda", generator=g) * 0.05)          # fp32 adapter matrices, read in place
+        B = (torch.randn((N, r), device="cuda", generator=g) * 0.05)
+        xa = quant_hip.lora_down(x, A)
+        dyb = quant_hip.lora_down(dy, B.t())
+        kw_f = dict(xa=xa, lora_bt=B.t(), lora_scale=2.0)
+        kw_b = dict(dyb=dyb, lora_a=A, lora_scale=2.0)
+        yref = yref + 2.0 * (xa.float() @ B.half().float().t())
+        dxref = dxref + 2.0 * (dyb.float() @ A.half().float())
+    y = quant_hip.gemm_fwd(x, t["qweight"], t["qzeros"], t["scales"], gi, gs, bias=bias, **kw_f)
+    dx = quant_hip.gemm_bwd_dx(dy, t["qweight"], t["qzeros"], t["scales"], gi, gs, **kw_b)
+    assert y.shape == (M, N) and dx.shape == (M, K)
+    for got, ref in ((y, yref), (dx, dxref)):
+        err = float((got.float() - ref).abs().max() / ref.abs().max())
+        assert err <= TOL and err <= 2e-3, err
+    # the forward product of every case has at least 144 wide tiles: it runs unsplit and wants no workspace
+    assert (N // 256) * -(-M // 256) >= 144 and _lib.lib().q4_gemm_workspace_bytes(1, M, K, N) == 0
+    if r:
+        # masked adapter term of the grad-input (dropout in front of lora_A): only kept positions carry it
+        drop = (1234, 0.25)
+        keep = quant_hip.dropout_keep_mask(M, K, drop[0], drop[1], x.device).float()
+        dxm = quant_hip.gemm_bwd_dx(dy, t["qweight"], t["qzeros"], t["scales"], gi, gs, dropout=drop, **kw_b)
+        ref = dy.float() @ W.t() + keep * quant_hip.dropout_scale(drop[1]) * 2.0 * (dyb.float() @ A.half().float())
+        assert float((dxm.float() - ref).abs().max() / ref.abs().max()) <= 2e-3
+
+
 def test_gemm_rejects_unsupported_shapes(oracle):
     import torch
     from alpaca_lora_4bit_amd import quant_hip
@@ -196,7 +241,7 @@ def test_gemm_forward_streaming_kernel_several_strips_per_workgroup(oracle, M, K
 
 
 @pytest.mark.parametrize("act", [False, True])
-@pytest.mark.parametrize("M,red,nout,tail_cols,tail_splits", [(1024, 1024, 11008, 22, 2), (520, 1024, 11008, 1, 2),
+@pytest.mark.parametrize("M,red,nout,tail_cols,tail_splits", [(1024, 1024, 11136, 23, 2), (520, 1024, 11008, 1, 2),
                                                               (1536, 4096, 11008, 1, 8)])
 def test_gemm_remainder_tiles_run_as_a_split_second_launch(oracle, M, red, nout, tail_cols, tail_splits, act):
     """More 256-row tiles than CUs with a last round that fills at most half of them: the remainder's column tiles
