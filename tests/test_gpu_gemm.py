@@ -282,3 +282,51 @@ def test_gemm_remainder_tiles_run_as_a_split_second_launch(oracle, M, red, nout,
             edge = (nout // 128 - tail_cols) * 128                  # first column of the second launch
             assert rel_err(out[:, edge - 128:edge + 128], want[:, edge - 128:edge + 128]) <= TOL
             assert rel_err(out[:, -128:], want[:, -128:]) <= TOL
+
+
+_GRAPH_SCRIPT = r'''
+import sys
+sys.path.insert(0, sys.argv[1])
+import torch
+import bench
+from alpaca_lora_4bit_amd import quant_hip
+
+gen = torch.Generator(device="cuda").manual_seed(3)
+cases = [(300, 1024, 768), (40, 1024, 768), (3072, 512, 3072), (1024, 2048, 1024)]   # split-K, streaming, wide tiles, two-way split
+for (M, K, N) in cases:
+    lay = bench.make_layer_gpu(K, N, 128, gen, False)
+    w = (lay["qweight"], lay["qzeros"], lay["scales"], lay["g_idx"], 128)
+    assert quant_hip.scales_fit_fused_dequant(lay["scales"])     # the content check reads back once: before the capture
+    x = torch.randn((M, K), device="cuda", generator=gen).half()
+    dy = torch.randn((M, N), device="cuda", generator=gen).half()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=side):         # the first products of this shape are issued under capture
+        y = quant_hip.gemm_fwd(x, *w)
+        dx = quant_hip.gemm_bwd_dx(dy, *w)
+    for rep in range(3):
+        x.normal_(generator=gen)
+        dy.normal_(generator=gen)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        y_e = quant_hip.gemm_fwd(x, *w)
+        dx_e = quant_hip.gemm_bwd_dx(dy, *w)
+        torch.cuda.synchronize()
+        assert torch.equal(y, y_e) and torch.equal(dx, dx_e), (M, K, N, rep)
+        assert float(y.float().abs().max()) > 0 and float(dx.float().abs().max()) > 0
+print("graph ok")
+'''
+
+
+def test_products_first_issued_under_graph_capture_replay_like_eager():
+    """A fresh process whose very first GEMM launches happen while a HIP graph is being captured (the launchers set a
+    kernel attribute on first use; only the per-tensor content check, which reads a value back, ran before): every
+    replay, with new inputs and eager work in between, equals the eager call bit for bit."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", _GRAPH_SCRIPT, root], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0 and "graph ok" in r.stdout, r.stdout[-2000:] + r.stderr[-4000:]
