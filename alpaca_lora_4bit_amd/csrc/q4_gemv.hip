@@ -611,6 +611,167 @@ void skinny_seq_kernel(SkinnyArgs a) {
     }
 }
 
+// ------------------------------------------------------------------ forward, some hundred rows (sequential groups)
+// Between the streaming kernel above and the tiled MFMA kernel lies a range of rows where an output has too few
+// 256-row tiles to fill the CUs without splitting the reduction (partial tiles, a second kernel) and the kernel
+// above pays its two barriers and an LDS sum per strip.  Here a workgroup owns one 64-column strip of 16*RB rows
+// for the WHOLE reduction: wavefront w walks the chunks w, w + 8, ... of 128 reduction rows with its accumulators
+// in registers, the next chunk's words, scales and activations in flight while it multiplies the current one, and
+// the eight wavefronts are summed through LDS once, at the end, into fp16 outputs: one launch, no workspace.
+// The B operand holds the dequantized weights rn16(rn16(s*q) - rn16(s*(z+1))) (the values of the dense kernel,
+// quant_cuda_kernel.cu:1148-1152): with one scale per column of a chunk the product of code and scale is one
+// packed fused multiply-add on (1024 + q) or (64 + q) (1024*s and 64*s are exact), the zero term one subtraction.
+template <int RB>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2)))
+void stream_fwd_kernel(SkinnyArgs a) {
+    constexpr int NSTEP = 4, NW = 8;
+    constexpr int kFar = 0x70000000;
+    // [row block][wavefront][row][column of the strip]; inside the loop, the activation tiles being turned
+    __shared__ __attribute__((aligned(16))) float red[RB][NW][16 * 64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kk = lane >> 4, c = lane & 15;
+    const int n0 = blockIdx.x << 6;
+    const int row0 = blockIdx.z * (16 * RB);
+    const int nchunks = a.K >> 7;
+
+    const rsrc_t rw = make_rsrc(a.qweight, (unsigned)((size_t)(a.K >> 3) * a.N * 4));
+    const rsrc_t rs = make_rsrc(a.scales, (unsigned)((size_t)a.G * a.N * 2));
+    const rsrc_t rz = make_rsrc(a.qzeros, (unsigned)((size_t)a.G * (a.N >> 3) * 4));
+    const rsrc_t rx = make_rsrc(a.x, (unsigned)((size_t)a.M * a.K * 2));
+    const int vw = (kk * a.N + n0 + 4 * c) * 4;
+    const int vs = (n0 + 4 * c) * 2;
+    const int vz = ((n0 >> 3) + (c >> 1)) * 4;
+    const int wstep = 16 * a.N;                    // bytes between the words of two steps (4 packed rows)
+    // Activations: a lane of the MFMA A operand wants 16 bytes of row c, so direct loads would touch 16 rows (16
+    // cache lines) per quarter wavefront.  They are loaded row-contiguous instead (a quarter wavefront = 256
+    // contiguous bytes of one row), straight into this wavefront's own 4 KB of LDS per row block (no registers in
+    // between: the next chunk's tile travels while this chunk is multiplied), and read back column-wise.  Lane
+    // (kk, c) of load i lands at unit c of row 4i + kk and fetches unit c ^ (4i + kk) of that row, so unit q of row
+    // r sits at q ^ r: the column-wise reads are conflict-free.  Rows beyond M lie beyond the buffer: zeros.
+    int vx[NSTEP];
+#pragma unroll
+    for (int i = 0; i < NSTEP; ++i) vx[i] = (kk * a.K + 8 * (c ^ (4 * i + kk))) * 2;
+    typedef __attribute__((address_space(3))) void lds_void;
+
+    uint4_t w0[NSTEP], w1[NSTEP];
+    uint2_t sv;
+    uint32_t zv;
+    // everything chunk `ch` of this wavefront needs; past the end of the reduction: zeros, without traffic
+    auto fetch = [&](int ch) {
+        const int off = ch < nchunks ? 0 : kFar;
+        const int k0 = ch << 7, g = k0 / a.groupsize;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int i = 0; i < NSTEP; ++i)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_void*)(&red[rb][wave][256 * i]), 16, vx[i],
+                                                         off + ((row0 + 16 * rb + 4 * i) * a.K + k0) * 2, 0, 0);
+        sv = buf_load64(rs, vs, off + g * a.N * 2);
+        zv = buf_load32(rz, vz, off + g * (a.N >> 3) * 4);
+#pragma unroll
+        for (int t = 0; t < NSTEP; ++t) w1[t] = buf_load128_stream(rw, vw, off + (ch << 4) * a.N * 4 + t * wstep);
+    };
+    fetch(wave);
+
+    float4_t acc[RB][4];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[rb][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+    for (int ch = wave; ch < nchunks; ch += NW) {
+        // the loads of this chunk have landed (vmcnt 0): the tile in LDS, words, scales and zeros in registers
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // A operands in the order the nibble split below produces: (e0,e4)(e1,e5)(e2,e6)(e3,e7)
+        half8_t av[RB][NSTEP];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const uint4_t* stage = reinterpret_cast<const uint4_t*>(&red[rb][wave][0]);
+#pragma unroll
+            for (int t = 0; t < NSTEP; ++t) {
+                const uint4_t u = stage[c * 16 + ((4 * t + kk) ^ c)];
+                av[rb][t] = make_half8(__builtin_amdgcn_perm(u.z, u.x, 0x05040100u), __builtin_amdgcn_perm(u.z, u.x, 0x07060302u),
+                                       __builtin_amdgcn_perm(u.w, u.y, 0x05040100u), __builtin_amdgcn_perm(u.w, u.y, 0x07060302u));
+            }
+        }
+        // scale and zero term of the four columns of this lane (one group per chunk)
+        const uint32_t zw = zv >> ((c & 1) * 16);
+        const uint32_t sraw[4] = {sv.x & 0xFFFFu, sv.x >> 16, sv.y & 0xFFFFu, sv.y >> 16};
+        half2_t s2[4], s1024[4], s64[4], zero2[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f}, k64 = {(half_t)64.0f, (half_t)64.0f};
+            s2[j] = as_half2(sraw[j] | (sraw[j] << 16));
+            s1024[j] = s2[j] * k1024;
+            s64[j] = s2[j] * k64;
+            const uint32_t z = (zw >> (4 * j)) & 0xFu;
+            zero2[j] = zero_term(s2[j], z, z);
+        }
+#pragma unroll
+        for (int t = 0; t < NSTEP; ++t) w0[t] = w1[t];
+        // the tile has been read (lgkmcnt 0): the next chunk of this wavefront may overwrite it
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(ch + NW);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < NSTEP; ++t) {
+            const uint32_t w[4] = {w0[t].x, w0[t].y, w0[t].z, w0[t].w};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                // a code in mantissa bits 0..3 of fp16 1024.0 reads 1024 + q, in bits 4..7 of fp16 64.0 it reads 64 + q
+                const uint32_t hi = w[j] >> 8;
+                const half2_t b0 = __builtin_elementwise_fma(as_half2((w[j] & 0x000F000Fu) | 0x64006400u), s2[j], -s1024[j]) - zero2[j];
+                const half2_t b1 = __builtin_elementwise_fma(as_half2((w[j] & 0x00F000F0u) | 0x54005400u), s2[j], -s64[j]) - zero2[j];
+                const half2_t b2 = __builtin_elementwise_fma(as_half2((hi & 0x000F000Fu) | 0x64006400u), s2[j], -s1024[j]) - zero2[j];
+                const half2_t b3 = __builtin_elementwise_fma(as_half2((hi & 0x00F000F0u) | 0x54005400u), s2[j], -s64[j]) - zero2[j];
+                const half8_t bv = make_half8(as_u32(b0), as_u32(b1), as_u32(b2), as_u32(b3));
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb)
+                    acc[rb][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[rb][t], bv, acc[rb][j], 0, 0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);     // B operands are built step by step, not all sixteen ahead
+        }
+    }
+    // the prefetch past the last chunk of this wavefront wrote zeros into the tile: landed before the sum reuses it
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // sum over the wavefronts; row 4*kk + r of the block, columns 4c .. 4c+3
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            *reinterpret_cast<float4_t*>(&red[rb][wave][((4 * kk + r) << 6) + 4 * c]) =
+                float4_t{acc[rb][0][r], acc[rb][1][r], acc[rb][2][r], acc[rb][3][r]};
+    __syncthreads();
+    {
+        // thread t finishes row t/32 of every block, columns 2*(t%32) and the next
+        const int e = 2 * threadIdx.x;
+        const int row = e >> 6, cc = n0 + (e & 63);
+        half2_t b2 = {(half_t)0.f, (half_t)0.f};
+        if (a.bias) b2 = *reinterpret_cast<const half2_t*>(a.bias + cc);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) {
+                const float* rp = &red[rb][w][e];
+                v0 += rp[0];
+                v1 += rp[1];
+            }
+            const int m = row0 + 16 * rb + row;
+            if (m < a.M) {
+                const half2_t h = {(half_t)(v0 + (float)b2[0]), (half_t)(v1 + (float)b2[1])};
+                *reinterpret_cast<half2_t*>(a.y + (size_t)m * a.N + cc) = h;
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------ grad-input, 17 <= M <= 48 (sequential groups)
 // dx[M, K] = dy[M, N] @ W^T with the same streaming scheme: the reduction runs over the columns n of W, the outputs
 // are its rows k.  A packed word holds 8 consecutive rows k of one column n, so the 8 words of columns n .. n+7
@@ -1166,6 +1327,55 @@ extern "C" int q4_launch_skinny(const void* x, const int32_t* qweight, const int
     if (hipGetLastError() != hipSuccess) return -4;
     if (S > 1) return q4_launch_splitk_reduce(a.part, y, (long)M * N, S, stream);
     return 0;
+}
+
+// Shapes the whole-reduction streaming kernel takes: more than 64 rows, sequential groups that are multiples of 128
+// rows, and an output small enough for ONE round of workgroups (at most one per CU): the kernel is bound by the
+// activation tiles every workgroup pulls through its CU's vector memory path, so a second round costs as much as the
+// first, while the tiled kernel only gets better with more tiles (measured on 4096 x 4096, 65..256 rows: 10.2-16.1 us
+// against 16.1-24.4 us; 2048 x 2048, 65..512 rows: 7-10.6 against 12.3-22.3 us; 11008 -> 4096, up to 192 rows: 22-31
+// against 22-34 us; 4096 -> 11008 never fits one round).
+// Row blocks of 32, 48 or 64 rows: the smallest that fits (more workgroups, fewer idle CUs).
+static int stream_fwd_row_blocks(int M, int N) {
+    static const int force_rb = getenv("Q4_STREAM_FWD_RB") ? atoi(getenv("Q4_STREAM_FWD_RB")) : 0;
+    if (force_rb >= 2 && force_rb <= 4) return force_rb;
+    const int strips = N / q4::kColsPerWave;
+    for (int rb = 2; rb <= 4; ++rb)
+        if (strips * ((M + 16 * rb - 1) / (16 * rb)) <= 256) return rb;
+    return 0;
+}
+extern "C" int q4_stream_fwd_applicable(int M, int K, int N, int groupsize, int has_gidx) {
+    static const int max_rows = getenv("Q4_STREAM_FWD_MAX_ROWS") ? atoi(getenv("Q4_STREAM_FWD_MAX_ROWS")) : 512;
+    if (!(M > 64 && M <= max_rows && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 64 == 0))
+        return 0;
+    // very long reductions with the larger row blocks: level with the tiled kernel or just behind (13824 -> 5120)
+    const int rb = stream_fwd_row_blocks(M, N);
+    return rb == 2 || (rb > 2 && K <= 12288);
+}
+
+extern "C" int q4_launch_stream_fwd(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                                    int groupsize, const void* bias, void* y, int M, int K, int N, int G,
+                                    hipStream_t stream) {
+    using namespace q4;
+    SkinnyArgs a;
+    a.x = reinterpret_cast<const half_t*>(x);
+    a.qweight = reinterpret_cast<const uint32_t*>(qweight);
+    a.qzeros = reinterpret_cast<const uint32_t*>(qzeros);
+    a.scales = reinterpret_cast<const half_t*>(scales);
+    a.bias = reinterpret_cast<const half_t*>(bias);
+    a.groupsize = groupsize;
+    a.y = reinterpret_cast<half_t*>(y);
+    a.part = nullptr;
+    a.M = M; a.K = K; a.N = N; a.G = G;
+    a.strips_per_wg = 1;
+    const int strips = N / kColsPerWave;
+    const int rb = stream_fwd_row_blocks(M, N);
+    if (rb == 0) return -2;
+    const dim3 grid(strips, 1, (M + 16 * rb - 1) / (16 * rb)), block(512);
+    if (rb == 2) hipLaunchKernelGGL(stream_fwd_kernel<2>, grid, block, 0, stream, a);
+    else if (rb == 3) hipLaunchKernelGGL(stream_fwd_kernel<3>, grid, block, 0, stream, a);
+    else hipLaunchKernelGGL(stream_fwd_kernel<4>, grid, block, 0, stream, a);
+    return hipGetLastError() == hipSuccess ? 0 : -4;
 }
 
 // Shapes the streaming grad-input kernel takes: 17..48 rows, sequential groups that are multiples of 128 rows.

@@ -240,6 +240,35 @@ def test_gemm_forward_streaming_kernel_several_strips_per_workgroup(oracle, M, K
     assert np.abs(y.float().cpu().numpy() - ref).max() <= 1e-2 * np.abs(ref).max()
 
 
+@pytest.mark.parametrize("M", [65, 96, 100, 128, 129, 192, 200, 256, 300, 512])
+@pytest.mark.parametrize("K,N,gs", [(4096, 4096, 128), (1408, 256, 128), (512, 384, 256), (11008, 1024, 128),
+                                    (1024, 2048, 1024), (128, 128, 128)])
+def test_gemm_forward_65_to_512_rows_whole_reduction_streaming_kernel(oracle, M, K, N, gs):
+    """More than 64 rows of an output that one round of workgroups covers: one 64-column strip of 32, 48 or 64 rows per
+    workgroup over the whole reduction (11 and 86 chunks of 128: uneven shares of the eight wavefronts; 1 and 4
+    chunks: idle wavefronts), activation tiles delivered to LDS by the loads themselves, row blocks cut off by M,
+    with bias.  Same dequantized weights as the tiled kernel, which the other shapes of this list still take."""
+    import torch
+    from alpaca_lora_4bit_amd import _lib, quant_hip
+    layer = oracle.make_layer(K, N, gs, seed=K + N + M)
+    t = to_cuda_layer(layer)
+    x = oracle.make_activations(M, K, seed=M + 13)
+    bias = (np.random.default_rng(M).standard_normal(N) * 0.5).astype(np.float16)
+    ref = oracle.matmul_recons(x, layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"]) + bias.astype(np.float32)
+    y = quant_hip.gemm_fwd(torch.from_numpy(x).cuda(), t["qweight"], t["qzeros"], t["scales"], None, gs,
+                           bias=torch.from_numpy(bias).cuda())
+    y2 = quant_hip.gemm_fwd(torch.from_numpy(x).cuda(), t["qweight"], t["qzeros"], t["scales"], None, gs,
+                            bias=torch.from_numpy(bias).cuda())
+    assert y.shape == (M, N) and torch.equal(y, y2)
+    assert np.abs(y.float().cpu().numpy() - ref).max() <= 1e-2 * np.abs(ref).max()
+    assert np.abs(y.float().cpu().numpy() - ref).max() <= 2e-3 * np.abs(ref).max()
+    lib = _lib.lib()
+    strips = N // 64
+    rb = next((rb for rb in (2, 3, 4) if strips * -(-M // (16 * rb)) <= 256), 0)
+    assert bool(lib.q4_stream_fwd_applicable(M, K, N, gs, 0)) == (rb == 2 or (rb > 2 and K <= 12288))
+    assert not lib.q4_stream_fwd_applicable(M, K, N, gs, 1) and not lib.q4_stream_fwd_applicable(64, K, N, gs, 0)
+
+
 @pytest.mark.parametrize("act", [False, True])
 @pytest.mark.parametrize("M,red,nout,tail_cols,tail_splits", [(1024, 1024, 11136, 23, 2), (520, 1024, 11008, 1, 2),
                                                               (1536, 4096, 11008, 1, 8)])
