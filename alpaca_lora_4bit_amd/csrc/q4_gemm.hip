@@ -862,6 +862,9 @@ extern "C" {
 int q4_stream_fwd_applicable(int M, int K, int N, int groupsize, int has_gidx);
 int q4_launch_stream_fwd(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales, int groupsize,
                          const void* bias, void* y, int M, int K, int N, int G, hipStream_t stream);
+int q4_stream_dx_applicable(int M, int K, int N, int groupsize, int has_gidx);
+int q4_launch_stream_dx(const void* dy, const int32_t* qweight, const int32_t* qzeros, const void* scales, int groupsize,
+                        void* dx, int M, int K, int N, int G, hipStream_t stream);
 int q4_skinny_applicable(int M, int K, int N, int groupsize, int has_gidx);
 size_t q4_skinny_workspace(int M, int K, int N);
 int q4_launch_skinny(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales, int groupsize,
@@ -900,12 +903,15 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     if (env_order > 0) a.phase_step |= (env_order > 64 ? 64 : env_order) << 8;
     const int nout = fwd ? N : K;
     const bool gidx = g_idx != nullptr;
-    // 17..64 rows, forward, no adapter: the weight-streaming kernel (one pass over the packed weights)
+    // some hundred rows of an output that one round of workgroups covers, no adapter: whole-reduction streaming kernels
     if (fwd && a.R == 0 && q4_stream_fwd_applicable(M, K, N, groupsize, gidx))
         return q4_launch_stream_fwd(act, qweight, qzeros, scales, groupsize, bias, out, M, K, N, G, stream);
+    // 17..64 rows, forward, no adapter: the weight-streaming kernel (one pass over the packed weights)
     if (fwd && a.R == 0 && q4_skinny_applicable(M, K, N, groupsize, gidx) && workspace &&
         workspace_bytes >= q4_skinny_workspace(M, K, N))
         return q4_launch_skinny(act, qweight, qzeros, scales, groupsize, bias, out, M, K, N, G, workspace, stream);
+    if (!fwd && a.R == 0 && q4_stream_dx_applicable(M, K, N, groupsize, gidx))
+        return q4_launch_stream_dx(act, qweight, qzeros, scales, groupsize, out, M, K, N, G, stream);
     // 17..48 rows, grad-input, no adapter: its transposed counterpart
     if (!fwd && a.R == 0 && q4_skinny_dx_applicable(M, K, N, groupsize, gidx) && workspace &&
         workspace_bytes >= q4_skinny_dx_workspace(M, K, N))

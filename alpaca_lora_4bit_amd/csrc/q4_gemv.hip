@@ -994,6 +994,187 @@ void skinny_dx_kernel(SkinnyDxArgs a) {
     }
 }
 
+// ------------------------------------------------------------------ grad-input, some hundred rows (sequential groups)
+// The whole-reduction counterpart of stream_fwd_kernel for dx = dy @ W^T, with the operand scheme of skinny_dx_kernel:
+// a workgroup owns one block of 128 outputs k (one quantization group) of 16*RB rows, wavefront w walks the chunks
+// w, w + 8, ... of 128 columns n with its accumulators in registers (the chunk's tile of dy delivered to LDS by the
+// loads themselves while the previous chunk is multiplied, words / scales / zeros one stage of SS steps ahead), and
+// the eight wavefronts are summed through LDS once, at the end, into fp16 outputs: one launch, no workspace.
+template <int RB, int SS>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2)))
+void stream_dx_kernel(SkinnyDxArgs a) {
+    constexpr int NSTEP = 4, NW = 8, NH = NSTEP / SS;
+    constexpr int kFar = 0x70000000;
+    __shared__ __attribute__((aligned(16))) float red[RB][NW][16 * 64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int kk = lane >> 4, c = lane & 15;
+    const int blk = blockIdx.x;
+    const int row0 = blockIdx.z * (16 * RB);
+    const int nchunks = a.N >> 7;
+    const int g = (blk << 7) / a.groupsize;
+
+    const rsrc_t rw = make_rsrc(a.qweight, (unsigned)((size_t)(a.K >> 3) * a.N * 4));
+    const rsrc_t rs = make_rsrc(a.scales, (unsigned)((size_t)a.G * a.N * 2));
+    const rsrc_t rz = make_rsrc(a.qzeros, (unsigned)((size_t)a.G * (a.N >> 3) * 4));
+    const rsrc_t rdy = make_rsrc(a.dy, (unsigned)((size_t)a.M * a.N * 2));
+    const int vw = (c * a.N + 8 * kk) * 4;
+    const int vs = 16 * kk;
+    const int vz = 4 * kk;
+    const int wbase = blk * 16 * a.N * 4, sbase = g * a.N * 2, zbase = g * (a.N >> 3) * 4;
+    // tile of dy: lane (kk, c) of load i lands at unit c of row 4i + kk and fetches unit c ^ (4i + kk) of that row (see
+    // stream_fwd_kernel); rows beyond M lie beyond the buffer and read as zeros
+    int vx[NSTEP];
+#pragma unroll
+    for (int i = 0; i < NSTEP; ++i) vx[i] = (kk * a.N + 8 * (c ^ (4 * i + kk))) * 2;
+    typedef __attribute__((address_space(3))) void lds_void;
+    auto fetch_tile = [&](int ch) {
+        const int off = ch < nchunks ? 0 : kFar;   // past the end: no traffic
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int i = 0; i < NSTEP; ++i)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rdy, (lds_void*)(&red[rb][wave][256 * i]), 16, vx[i],
+                                                         off + ((row0 + 16 * rb + 4 * i) * a.N + (ch << 7)) * 2, 0, 0);
+    };
+    // one pipeline stage = SS steps of 32 columns of one chunk
+    struct Stage { uint4_t w[SS][2]; uint4_t s[SS]; uint32_t z[SS]; };
+    auto load_stage = [&](Stage& st, int ch, int h) {
+        const int off = ch < nchunks ? 0 : kFar;
+        const int n0 = ch << 7;
+#pragma unroll
+        for (int u = 0; u < SS; ++u) {
+            const int t = SS * h + u;
+            st.s[u] = buf_load128(rs, vs, off + sbase + n0 * 2 + t * 64);
+            st.z[u] = buf_load32(rz, vz, off + zbase + (n0 >> 1) + t * 16);
+        }
+#pragma unroll
+        for (int u = 0; u < SS; ++u) {
+            const int t = SS * h + u;
+            st.w[u][0] = buf_load128_stream(rw, vw, off + wbase + n0 * 4 + t * 128);
+            st.w[u][1] = buf_load128_stream(rw, vw, off + wbase + n0 * 4 + t * 128 + 16);
+        }
+    };
+
+    float4_t acc[RB][8], corr[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        corr[rb] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[rb][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    half8_t av[RB][NSTEP];
+    auto multiply = [&](const Stage& st, auto htag) {
+        constexpr int h = decltype(htag)::value;
+#pragma unroll
+        for (int u = 0; u < SS; ++u) {
+            constexpr int tbase = SS * h;
+            const half8_t s8 = __builtin_bit_cast(half8_t, st.s[u]);
+            half8_t as[RB];
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) as[rb] = av[rb][tbase + u] * s8;
+            // B operand of the zero term: 1025 + z for this lane's eight columns
+            const uint32_t zlo = st.z[u] & 0x0F0F0F0Fu, zhi = (st.z[u] >> 4) & 0x0F0F0F0Fu;
+            const half2_t one2 = {(half_t)1.f, (half_t)1.f};
+            uint32_t zb[4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p)
+                zb[p] = as_u32(as_half2(__builtin_amdgcn_perm(zhi, zlo, 0x0c040c00u + 0x00010001u * p) | kMagic) + one2);
+            const half8_t zB = make_half8(zb[0], zb[1], zb[2], zb[3]);
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) corr[rb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as[rb], zB, corr[rb], 0, 0, 0);
+            // code operands: byte b of a word holds the codes of rows 2b (low nibble) and 2b + 1
+            const uint32_t wd[8] = {st.w[u][0].x, st.w[u][0].y, st.w[u][0].z, st.w[u][0].w,
+                                    st.w[u][1].x, st.w[u][1].y, st.w[u][1].z, st.w[u][1].w};
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                uint32_t ev[4], od[4];
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    const uint32_t sel = 0x0c000c00u | ((4u + b) << 16) | (uint32_t)b;
+                    const uint32_t pb = __builtin_amdgcn_perm(wd[2 * p + 1], wd[2 * p], sel);   // byte b of columns 2p, 2p+1
+                    ev[p] = (pb & 0x000F000Fu) | kMagic;
+                    od[p] = ((pb >> 4) & 0x000F000Fu) | kMagic;
+                }
+                const half8_t be = make_half8(ev[0], ev[1], ev[2], ev[3]), bo = make_half8(od[0], od[1], od[2], od[3]);
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) {
+                    acc[rb][2 * b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as[rb], be, acc[rb][2 * b], 0, 0, 0);
+                    acc[rb][2 * b + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(as[rb], bo, acc[rb][2 * b + 1], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    Stage buf[2];
+    fetch_tile(wave);
+    load_stage(buf[0], wave, 0);
+    for (int ch = wave; ch < nchunks; ch += NW) {
+        // the tile of this chunk and the first stage have landed (vmcnt 0)
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // natural order: unit (4t + kk) of row c = dy[row0 + 16 rb + c][128 ch + 32t + 8kk .. + 7]
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const uint4_t* stage = reinterpret_cast<const uint4_t*>(&red[rb][wave][0]);
+#pragma unroll
+            for (int t = 0; t < NSTEP; ++t) av[rb][t] = __builtin_bit_cast(half8_t, stage[c * 16 + ((4 * t + kk) ^ c)]);
+        }
+        // the tile has been read (lgkmcnt 0): the next chunk of this wavefront may overwrite it
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_sched_barrier(0);
+        fetch_tile(ch + NW);
+        static_for_dx<0, NH>([&](auto hc) {
+            constexpr int h = decltype(hc)::value;
+            if constexpr (h + 1 < NH) load_stage(buf[(h + 1) & 1], ch, h + 1);
+            else load_stage(buf[0], ch + NW, 0);                // NH is even: the next chunk starts in buf[0] again
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(buf[h & 1], hc);
+        });
+    }
+    // the prefetch past the last chunk may still be writing the tile: landed before the sums reuse the memory
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+    // sums 64 outputs of the block over the wavefronts: local column lc = 4c + jj stands for output
+    // 128*blk + 8*(lc / 4) + 4*hf + lc % 4; acc[rb][4*hf + jj][r] is row row0 + 16*rb + 4*kk + r
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float4_t v;
+#pragma unroll
+                for (int jj = 0; jj < 4; ++jj) v[jj] = acc[rb][4 * hf + jj][r] - corr[rb][r];
+                *reinterpret_cast<float4_t*>(&red[rb][wave][((4 * kk + r) << 6) + 4 * c]) = v;
+            }
+        __syncthreads();
+        {
+            const int e = 2 * threadIdx.x;
+            const int row = e >> 6, lc = e & 63;
+            const int cc = (blk << 7) + 8 * (lc >> 2) + 4 * hf + (lc & 3);
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) {
+                    const float* rp = &red[rb][w][e];
+                    v0 += rp[0];
+                    v1 += rp[1];
+                }
+                const int m = row0 + 16 * rb + row;
+                if (m < a.M) {
+                    const half2_t hv = {(half_t)v0, (half_t)v1};
+                    *reinterpret_cast<half2_t*>(a.dx + (size_t)m * a.K + cc) = hv;
+                }
+            }
+        }
+        __syncthreads();
+    }
+}
+
 // ------------------------------------------------------------------ act-order (per-row groups)
 template <int NSTEP>
 __global__ __launch_bounds__(512) void gemv_gidx_kernel(GemvArgs a) {
@@ -1375,6 +1556,48 @@ extern "C" int q4_launch_stream_fwd(const void* x, const int32_t* qweight, const
     if (rb == 2) hipLaunchKernelGGL(stream_fwd_kernel<2>, grid, block, 0, stream, a);
     else if (rb == 3) hipLaunchKernelGGL(stream_fwd_kernel<3>, grid, block, 0, stream, a);
     else hipLaunchKernelGGL(stream_fwd_kernel<4>, grid, block, 0, stream, a);
+    return hipGetLastError() == hipSuccess ? 0 : -4;
+}
+
+// Shapes the whole-reduction grad-input kernel takes: as q4_stream_fwd_applicable, with blocks of 128 outputs and row
+// blocks of 32 or 48 rows (the accumulators of 64 rows do not fit the registers).  Measured, 49..256 rows: 4096 x 4096
+// 15.5-17.3 against 15.5-24.8 us, 2048 x 2048 10 against 12-18.5 us, 4096 outputs over 1024 columns 7.6 against 11-18 us,
+// 11008 outputs over 4096 columns (up to 96 rows) 18-21 against 28-32 us.
+static int stream_dx_row_blocks(int M, int K) {
+    static const int force_rb = getenv("Q4_STREAM_DX_RB") ? atoi(getenv("Q4_STREAM_DX_RB")) : 0;
+    if (force_rb >= 2 && force_rb <= 3) return force_rb;
+    const int blocks = K / 128;
+    for (int rb = 2; rb <= 3; ++rb)
+        if (blocks * ((M + 16 * rb - 1) / (16 * rb)) <= 256) return rb;
+    return 0;
+}
+extern "C" int q4_stream_dx_applicable(int M, int K, int N, int groupsize, int has_gidx) {
+    static const int max_rows = getenv("Q4_STREAM_DX_MAX_ROWS") ? atoi(getenv("Q4_STREAM_DX_MAX_ROWS")) : 512;
+    if (!(M > 48 && M <= max_rows && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 128 == 0))
+        return 0;
+    // a workgroup walks the whole reduction alone: with a long reduction and few output blocks (4096 outputs over 11008
+    // columns: 38-42 us against 24-38 us) the tiled kernel with its split reduction is faster
+    return N <= 2 * K && stream_dx_row_blocks(M, K) != 0;
+}
+
+extern "C" int q4_launch_stream_dx(const void* dy, const int32_t* qweight, const int32_t* qzeros, const void* scales,
+                                   int groupsize, void* dx, int M, int K, int N, int G, hipStream_t stream) {
+    using namespace q4;
+    SkinnyDxArgs a;
+    a.dy = reinterpret_cast<const half_t*>(dy);
+    a.qweight = reinterpret_cast<const uint32_t*>(qweight);
+    a.qzeros = reinterpret_cast<const uint32_t*>(qzeros);
+    a.scales = reinterpret_cast<const half_t*>(scales);
+    a.groupsize = groupsize;
+    a.dx = reinterpret_cast<half_t*>(dx);
+    a.part = nullptr;
+    a.M = M; a.K = K; a.N = N; a.G = G;
+    a.strips_per_wg = 1;
+    const int rb = stream_dx_row_blocks(M, K);
+    if (rb == 0) return -2;
+    const dim3 grid(K / 128, 1, (M + 16 * rb - 1) / (16 * rb)), block(512);
+    if (rb == 2) hipLaunchKernelGGL((stream_dx_kernel<2, 2>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((stream_dx_kernel<3, 1>), grid, block, 0, stream, a);
     return hipGetLastError() == hipSuccess ? 0 : -4;
 }
 

@@ -269,6 +269,30 @@ def test_gemm_forward_65_to_512_rows_whole_reduction_streaming_kernel(oracle, M,
     assert not lib.q4_stream_fwd_applicable(M, K, N, gs, 1) and not lib.q4_stream_fwd_applicable(64, K, N, gs, 0)
 
 
+@pytest.mark.parametrize("M", [49, 64, 65, 96, 100, 128, 129, 192, 200, 256, 300, 512])
+@pytest.mark.parametrize("K,N,gs", [(4096, 4096, 128), (256, 1408, 128), (384, 512, 128), (1024, 11008, 128),
+                                    (2048, 1024, 1024), (128, 128, 128)])
+def test_gemm_grad_input_49_to_512_rows_whole_reduction_streaming_kernel(oracle, M, K, N, gs):
+    """Grad-input counterpart: one block of 128 outputs of 32 or 48 rows per workgroup over the whole reduction (11 and
+    86 chunks of 128 columns: uneven shares of the eight wavefronts; 1 and 4 chunks: idle wavefronts), row blocks cut
+    off by M.  Shapes of this list with more row blocks than one round of workgroups holds take the tiled kernel."""
+    import torch
+    from alpaca_lora_4bit_amd import _lib, quant_hip
+    layer = oracle.make_layer(K, N, gs, seed=K + N + M + 1)
+    t = to_cuda_layer(layer)
+    dy = oracle.make_activations(M, N, seed=M + 17)
+    ref = oracle.matmul_recons_t(dy, layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
+    dx = quant_hip.gemm_bwd_dx(torch.from_numpy(dy).cuda(), t["qweight"], t["qzeros"], t["scales"], None, gs)
+    dx2 = quant_hip.gemm_bwd_dx(torch.from_numpy(dy).cuda(), t["qweight"], t["qzeros"], t["scales"], None, gs)
+    assert dx.shape == (M, K) and torch.equal(dx, dx2)
+    assert np.abs(dx.float().cpu().numpy() - ref).max() <= 1e-2 * np.abs(ref).max()
+    assert np.abs(dx.float().cpu().numpy() - ref).max() <= 2e-3 * np.abs(ref).max()
+    lib = _lib.lib()
+    rb = next((rb for rb in (2, 3) if (K // 128) * -(-M // (16 * rb)) <= 256), 0)
+    assert bool(lib.q4_stream_dx_applicable(M, K, N, gs, 0)) == (rb != 0 and N <= 2 * K)
+    assert not lib.q4_stream_dx_applicable(M, K, N, gs, 1) and not lib.q4_stream_dx_applicable(48, K, N, gs, 0)
+
+
 @pytest.mark.parametrize("act", [False, True])
 @pytest.mark.parametrize("M,red,nout,tail_cols,tail_splits", [(1024, 1024, 11136, 23, 2), (520, 1024, 11008, 1, 2),
                                                               (1536, 4096, 11008, 1, 8)])
