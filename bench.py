@@ -423,6 +423,15 @@ def bench_gemm_only(M, K, N, act_order, reps, seed=7):
     return res
 
 
+def bench_mid_rows(reps):
+    """Forward and grad-input products at 128 and 256 rows, 4096 x 4096 and the MLP shapes."""
+    mid = {}
+    for (M, K, N) in ((128, 4096, 4096), (256, 4096, 4096), (256, 4096, 11008), (256, 11008, 4096)):
+        r = bench_gemm_only(M, K, N, False, reps)
+        mid[f"M{M}_K{K}_N{N}"] = {"fwd_us": round(r["fwd"]["us"], 2), "bwd_dx_us": round(r["bwd_dx"]["us"], 2)}
+    return mid
+
+
 def cpu_baseline(seconds_budget=20.0):
     """Torch-CPU restatement of the reference's recons+matmul on the same workload shapes
     (one MLP: gate, up, down at M=1), repeated until ~seconds_budget of CPU time is spent."""
@@ -478,6 +487,8 @@ def main():
                     help="run only the greedy decode of the random-init 4-bit LLaMA-7B through transformers' generate")
     ap.add_argument("--dequant-only", action="store_true",
                     help="run only the dense dequantization of a 4096x11008 layer (short run for profiling)")
+    ap.add_argument("--mid-rows-only", action="store_true",
+                    help="only the 128- and 256-row products (for profiling runs)")
     ap.add_argument("--lora-step-only", action="store_true",
                     help="run only the config-2 LoRA layer step (forward + backward, M=2048) and print its figures: "
                          "a short run for profiling the GEMM and adapter kernels")
@@ -503,6 +514,9 @@ def main():
     if args.dequant_only:
         r = bench_dequant(4096, 11008, False, max(args.steps, 5))
         print(json.dumps({"workload": "dense_dequant_K4096_N11008", **{k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()}}))
+        return
+    if args.mid_rows_only:
+        print(json.dumps({"workload": "gemm_some_hundred_rows", **bench_mid_rows(max(args.steps, 5))}))
         return
     if args.lora_step_only:
         r = bench_lora_step(max(args.steps, 5))
@@ -585,6 +599,9 @@ def main():
         extra["config2_gemm_kernels"] = {k: {kk: round(vv, 4) for kk, vv in v.items()} for k, v in gm.items()}
         g3 = bench_gemm_only(512, 5120, 13824, True, 10)
         extra["config3_actorder_M512"] = {k: {kk: round(vv, 4) for kk, vv in v.items()} for k, v in g3.items()}
+        # between the decode and the training shapes: 128 and 256 rows (a short prompt; the reference's default
+        # micro-batch of one 256-token sample) on the 4096 x 4096 projections and the MLP shapes
+        extra["gemm_some_hundred_rows"] = bench_mid_rows(20)
         try:
             with contextlib.redirect_stdout(sys.stderr):
                 c4 = bench_llama7b_lora_train_step(4)
