@@ -673,6 +673,11 @@ void stream_fwd_kernel(SkinnyArgs a) {
         for (int t = 0; t < NSTEP; ++t) w1[t] = buf_load128_stream(rw, vw, off + (ch << 4) * a.N * 4 + t * wstep);
     };
     fetch(wave);
+    // mask (scalar register) and magic number (vector register) as opaque values: with two literals the compiler
+    // emits an AND and an OR, with register operands the single three-operand and-or instruction
+    uint32_t m_lo = 0x000F000Fu, m_hi = 0x00F000F0u, g_lo = 0x64006400u, g_hi = 0x54005400u;
+    asm volatile("" : "+s"(m_lo), "+s"(m_hi));
+    asm volatile("" : "+v"(g_lo), "+v"(g_hi));
 
     float4_t acc[RB][4];
 #pragma unroll
@@ -724,10 +729,10 @@ void stream_fwd_kernel(SkinnyArgs a) {
             for (int j = 0; j < 4; ++j) {
                 // a code in mantissa bits 0..3 of fp16 1024.0 reads 1024 + q, in bits 4..7 of fp16 64.0 it reads 64 + q
                 const uint32_t hi = w[j] >> 8;
-                const half2_t b0 = __builtin_elementwise_fma(as_half2((w[j] & 0x000F000Fu) | 0x64006400u), s2[j], -s1024[j]) - zero2[j];
-                const half2_t b1 = __builtin_elementwise_fma(as_half2((w[j] & 0x00F000F0u) | 0x54005400u), s2[j], -s64[j]) - zero2[j];
-                const half2_t b2 = __builtin_elementwise_fma(as_half2((hi & 0x000F000Fu) | 0x64006400u), s2[j], -s1024[j]) - zero2[j];
-                const half2_t b3 = __builtin_elementwise_fma(as_half2((hi & 0x00F000F0u) | 0x54005400u), s2[j], -s64[j]) - zero2[j];
+                const half2_t b0 = __builtin_elementwise_fma(as_half2((w[j] & m_lo) | g_lo), s2[j], -s1024[j]) - zero2[j];
+                const half2_t b1 = __builtin_elementwise_fma(as_half2((w[j] & m_hi) | g_hi), s2[j], -s64[j]) - zero2[j];
+                const half2_t b2 = __builtin_elementwise_fma(as_half2((hi & m_lo) | g_lo), s2[j], -s1024[j]) - zero2[j];
+                const half2_t b3 = __builtin_elementwise_fma(as_half2((hi & m_hi) | g_hi), s2[j], -s64[j]) - zero2[j];
                 const half8_t bv = make_half8(as_u32(b0), as_u32(b1), as_u32(b2), as_u32(b3));
 #pragma unroll
                 for (int rb = 0; rb < RB; ++rb)
@@ -1064,6 +1069,10 @@ void stream_dx_kernel(SkinnyDxArgs a) {
         for (int j = 0; j < 8; ++j) acc[rb][j] = float4_t{0.f, 0.f, 0.f, 0.f};
     }
     half8_t av[RB][NSTEP];
+    // mask in a scalar, magic number in a vector register (opaque): one and-or instruction instead of AND + OR
+    uint32_t m_lo = 0x000F000Fu, g_lo = kMagic;
+    asm volatile("" : "+s"(m_lo));
+    asm volatile("" : "+v"(g_lo));
     auto multiply = [&](const Stage& st, auto htag) {
         constexpr int h = decltype(htag)::value;
 #pragma unroll
@@ -1093,8 +1102,8 @@ void stream_dx_kernel(SkinnyDxArgs a) {
                 for (int p = 0; p < 4; ++p) {
                     const uint32_t sel = 0x0c000c00u | ((4u + b) << 16) | (uint32_t)b;
                     const uint32_t pb = __builtin_amdgcn_perm(wd[2 * p + 1], wd[2 * p], sel);   // byte b of columns 2p, 2p+1
-                    ev[p] = (pb & 0x000F000Fu) | kMagic;
-                    od[p] = ((pb >> 4) & 0x000F000Fu) | kMagic;
+                    ev[p] = (pb & m_lo) | g_lo;
+                    od[p] = ((pb >> 4) & m_lo) | g_lo;
                 }
                 const half8_t be = make_half8(ev[0], ev[1], ev[2], ev[3]), bo = make_half8(od[0], od[1], od[2], od[3]);
 #pragma unroll
