@@ -173,8 +173,12 @@ int q4_dropout_keep_u8(uint8_t *keep, int M, int C, const q4_dropout_t *drop, vo
  * multiply-add on 1024+q; pass g_idx to lift the restriction on the scales).
  * `workspace` (optional, may be NULL; 256-byte aligned, contents irrelevant): with few output tiles (small M),
  * and for the tiles of a last round that would fill at most half of the CUs, the reduction is split over
- * several workgroups per tile that leave fp32 partial tiles in it, added in a fixed order by a second kernel.  q4_gemm_workspace_bytes(fwd, M, K, N) is the size that allows the
- * preferred split (0 when none is wanted); a smaller workspace means fewer splits, none means no split. */
+ * several workgroups per tile that leave fp32 partial tiles in it, added in a fixed order by a second kernel.
+ * q4_gemm_workspace_bytes(fwd, M, K, N) is the size that allows the preferred split (0 when none is wanted); a
+ * smaller workspace means fewer splits, none means no split.  Products without adapter term on sequential groups
+ * of a multiple of 128 rows take weight-streaming kernels where those are faster: 17..64 rows (grad-input: 17..48)
+ * with partial rows in the workspace, and some hundred rows of an output that one round of workgroups covers as a
+ * single launch without workspace.  Every route returns the same values for the same inputs on every call. */
 size_t q4_gemm_workspace_bytes(int fwd, int M, int K, int N);
 int q4_gemm_fwd_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                     const int32_t *g_idx, int groupsize, const void *bias,
