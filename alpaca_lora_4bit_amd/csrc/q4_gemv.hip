@@ -1538,6 +1538,7 @@ extern "C" int q4_stream_fwd_applicable(int M, int K, int N, int groupsize, int 
     static const int max_rows = getenv("Q4_STREAM_FWD_MAX_ROWS") ? atoi(getenv("Q4_STREAM_FWD_MAX_ROWS")) : 512;
     if (!(M > 64 && M <= max_rows && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 64 == 0))
         return 0;
+    if (K > 65536 || N > 65536 || (long)K * N > (1L << 28)) return 0;      // 32-bit byte offsets, far offset included
     // very long reductions with the larger row blocks: level with the tiled kernel or just behind (13824 -> 5120)
     const int rb = stream_fwd_row_blocks(M, N);
     return rb == 2 || (rb > 2 && K <= 12288);
@@ -1584,6 +1585,7 @@ extern "C" int q4_stream_dx_applicable(int M, int K, int N, int groupsize, int h
     static const int max_rows = getenv("Q4_STREAM_DX_MAX_ROWS") ? atoi(getenv("Q4_STREAM_DX_MAX_ROWS")) : 512;
     if (!(M > 48 && M <= max_rows && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 128 == 0))
         return 0;
+    if (K > 65536 || N > 65536 || (long)K * N > (1L << 28)) return 0;      // 32-bit byte offsets, far offset included
     // a workgroup walks the whole reduction alone: with a long reduction and few output blocks (4096 outputs over 11008
     // columns: 38-42 us against 24-38 us) the tiled kernel with its split reduction is faster
     return N <= 2 * K && stream_dx_row_blocks(M, K) != 0;
