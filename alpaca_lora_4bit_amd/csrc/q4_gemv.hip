@@ -1520,9 +1520,9 @@ extern "C" int q4_launch_skinny(const void* x, const int32_t* qweight, const int
 }
 
 // Shapes the whole-reduction streaming kernel takes: more than 64 rows, sequential groups that are multiples of 128
-// rows, and an output small enough for ONE round of workgroups (at most one per CU): the kernel is bound by the
-// activation tiles every workgroup pulls through its CU's vector memory path, so a second round costs as much as the
-// first, while the tiled kernel only gets better with more tiles (measured on 4096 x 4096, 65..256 rows: 10.2-16.1 us
+// rows, and an output small enough for ONE round of workgroups (at most one per CU): the kernel is bound per CU (the
+// vector-ALU work of the operand build, the activation tiles every wavefront pulls), so a second round costs as much as
+// the first, while the tiled kernel only gets better with more tiles (measured on 4096 x 4096, 65..256 rows: 10.2-16.1 us
 // against 16.1-24.4 us; 2048 x 2048, 65..512 rows: 7-10.6 against 12.3-22.3 us; 11008 -> 4096, up to 192 rows: 22-31
 // against 22-34 us; 4096 -> 11008 never fits one round).
 // Row blocks of 32, 48 or 64 rows: the smallest that fits (more workgroups, fewer idle CUs).
