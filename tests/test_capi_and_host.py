@@ -124,6 +124,30 @@ def test_error_codes_and_validation_need_no_gpu():
     assert L.q4_gemv_workspace_bytes(0, 4096, 11008) == 0
 
 
+def test_streaming_kernel_selection_rules_need_no_gpu():
+    """Which products of some hundred rows take the whole-reduction streaming kernels (host logic only): outputs that
+    one round of at most 256 workgroups covers with row blocks of 32, 48 or 64 rows (grad-input: 32 or 48), sequential
+    groups of a multiple of 128 rows, no act-order; the grad-input form only while the reduction is at most twice the
+    output width; very long reductions only with the smallest row block."""
+    from alpaca_lora_4bit_amd import _lib
+    L = _lib.lib()
+    fwd, dx = L.q4_stream_fwd_applicable, L.q4_stream_dx_applicable
+    # (M, K, N, groupsize, has_gidx)
+    assert fwd(128, 4096, 4096, 128, 0) and fwd(256, 4096, 4096, 128, 0) and fwd(65, 4096, 4096, 128, 0)
+    assert not fwd(64, 4096, 4096, 128, 0)            # up to 64 rows: the other streaming kernel
+    assert not fwd(257, 4096, 4096, 128, 0)           # 64 strips x 5 blocks of 64 rows
+    assert not fwd(128, 4096, 11008, 128, 0)          # 172 strips never fit one round above 64 rows
+    assert fwd(192, 11008, 4096, 128, 0) and fwd(512, 2048, 2048, 128, 0) and not fwd(513, 2048, 2048, 128, 0)
+    assert not fwd(128, 4096, 4096, 128, 1) and not fwd(128, 4096, 4096, 64, 0) and not fwd(128, 4096 + 64, 4096, 128, 0)
+    assert fwd(65, 13824, 5120, 128, 0) and not fwd(128, 13824, 5120, 128, 0)     # long reduction: 32-row blocks only
+    assert dx(49, 4096, 4096, 128, 0) and dx(256, 4096, 4096, 128, 0) and dx(384, 4096, 4096, 128, 0)
+    assert not dx(48, 4096, 4096, 128, 0) and not dx(385, 4096, 4096, 128, 0)     # 32 blocks x 9 blocks of 48 rows
+    assert dx(96, 11008, 4096, 128, 0) and not dx(97, 11008, 4096, 128, 0)        # 86 blocks x 2 / x 3
+    assert not dx(128, 4096, 11008, 128, 0)           # reduction over 11008 columns for 4096 outputs
+    assert not dx(128, 4096, 4096, 128, 1) and not dx(128, 4096, 4096, 64, 0)
+    assert not fwd(128, 131072, 4096, 128, 0) and not dx(128, 4096, 131072, 128, 0)   # beyond the 32-bit offsets
+
+
 def test_compiled_host_binding_is_built_and_matches_the_library():
     """The pybind11 host module (csrc/host/q4_host.cpp) sits next to the library, was built against the same ABI
     version, and quant_hip routes its operators through it.  Its argument checks run without a GPU."""
