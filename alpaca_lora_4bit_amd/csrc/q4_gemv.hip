@@ -1519,8 +1519,8 @@ extern "C" int q4_launch_skinny(const void* x, const int32_t* qweight, const int
     return 0;
 }
 
-// Shapes the whole-reduction streaming kernel takes: more than 64 rows, sequential groups that are multiples of 128
-// rows, and an output small enough for ONE round of workgroups (at most one per CU): the kernel is bound per CU (the
+// Shapes the whole-reduction streaming kernel takes: more than 64 rows (from 17 rows on wide outputs), sequential groups
+// that are multiples of 128 rows, and an output small enough for ONE round of workgroups (at most one per CU): the kernel is bound per CU (the
 // vector-ALU work of the operand build, the activation tiles every wavefront pulls), so a second round costs as much as
 // the first, while the tiled kernel only gets better with more tiles (measured on 4096 x 4096, 65..256 rows: 10.2-16.1 us
 // against 16.1-24.4 us; 2048 x 2048, 65..512 rows: 7-10.6 against 12.3-22.3 us; 11008 -> 4096, up to 192 rows: 22-31
@@ -1536,8 +1536,12 @@ static int stream_fwd_row_blocks(int M, int N) {
 }
 extern "C" int q4_stream_fwd_applicable(int M, int K, int N, int groupsize, int has_gidx) {
     static const int max_rows = getenv("Q4_STREAM_FWD_MAX_ROWS") ? atoi(getenv("Q4_STREAM_FWD_MAX_ROWS")) : 512;
-    if (!(M > 64 && M <= max_rows && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 64 == 0))
+    if (!(M > 16 && M <= max_rows && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 64 == 0))
         return 0;
+    // up to 64 rows there is one row block, i.e. one workgroup per strip: worth it from 128 strips on, where it beats
+    // the kernel with the split reduction and the second launch (4096 -> 11008 at 17..64 rows: 9.7-14.7 against
+    // 14.5-18.1 us, 5120 -> 13824: 11.9-17.7 against 18.5-35.2 us; at 64 strips it loses, 4096 x 4096: 9.7-10.4 against 8.7-10.8 us)
+    if (M <= 64 && N < 8192) return 0;
     if (K > 65536 || N > 65536 || (long)K * N > (1L << 28)) return 0;      // 32-bit byte offsets, far offset included
     // very long reductions with the larger row blocks: level with the tiled kernel or just behind (13824 -> 5120)
     const int rb = stream_fwd_row_blocks(M, N);
@@ -1570,7 +1574,8 @@ extern "C" int q4_launch_stream_fwd(const void* x, const int32_t* qweight, const
 }
 
 // Shapes the whole-reduction grad-input kernel takes: as q4_stream_fwd_applicable, with blocks of 128 outputs and row
-// blocks of 32 or 48 rows (the accumulators of 64 rows do not fit the registers).  Measured, 49..256 rows: 4096 x 4096
+// blocks of 32 or 48 rows (the accumulators of 64 rows do not fit the registers); below 49 rows skinny_dx_kernel is
+// faster on every shape measured (e.g. 8192 x 8192 at 17..48 rows: 15-18 against 28-30 us).  Measured, 49..256 rows: 4096 x 4096
 // 15.5-17.3 against 15.5-24.8 us, 2048 x 2048 10 against 12-18.5 us, 4096 outputs over 1024 columns 7.6 against 11-18 us,
 // 11008 outputs over 4096 columns (up to 96 rows) 18-21 against 28-32 us.
 static int stream_dx_row_blocks(int M, int K) {

@@ -134,7 +134,9 @@ def test_streaming_kernel_selection_rules_need_no_gpu():
     fwd, dx = L.q4_stream_fwd_applicable, L.q4_stream_dx_applicable
     # (M, K, N, groupsize, has_gidx)
     assert fwd(128, 4096, 4096, 128, 0) and fwd(256, 4096, 4096, 128, 0) and fwd(65, 4096, 4096, 128, 0)
-    assert not fwd(64, 4096, 4096, 128, 0)            # up to 64 rows: the other streaming kernel
+    assert not fwd(64, 4096, 4096, 128, 0)            # up to 64 rows and fewer than 128 strips: the other streaming kernel
+    assert fwd(17, 4096, 11008, 128, 0) and fwd(64, 5120, 13824, 128, 0) and not fwd(16, 4096, 11008, 128, 0)
+    assert not fwd(40, 4096, 16512, 128, 0)           # 258 strips
     assert not fwd(257, 4096, 4096, 128, 0)           # 64 strips x 5 blocks of 64 rows
     assert not fwd(128, 4096, 11008, 128, 0)          # 172 strips never fit one round above 64 rows
     assert fwd(192, 11008, 4096, 128, 0) and fwd(512, 2048, 2048, 128, 0) and not fwd(513, 2048, 2048, 128, 0)

@@ -227,7 +227,7 @@ def test_gemm_forward_17_to_64_rows(oracle, M, K, N, gs, act):
 def test_gemm_forward_streaming_kernel_several_strips_per_workgroup(oracle, M, K, N):
     """Wide outputs: a workgroup of the streaming kernel walks over 2 or 3 neighbouring 64-column strips with the
     activations held in registers; 16512 and 24704 columns (258 and 386 strips, 4 and 3 per workgroup) leave the
-    last workgroup two strips."""
+    last workgroup two strips.  (11008 columns = 172 strips take the whole-reduction kernel: one workgroup per strip.)"""
     import torch
     from alpaca_lora_4bit_amd import quant_hip
     layer = oracle.make_layer(K, N, 128, seed=K + N + M)
@@ -267,6 +267,24 @@ def test_gemm_forward_65_to_512_rows_whole_reduction_streaming_kernel(oracle, M,
     rb = next((rb for rb in (2, 3, 4) if strips * -(-M // (16 * rb)) <= 256), 0)
     assert bool(lib.q4_stream_fwd_applicable(M, K, N, gs, 0)) == (rb == 2 or (rb > 2 and K <= 12288))
     assert not lib.q4_stream_fwd_applicable(M, K, N, gs, 1) and not lib.q4_stream_fwd_applicable(64, K, N, gs, 0)
+
+
+@pytest.mark.parametrize("M", [17, 32, 33, 48, 49, 64])
+@pytest.mark.parametrize("K,N", [(512, 8192), (1408, 11008), (128, 16384)])
+def test_gemm_forward_17_to_64_rows_of_wide_outputs_whole_reduction_streaming_kernel(oracle, M, K, N):
+    """17..64 rows of an output with 128..256 strips: one workgroup per strip over the whole reduction (one row block of
+    32, 48 or 64 rows), instead of the split reduction with partial rows and a second kernel."""
+    import torch
+    from alpaca_lora_4bit_amd import _lib, quant_hip
+    layer = oracle.make_layer(K, N, 128, seed=K + N + M)
+    t = to_cuda_layer(layer)
+    x = oracle.make_activations(M, K, seed=M + 19)
+    ref = oracle.matmul_recons(x, layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
+    y = quant_hip.gemm_fwd(torch.from_numpy(x).cuda(), t["qweight"], t["qzeros"], t["scales"], None, 128)
+    y2 = quant_hip.gemm_fwd(torch.from_numpy(x).cuda(), t["qweight"], t["qzeros"], t["scales"], None, 128)
+    assert y.shape == (M, N) and torch.equal(y, y2)
+    assert np.abs(y.float().cpu().numpy() - ref).max() <= 2e-3 * np.abs(ref).max()
+    assert _lib.lib().q4_stream_fwd_applicable(M, K, N, 128, 0)
 
 
 @pytest.mark.parametrize("M", [49, 64, 65, 96, 100, 128, 129, 192, 200, 256, 300, 512])
