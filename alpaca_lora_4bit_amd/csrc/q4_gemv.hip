@@ -892,6 +892,10 @@ void skinny_dx_kernel(SkinnyDxArgs a) {
         }
     };
 
+    // mask in a scalar, magic number in a vector register (opaque): one and-or instruction instead of AND + OR
+    uint32_t m_lo = 0x000F000Fu, g_lo = kMagic;
+    asm volatile("" : "+s"(m_lo));
+    asm volatile("" : "+v"(g_lo));
     float4_t acc[RB][8], corr[RB];
     auto clear_acc = [&]() {
 #pragma unroll
@@ -930,8 +934,8 @@ void skinny_dx_kernel(SkinnyDxArgs a) {
                 for (int p = 0; p < 4; ++p) {
                     const uint32_t sel = 0x0c000c00u | ((4u + b) << 16) | (uint32_t)b;
                     const uint32_t pb = __builtin_amdgcn_perm(wd[2 * p + 1], wd[2 * p], sel);   // byte b of columns 2p, 2p+1
-                    ev[p] = (pb & 0x000F000Fu) | kMagic;
-                    od[p] = ((pb >> 4) & 0x000F000Fu) | kMagic;
+                    ev[p] = (pb & m_lo) | g_lo;
+                    od[p] = ((pb >> 4) & m_lo) | g_lo;
                 }
                 const half8_t be = make_half8(ev[0], ev[1], ev[2], ev[3]), bo = make_half8(od[0], od[1], od[2], od[3]);
 #pragma unroll
