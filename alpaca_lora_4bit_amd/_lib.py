@@ -6,7 +6,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libq4gptq.so")
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 _lib = None
 
@@ -17,6 +17,7 @@ SIGNATURES = {
     "q4_error_string": (ctypes.c_char_p, [_i]),
     "q4_dequant_f16": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp]),
     "q4_permute_rows": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
+    "q4_permute_cols_f16": (_i, [_vp, _vp, _vp, _i, _i, _vp]),
     "q4_gemv_workspace_bytes": (_sz, [_i, _i, _i]),
     "q4_gemv_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "q4_gemv_noalloc_max_outputs": (_sz, []),

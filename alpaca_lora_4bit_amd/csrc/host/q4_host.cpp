@@ -265,12 +265,24 @@ LoraPair check_lora(const c10::optional<at::Tensor>& la, const c10::optional<at:
     return p;
 }
 
+// out[m, p] = in[m, idx[p]]: activations gathered through the row sort of an act-order layer's weights (or grad_input
+// gathered back through the inverse permutation).  `idx` int32 [K] on the same device.
+at::Tensor permute_cols(const at::Tensor& in2, const at::Tensor& idx, void* stream) {
+    const int64_t M = in2.size(0), K = in2.size(1);
+    TORCH_CHECK_VALUE(idx.scalar_type() == at::kInt && idx.dim() == 1 && idx.size(0) == K && idx.is_contiguous() &&
+                      idx.device() == in2.device(), "the column index must be a contiguous int32 [K] tensor on the same device");
+    at::Tensor out = at::empty_like(in2);
+    const int rc = q4_permute_cols_f16(in2.data_ptr(), idx.data_ptr<int32_t>(), out.data_ptr(), (int)M, (int)K, stream);
+    if (rc != Q4_OK) raise_q4(rc, "q4_permute_cols_f16");
+    return out;
+}
+
 at::Tensor gemm_fwd(const at::Tensor& x, const at::Tensor& qweight, const at::Tensor& qzeros, const at::Tensor& scales,
                     const c10::optional<at::Tensor>& g_idx, int64_t groupsize, const c10::optional<at::Tensor>& bias,
                     const c10::optional<at::Tensor>& xa, const c10::optional<at::Tensor>& lora_bt, double lora_scale,
-                    const c10::optional<std::vector<int64_t>>& out_shape) {
+                    const c10::optional<std::vector<int64_t>>& out_shape, const c10::optional<at::Tensor>& in_perm) {
     const Layer l = check_layer(qweight, qzeros, scales, g_idx, groupsize);
-    const at::Tensor x2 = flat_half(x, l.K, l.device, "x");
+    at::Tensor x2 = flat_half(x, l.K, l.device, "x");
     const int64_t M = x2.size(0);
     if (M == 0) return at::empty(out_sizes(out_shape, 0, l.N), x2.options());
     const void* bp = nullptr;
@@ -282,6 +294,7 @@ at::Tensor gemm_fwd(const at::Tensor& x, const at::Tensor& qweight, const at::Te
     const LoraPair lp = check_lora(xa, lora_bt, M, l.N, l.device);
     at::Tensor o = at::empty(out_sizes(out_shape, M, l.N), x2.options());
     Launch L(l.device);
+    if (in_perm.has_value()) x2 = permute_cols(x2, *in_perm, L.stream);     // `qweight` holds the rows in that order
     size_t have = 0;
     void* ws = scratch_workspace(l.device, L.stream, q4_gemm_workspace_bytes(1, (int)M, l.K, l.N), &have);
     const int rc = q4_gemm_fwd_f16(x2.data_ptr(), l.qweight, l.qzeros, l.scales, l.g_idx, l.groupsize, bp, lp.la, lp.lb, lp.sr,
@@ -294,7 +307,7 @@ at::Tensor gemm_bwd_dx(const at::Tensor& dy, const at::Tensor& qweight, const at
                        const c10::optional<at::Tensor>& g_idx, int64_t groupsize, const c10::optional<at::Tensor>& dyb,
                        const c10::optional<at::Tensor>& lora_a, double lora_scale,
                        const c10::optional<std::vector<int64_t>>& out_shape,
-                       const c10::optional<std::pair<int64_t, double>>& dropout) {
+                       const c10::optional<std::pair<int64_t, double>>& dropout, const c10::optional<at::Tensor>& out_perm) {
     const Layer l = check_layer(qweight, qzeros, scales, g_idx, groupsize);
     const at::Tensor dy2 = flat_half(dy, l.N, l.device, "grad_output");
     const int64_t M = dy2.size(0);
@@ -310,6 +323,8 @@ at::Tensor gemm_bwd_dx(const at::Tensor& dy, const at::Tensor& qweight, const at
                                       lp.sc, lp.f32, (float)lora_scale, lp.R, o.data_ptr(), (int)M, l.K, l.N, l.G,
                                       has_drop ? &d : nullptr, ws, have, L.stream);
     if (rc != Q4_OK) raise_q4(rc, "q4_gemm_bwd_dx_f16");
+    if (out_perm.has_value())               // the rows of `qweight` are sorted: grad_input back into the original order
+        return permute_cols(o.view({M, (int64_t)l.K}), *out_perm, L.stream).view(o.sizes());
     return o;
 }
 
@@ -397,10 +412,10 @@ PYBIND11_MODULE(_q4_host, m) {
           py::arg("accumulate") = false);
     m.def("gemm_fwd", &gemm_fwd, py::arg("x"), py::arg("qweight"), py::arg("qzeros"), py::arg("scales"), py::arg("g_idx"),
           py::arg("groupsize"), py::arg("bias") = py::none(), py::arg("xa") = py::none(), py::arg("lora_bt") = py::none(),
-          py::arg("lora_scale") = 1.0, py::arg("out_shape") = py::none());
+          py::arg("lora_scale") = 1.0, py::arg("out_shape") = py::none(), py::arg("in_perm") = py::none());
     m.def("gemm_bwd_dx", &gemm_bwd_dx, py::arg("dy"), py::arg("qweight"), py::arg("qzeros"), py::arg("scales"), py::arg("g_idx"),
           py::arg("groupsize"), py::arg("dyb") = py::none(), py::arg("lora_a") = py::none(), py::arg("lora_scale") = 1.0,
-          py::arg("out_shape") = py::none(), py::arg("dropout") = py::none());
+          py::arg("out_shape") = py::none(), py::arg("dropout") = py::none(), py::arg("out_perm") = py::none());
     m.def("lora_down", &lora_down, py::arg("inp"), py::arg("w"), py::arg("dropout") = py::none());
     m.def("lora_grad_pair", &lora_grad_pair, py::arg("p1"), py::arg("inp1"), py::arg("p2"), py::arg("inp2"), py::arg("alpha"),
           py::arg("dropout") = py::none());

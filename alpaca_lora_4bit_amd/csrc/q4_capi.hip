@@ -7,6 +7,7 @@
 extern "C" {
 int q4_launch_dequant(const int32_t*, const int32_t*, const void*, const int32_t*, int, void*, int, int, hipStream_t);
 int q4_launch_permute_rows(const int32_t*, const int32_t*, int32_t*, int, int, hipStream_t);
+int q4_launch_permute_cols(const void*, const int32_t*, void*, int, int, hipStream_t);
 int q4_launch_gemv(const void*, const int32_t*, const int32_t*, const void*, const int32_t*, const int32_t*, int, void*,
                    int, int, int, int, int, void*, hipStream_t);
 struct q4_drop_args { uint32_t seed_lo, seed_hi, thr15; float scale; };     // q4::DropArgs of q4_common.hpp
@@ -60,7 +61,7 @@ int check_layer(const void* qweight, const void* qzeros, const void* scales, con
 }
 }  // namespace
 
-extern "C" int q4_abi_version(void) { return 10; }
+extern "C" int q4_abi_version(void) { return 11; }
 
 extern "C" const char* q4_error_string(int code) {
     switch (code) {
@@ -116,6 +117,14 @@ extern "C" int q4_permute_rows(const int32_t* qweight, const int32_t* perm, int3
     if ((reinterpret_cast<uintptr_t>(qweight) | reinterpret_cast<uintptr_t>(perm) | reinterpret_cast<uintptr_t>(out)) & 3u)
         return Q4_ERR_MISALIGNED;
     return q4_launch_permute_rows(qweight, perm, out, K, N, (hipStream_t)stream);
+}
+
+extern "C" int q4_permute_cols_f16(const void* in, const int32_t* idx, void* out, int M, int K, void* stream) {
+    if (!in || !idx || !out) return Q4_ERR_NULL_POINTER;
+    if (M < 1 || K < 8 || (K % 8) != 0 || K > 32768) return Q4_ERR_BAD_SHAPE;        // one row fits 64 KB of LDS
+    if (in == out) return Q4_ERR_BAD_SHAPE;                                          // not in place
+    if (misaligned(in) || misaligned(out) || misaligned(idx)) return Q4_ERR_MISALIGNED;
+    return q4_launch_permute_cols(in, idx, out, M, K, (hipStream_t)stream);
 }
 
 static int gemv_check(const void* x, const int32_t* qweight, const int32_t* qzeros, const void* scales,

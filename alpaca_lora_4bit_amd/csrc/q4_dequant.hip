@@ -76,6 +76,35 @@ __global__ __launch_bounds__(256) void permute_rows_kernel(const uint32_t* __res
     out[tid] = word;
 }
 
+// Column gather of an activation matrix: out[m, p] = in[m, idx[p]] (fp16, row-major [M, K]).  The companion of
+// permute_rows_kernel at run time: x is gathered through the row sort before a product with the sorted weights, and
+// grad_input is gathered back through the inverse permutation after it.  A workgroup stages `rows` whole rows in LDS
+// with coalesced 16-byte loads and gathers from there (two-byte gathers from global memory cost one cache-line lookup
+// per element), eight outputs per thread and row, written as 16-byte pieces.
+__global__ __launch_bounds__(256) void permute_cols_kernel(const half_t* __restrict__ in, const int32_t* __restrict__ idx,
+                                                           half_t* __restrict__ out, int M, int K, int rows) {
+    extern __shared__ __attribute__((aligned(16))) half_t srow[];      // [rows][K]
+    const int m0 = blockIdx.x * rows;
+    const int nr = min(rows, M - m0);
+    const int k8 = K >> 3;
+    for (int i = threadIdx.x; i < nr * k8; i += 256)
+        reinterpret_cast<uint4_t*>(srow)[i] = reinterpret_cast<const uint4_t*>(in + (size_t)m0 * K)[i];
+    __syncthreads();
+    for (int g = threadIdx.x; g < k8; g += 256) {
+        const uint4_t i0 = *reinterpret_cast<const uint4_t*>(idx + 8 * g);
+        const uint4_t i1 = *reinterpret_cast<const uint4_t*>(idx + 8 * g + 4);
+        const uint32_t src[8] = {i0.x, i0.y, i0.z, i0.w, i1.x, i1.y, i1.z, i1.w};
+        for (int r = 0; r < nr; ++r) {
+            const unsigned short* row = reinterpret_cast<const unsigned short*>(srow) + r * K;
+            uint32_t o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                o[e] = (uint32_t)row[min(src[2 * e], (uint32_t)(K - 1))] | ((uint32_t)row[min(src[2 * e + 1], (uint32_t)(K - 1))] << 16);
+            *reinterpret_cast<uint4_t*>(out + (size_t)(m0 + r) * K + 8 * g) = uint4_t{o[0], o[1], o[2], o[3]};
+        }
+    }
+}
+
 // v1 layout: one fp16 scale and one fp16 zero per column, W = rn16(rn16(s*q) - zero)
 // (src/alpaca_lora_4bit/quant_cuda/quant_cuda_kernel.cu:1076-1097).  Same thread mapping as dequant_kernel.
 __global__ __launch_bounds__(256) void dequant_v1_kernel(const uint32_t* __restrict__ qweight,
@@ -176,6 +205,17 @@ extern "C" int q4_launch_permute_rows(const int32_t* qweight, const int32_t* per
     const long total = (long)(K / 8) * N;
     hipLaunchKernelGGL(q4::permute_rows_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
                        reinterpret_cast<const uint32_t*>(qweight), perm, reinterpret_cast<uint32_t*>(out), K, N);
+    return hipGetLastError() == hipSuccess ? 0 : -4;
+}
+
+// Rows per workgroup: as many as 64 KB of LDS hold, fewer when that would leave CUs without a workgroup.
+extern "C" int q4_launch_permute_cols(const void* in, const int32_t* idx, void* out, int M, int K, hipStream_t stream) {
+    const int fit = (64 * 1024) / (K * 2);
+    if (fit < 1) return -2;
+    int rows = fit > 16 ? 16 : fit;
+    while (rows > 1 && (M + rows - 1) / rows < 512) --rows;
+    hipLaunchKernelGGL(q4::permute_cols_kernel, dim3((unsigned)((M + rows - 1) / rows)), dim3(256), (size_t)rows * K * 2, stream,
+                       reinterpret_cast<const q4::half_t*>(in), idx, reinterpret_cast<q4::half_t*>(out), M, K, rows);
     return hipGetLastError() == hipSuccess ? 0 : -4;
 }
 

@@ -190,6 +190,19 @@ def sorted_layer(qweight, g_idx, G):
     return plan
 
 
+def permute_cols(x, idx):
+    """out fp16 [M, K] with out[m, p] = x[m, idx[p]] (idx int32 [K]): the activations of an act-order layer gathered through
+    the row sort of its weights, or a grad_input gathered back through the inverse permutation."""
+    M, K = x.shape
+    if M == 0 or K % 8 or K > 32768 or x.data_ptr() % 16:
+        return x.index_select(1, idx)
+    out = torch.empty_like(x)
+    with _device_ctx(x.device):
+        rc = _lib.lib().q4_permute_cols_f16(x.data_ptr(), idx.data_ptr(), out.data_ptr(), M, K, _stream(x.device))
+    _lib.check(rc, "q4_permute_cols_f16")
+    return out
+
+
 def _actorder_plan(qweight, scales, g_idx, groupsize, G):
     """The sorted-copy plan when this call should use it, else None."""
     if g_idx is None or not actorder_repack:
@@ -475,7 +488,7 @@ def gemv(x, qweight, qzeros, scales, g_idx=None, groupsize=None, out=None, accum
         return out
     if plan is not None:
         perm, _, qweight, gs_sorted = plan
-        x2 = x2.index_select(1, perm)
+        x2 = permute_cols(x2, perm)
         gp, gs = 0, gs_sorted
     else:
         gp, gs = _gidx_arg(g_idx, groupsize, G)
@@ -578,6 +591,11 @@ def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, 
             gi, gs = info.gemm_args()
             return _host.gemm_fwd(x, qweight, qzeros, scales, gi, gs, bias, xa, lora_bt,
                                   float(lora_scale), _shape_arg(out_shape))
+        if info.K % 8 == 0 and info.K <= 32768:
+            # act-order layer with a sorted copy of its rows: x gathered through the sort, then sequential groups
+            perm, _, qsorted, gs_sorted = info.plan
+            return _host.gemm_fwd(x, qsorted, qzeros, scales, None, gs_sorted, bias, xa, lora_bt,
+                                  float(lora_scale), _shape_arg(out_shape), perm)
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     x2 = _flat_half(x, K, dev, "x")
     M = x2.shape[0]
@@ -590,7 +608,7 @@ def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, 
     plan = _actorder_plan(qweight, scales, g_idx, groupsize, G)
     if plan is not None:
         perm, _, qweight, gs_sorted = plan
-        x2 = x2.index_select(1, perm)
+        x2 = permute_cols(x2, perm)
         gp, gs = 0, gs_sorted
     else:
         gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
@@ -659,6 +677,11 @@ def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=Non
             return _host.gemm_bwd_dx(dy, qweight, qzeros, scales, gi, gs, dyb, lora_a,
                                      float(lora_scale), _shape_arg(out_shape),
                                      None if dropout is None else (int(dropout[0]), float(dropout[1])))
+        if dyb is None and info.K % 8 == 0 and info.K <= 32768:
+            # act-order layer, no adapter term: grad_input in sorted order, gathered back through the inverse permutation
+            _, inv, qsorted, gs_sorted = info.plan
+            return _host.gemm_bwd_dx(dy, qsorted, qzeros, scales, None, gs_sorted, None, None, 1.0,
+                                     _shape_arg(out_shape), None, inv)
     dev, K, N, G = _check_layer(qweight, qzeros, scales, g_idx, groupsize)
     dy2 = _flat_half(dy, N, dev, "grad_output")
     M = dy2.shape[0]
@@ -671,11 +694,11 @@ def gemm_bwd_dx(dy, qweight, qzeros, scales, g_idx=None, groupsize=None, dyb=Non
         if dropout is not None and dyb is not None:
             # the mask is indexed by the ORIGINAL column: add the masked adapter term after the scatter
             dx_sorted = gemm_bwd_dx(dy2, qs, qzeros, scales, None, gs_sorted)
-            dx = dx_sorted.index_select(1, inv)
+            dx = permute_cols(dx_sorted, inv)
             return dx.add_(masked_adapter_term(dyb, lora_a, lora_scale, dropout)).reshape(_out_shape(out_shape, M, K))
         la_sorted = None if lora_a is None else lora_a.index_select(1, perm)
         dx_sorted = gemm_bwd_dx(dy2, qs, qzeros, scales, None, gs_sorted, dyb=dyb, lora_a=la_sorted, lora_scale=lora_scale)
-        return dx_sorted.index_select(1, inv).reshape(_out_shape(out_shape, M, K))
+        return permute_cols(dx_sorted, inv).reshape(_out_shape(out_shape, M, K))
     dyb, lora_a, R, sr, sc, f32 = _lora_pair(dyb, lora_a, M, K, dev)
     gp, gs, _keepalive = _gemm_gidx_arg(g_idx, groupsize, G, K, scales)
     out = torch.empty(_out_shape(out_shape, M, K), dtype=torch.float16, device=dev)

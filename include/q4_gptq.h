@@ -70,6 +70,13 @@ int q4_dequant2_f16(const int32_t *qweight, const int32_t *qzeros, const void *s
  * the rows by group, gather x through the same permutation.  Not in place. */
 int q4_permute_rows(const int32_t *qweight, const int32_t *perm, int32_t *out, int K, int N, void *stream);
 
+/* Column gather of activations: out fp16 [M, K], out[m, p] = in[m, idx[p]] (idx int32 [K], values in 0..K-1; out of
+ * range values are clamped).  The run-time companion of q4_permute_rows: gather x through the row sort before a
+ * product with the sorted weights (idx = perm), gather grad_input back after it (idx = inverse permutation).  No
+ * counterpart in the reference (its kernels read g_idx per row instead).  K % 8 == 0, K <= 32768; in, out and idx
+ * 16-byte aligned; not in place. */
+int q4_permute_cols_f16(const void *in, const int32_t *idx, void *out, int M, int K, void *stream);
+
 /* Decode GEMV / skinny GEMM, 1 <= M <= 16:  y fp16 [M, N] = x fp16 [M, K] @ W  (fp32 accumulate).
  * If accumulate != 0 the product is added to the existing contents of y.
  * Replaces quant_cuda.vecquant4matmul / vecquant4matmul_faster / vecquant4matmul_old_faster

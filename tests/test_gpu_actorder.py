@@ -34,6 +34,29 @@ def test_permute_rows_bit_exact(oracle):
     assert _lib.lib().q4_permute_rows(qw.data_ptr(), qw.data_ptr(), qw.data_ptr(), K, N, None) == -2   # in place refused
 
 
+@pytest.mark.parametrize("M,K", [(1, 128), (7, 4096), (64, 4096), (300, 11008), (2049, 5120), (33, 32768), (1000, 256)])
+def test_permute_cols_bit_exact(M, K):
+    """q4_permute_cols_f16 through the C ABI: out[m, p] = in[m, idx[p]] for a permutation and for an index vector with
+    repeats (1, 2, 5, 16 rows per workgroup and a last workgroup with fewer); argument checks."""
+    import torch
+    from alpaca_lora_4bit_amd import _lib, quant_hip
+    g = torch.Generator().manual_seed(M + K)
+    x = torch.randn((M, K), generator=g).half().cuda()
+    L = _lib.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    for idx in (torch.randperm(K, generator=g).int().cuda(), torch.randint(0, K, (K,), generator=g).int().cuda()):
+        out = torch.full_like(x, float("nan"))
+        assert L.q4_permute_cols_f16(x.data_ptr(), idx.data_ptr(), out.data_ptr(), M, K, st) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), x.index_select(1, idx.long()).view(torch.int16))
+        assert torch.equal(quant_hip.permute_cols(x, idx).view(torch.int16), out.view(torch.int16))
+    assert L.q4_permute_cols_f16(x.data_ptr(), idx.data_ptr(), x.data_ptr(), M, K, st) == -2          # in place refused
+    assert L.q4_permute_cols_f16(x.data_ptr(), idx.data_ptr(), out.data_ptr(), M, K + 4, st) == -2      # K % 8
+    assert L.q4_permute_cols_f16(x.data_ptr(), idx.data_ptr(), out.data_ptr(), M, 32768 + 8, st) == -2  # a row must fit the LDS
+    assert L.q4_permute_cols_f16(None, idx.data_ptr(), out.data_ptr(), M, K, st) == -1
+    assert L.q4_permute_cols_f16(x.data_ptr() + 2, idx.data_ptr(), out.data_ptr(), M, K, st) == -5
+
+
 def test_sorted_layer_plan(oracle):
     """Sorted copy dequantizes (with sequential groups) to the row-permuted dense weight."""
     import torch
