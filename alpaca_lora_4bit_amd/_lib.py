@@ -27,6 +27,7 @@ SIGNATURES = {
     "q4_dequant_v1_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp]),
     "q4_dequant2_f16": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _vp]),
     "q4_gemm_workspace_bytes": (_sz, [_i, _i, _i, _i]),
+    "q4_gemm_route": (_i, [_i, _i, _i, _i, _i, _i]),
     "q4_gemm_fwd_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _f, _i, _vp, _i, _i, _i, _i, _vp, _sz, _vp]),
     "q4_gemm_bwd_dx_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _f, _i, _vp, _i, _i, _i, _i, _vp, _vp, _sz, _vp]),
     "q4_lora_down_f16": (_i, [_vp, _vp, _i, _i, _i, _vp, _i, _i, _i, _vp, _vp]),

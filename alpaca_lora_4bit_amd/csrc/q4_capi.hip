@@ -29,6 +29,10 @@ int q4_launch_gemv_group(int, const void* const*, const int32_t* const*, const i
 size_t q4_noalloc_scratch_bytes(void);
 void* q4_noalloc_scratch_ptr(int*);
 int q4_launch_zero_words(void*, size_t, hipStream_t);
+int q4_stream_fwd_applicable(int, int, int, int, int);
+int q4_stream_dx_applicable(int, int, int, int, int);
+int q4_skinny_applicable(int, int, int, int, int);
+int q4_skinny_dx_applicable(int, int, int, int, int);
 }
 
 namespace {
@@ -274,6 +278,20 @@ extern "C" int q4_gemm_bwd_dx_f16(const void* dy, const int32_t* qweight, const 
 extern "C" size_t q4_gemm_workspace_bytes(int fwd, int M, int K, int N) {
     if (M < 1 || K < 128 || N < 128) return 0;
     return q4_gemm_plan_workspace(fwd, M, K, N);
+}
+
+// The same tests, in the same order, as q4_launch_gemm applies to a product without adapter term.
+extern "C" int q4_gemm_route(int fwd, int M, int K, int N, int groupsize, int has_g_idx) {
+    if (M < 1 || K < 128 || N < 128 || (K % 128) != 0 || (N % 128) != 0) return Q4_ERR_BAD_SHAPE;
+    if (!has_g_idx && (groupsize < 1 || (groupsize % 64) != 0)) return Q4_ERR_BAD_SHAPE;
+    if (fwd) {
+        if (q4_stream_fwd_applicable(M, K, N, groupsize, has_g_idx)) return Q4_ROUTE_STREAM;
+        if (q4_skinny_applicable(M, K, N, groupsize, has_g_idx)) return Q4_ROUTE_SKINNY;
+    } else {
+        if (q4_stream_dx_applicable(M, K, N, groupsize, has_g_idx)) return Q4_ROUTE_STREAM;
+        if (q4_skinny_dx_applicable(M, K, N, groupsize, has_g_idx)) return Q4_ROUTE_SKINNY;
+    }
+    return Q4_ROUTE_TILED;
 }
 
 extern "C" int q4_lora_down_f16(const void* in, const void* w, int w_sr, int w_sc, int w_is_f32, void* out,

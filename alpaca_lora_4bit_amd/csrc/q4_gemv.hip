@@ -37,6 +37,7 @@
 // is independent of arrival order (bit-reproducible), and the whole exchange costs a single
 // memory round trip, with no fences and no spinning.
 #include "q4_common.hpp"
+#include "q4_gptq.h"
 #include <stdlib.h>
 #include <type_traits>
 

@@ -3,7 +3,7 @@
 
 Headline workload (configs[1] of the benchmark definition): LLaMA-7B MLP decode GEMVs at M=1 -- gate and up
 4096->11008, down 11008->4096, groupsize 128, no act-order.  One STEP = one token through the
-MLP GEMVs of all 32 decoder layers (96 launches over 2.25 GB of DISTINCT packed weights, so
+MLP GEMVs of all 32 decoder layers (64 launches: gate|up as one grouped launch + down, over 2.25 GB of DISTINCT packed weights, so
 nothing is served from the 256 MB Infinity Cache, exactly as in a real decode).  The step is
 captured once in a HIP graph and replayed; inputs and weights are resident in HBM.
 

@@ -28,6 +28,9 @@
 extern "C" {
 #endif
 
+/* The library is built with -fvisibility=hidden: the functions declared here are its whole exported set. */
+#define Q4_API __attribute__((visibility("default")))
+
 #define Q4_OK 0
 #define Q4_ERR_NULL_POINTER (-1)   /* a required pointer is NULL */
 #define Q4_ERR_BAD_SHAPE (-2)      /* a size violates the limits above / of the entry point */
@@ -38,29 +41,29 @@ extern "C" {
 #define Q4_ERR_RUNTIME (-7)        /* a HIP runtime call other than a launch failed */
 
 /* Library ABI version (bumped when a signature changes). */
-int q4_abi_version(void);
+Q4_API int q4_abi_version(void);
 
 /* Static string for a return code. */
-const char *q4_error_string(int code);
+Q4_API const char *q4_error_string(int code);
 
 /* Dense dequantization: out fp16 [K, N] = W.
  * Replaces quant_cuda.vecquant4recons_v2(mat, res, scales, zeros, g_idx)
  * (quant_cuda/quant_cuda.cpp:137-148, kernel quant_cuda/quant_cuda_kernel.cu:1127-1183).
  * Bit-exact with that kernel's fp16 instantiation. */
-int q4_dequant_f16(const int32_t *qweight, const int32_t *qzeros, const void *scales,
+Q4_API int q4_dequant_f16(const int32_t *qweight, const int32_t *qzeros, const void *scales,
                    const int32_t *g_idx, int groupsize, void *out,
                    int K, int N, int G, void *stream);
 
 /* Dense dequantization of the older "v1" layout: one fp16 scale and one fp16 zero per column
  * (scales, zeros: [N]),  W[k,n] = rn16( rn16(s[n]*q) - zero[n] ).
  * Replaces quant_cuda.vecquant4recons_v1 (quant_cuda/quant_cuda.cpp:131-135, kernel quant_cuda_kernel.cu:1076-1097). */
-int q4_dequant_v1_f16(const int32_t *qweight, const void *scales, const void *zeros, void *out,
+Q4_API int q4_dequant_v1_f16(const int32_t *qweight, const void *scales, const void *zeros, void *out,
                       int K, int N, void *stream);
 
 /* Dense dequantization of 2-bit v2 layers: qweight int32 [K/16, N] (sixteen codes per word along K),
  * qzeros int32 [G, N/16], scales fp16 [G, N], W = rn16( rn16(s*q) - rn16(s*(z+1)) ).  K % 16 == 0.
  * Replaces quant_cuda.vecquant2recons_v2 (quant_cuda/quant_cuda.cpp:150-161, kernel quant_cuda_kernel.cu:1185-1211). */
-int q4_dequant2_f16(const int32_t *qweight, const int32_t *qzeros, const void *scales,
+Q4_API int q4_dequant2_f16(const int32_t *qweight, const int32_t *qzeros, const void *scales,
                     const int32_t *g_idx, int groupsize, void *out, int K, int N, int G, void *stream);
 
 /* Row permutation of packed weights: out int32 [K/8, N] holds in row p the 4-bit codes of row perm[p]
@@ -68,14 +71,14 @@ int q4_dequant2_f16(const int32_t *qweight, const int32_t *qzeros, const void *s
  * it is the one-time repack that lets an act-order layer (rows assigned to groups through g_idx,
  * autograd_4bit.py:185, quant_cuda_kernel.cu:1143) run through the sequential-group kernels -- sort
  * the rows by group, gather x through the same permutation.  Not in place. */
-int q4_permute_rows(const int32_t *qweight, const int32_t *perm, int32_t *out, int K, int N, void *stream);
+Q4_API int q4_permute_rows(const int32_t *qweight, const int32_t *perm, int32_t *out, int K, int N, void *stream);
 
 /* Column gather of activations: out fp16 [M, K], out[m, p] = in[m, idx[p]] (idx int32 [K], values in 0..K-1; out of
  * range values are clamped).  The run-time companion of q4_permute_rows: gather x through the row sort before a
  * product with the sorted weights (idx = perm), gather grad_input back after it (idx = inverse permutation).  No
  * counterpart in the reference (its kernels read g_idx per row instead).  K % 8 == 0, K <= 32768; in, out and idx
  * 16-byte aligned; not in place. */
-int q4_permute_cols_f16(const void *in, const int32_t *idx, void *out, int M, int K, void *stream);
+Q4_API int q4_permute_cols_f16(const void *in, const int32_t *idx, void *out, int M, int K, void *stream);
 
 /* Decode GEMV / skinny GEMM, 1 <= M <= 16:  y fp16 [M, N] = x fp16 [M, K] @ W  (fp32 accumulate).
  * If accumulate != 0 the product is added to the existing contents of y.
@@ -87,8 +90,8 @@ int q4_permute_cols_f16(const void *in, const int32_t *idx, void *out, int M, in
  * `workspace` must hold q4_gemv_workspace_bytes(M, K, N) = 8*M*N bytes, 256-byte aligned, and must be
  * ZERO before its first use; every call leaves it zeroed again (it carries the fixed-point split-K
  * sums).  Calls sharing one workspace must be ordered on one stream.  K <= 1 044 480. */
-size_t q4_gemv_workspace_bytes(int M, int K, int N);
-int q4_gemv_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+Q4_API size_t q4_gemv_workspace_bytes(int M, int K, int N);
+Q4_API int q4_gemv_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                 const int32_t *g_idx, int groupsize, void *y, int accumulate,
                 int M, int K, int N, int G,
                 void *workspace, size_t workspace_bytes, void *stream);
@@ -111,8 +114,8 @@ typedef struct q4_gemv_layer {
     void *y;                   /* fp16 [M, N] */
     int N;
 } q4_gemv_layer_t;
-size_t q4_gemv_grouped_workspace_bytes(int M, int total_N);
-int q4_gemv_grouped_f16(const q4_gemv_layer_t *layers, int n_layers, int groupsize, int accumulate,
+Q4_API size_t q4_gemv_grouped_workspace_bytes(int M, int total_N);
+Q4_API int q4_gemv_grouped_f16(const q4_gemv_layer_t *layers, int n_layers, int groupsize, int accumulate,
                         int M, int K, void *workspace, size_t workspace_bytes, void *stream);
 
 /* q4_gemv_f16 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
@@ -123,8 +126,8 @@ int q4_gemv_grouped_f16(const q4_gemv_layer_t *layers, int n_layers, int groupsi
  * hipFree and no allocating library routine; it enqueues a small fill kernel that zeroes the accumulators and
  * then the same kernels as q4_gemv_f16, and gives bit-identical results.  All calls on one device share the
  * one array: calls that overlap on a device (two streams, two threads) race -- order them on one stream. */
-size_t q4_gemv_noalloc_max_outputs(void);
-int q4_gemv_noalloc_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+Q4_API size_t q4_gemv_noalloc_max_outputs(void);
+Q4_API int q4_gemv_noalloc_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                         const int32_t *g_idx, int groupsize, void *y, int accumulate,
                         int M, int K, int N, int G, void *stream);
 
@@ -136,7 +139,7 @@ int q4_gemv_noalloc_f16(const void *x, const int32_t *qweight, const int32_t *qz
  * x[:, perm[p]] itself, through LDS, while its weight loads are in flight, which replaces the separate gather
  * the caller would otherwise run before q4_gemv_f16.  The values are those of the reference's act-order
  * product (quant_cuda_kernel.cu:443-536 with per-row g_idx).  Workspace as for q4_gemv_f16. */
-int q4_gemv_sorted_f16(const void *x, const int32_t *qweight_sorted, const int32_t *qzeros, const void *scales,
+Q4_API int q4_gemv_sorted_f16(const void *x, const int32_t *qweight_sorted, const int32_t *qzeros, const void *scales,
                        const int32_t *perm, int groupsize, void *y, int accumulate,
                        int M, int K, int N, int G,
                        void *workspace, size_t workspace_bytes, void *stream);
@@ -146,7 +149,7 @@ int q4_gemv_sorted_f16(const void *x, const int32_t *qweight_sorted, const int32
  * Replaces quant_cuda.vecquant4matmul_v1_faster (quant_cuda/quant_cuda.cpp:163-175; kernel
  * quant_cuda_kernel.cu:1244-1302, launcher :1304-1335) as called from matmul_utils_4bit.py:36-56.
  * `scales`, `zeros` fp16 [N], 8-byte aligned.  Workspace as for q4_gemv_f16. */
-int q4_gemv_v1_f16(const void *x, const int32_t *qweight, const void *scales, const void *zeros, void *y,
+Q4_API int q4_gemv_v1_f16(const void *x, const int32_t *qweight, const void *scales, const void *zeros, void *y,
                    int accumulate, int M, int K, int N,
                    void *workspace, size_t workspace_bytes, void *stream);
 
@@ -163,8 +166,8 @@ typedef struct q4_dropout {
     uint32_t seed_lo, seed_hi;
     float p;
 } q4_dropout_t;
-float q4_dropout_scale(float p);
-int q4_dropout_keep_u8(uint8_t *keep, int M, int C, const q4_dropout_t *drop, void *stream);
+Q4_API float q4_dropout_scale(float p);
+Q4_API int q4_dropout_keep_u8(uint8_t *keep, int M, int C, const q4_dropout_t *drop, void *stream);
 
 /* Forward GEMM, any M >= 1:
  *   y fp16 [M, N] = x fp16 [M, K] @ W  (+ bias fp16 [N])  (+ lora_scale * xa fp16 [M, R] @ Bm [R, N])
@@ -186,8 +189,18 @@ int q4_dropout_keep_u8(uint8_t *keep, int M, int C, const q4_dropout_t *drop, vo
  * of a multiple of 128 rows take weight-streaming kernels where those are faster: 17..64 rows (grad-input: 17..48)
  * with partial rows in the workspace, and some hundred rows of an output that one round of workgroups covers as a
  * single launch without workspace.  Every route returns the same values for the same inputs on every call. */
-size_t q4_gemm_workspace_bytes(int fwd, int M, int K, int N);
-int q4_gemm_fwd_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+Q4_API size_t q4_gemm_workspace_bytes(int fwd, int M, int K, int N);
+
+/* Which kernel family the two GEMM entry points run for a product WITHOUT adapter term, given a workspace of
+ * q4_gemm_workspace_bytes(): Q4_ROUTE_TILED (dequantize-into-LDS MFMA tiles), Q4_ROUTE_SKINNY (17..64 rows, partial rows
+ * in the workspace), Q4_ROUTE_STREAM (some hundred rows, one launch without workspace), or a negative Q4_ERR_* code for
+ * a shape neither entry point takes.  A planning query for callers and tests; it launches nothing.  No counterpart in
+ * the reference, whose only route is recons + torch.matmul (matmul_utils_4bit.py:114-127). */
+#define Q4_ROUTE_TILED 0
+#define Q4_ROUTE_SKINNY 1
+#define Q4_ROUTE_STREAM 2
+Q4_API int q4_gemm_route(int fwd, int M, int K, int N, int groupsize, int has_g_idx);
+Q4_API int q4_gemm_fwd_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                     const int32_t *g_idx, int groupsize, const void *bias,
                     const void *xa, const void *lora_b, int ldb_r, int ldb_n, int lora_is_f32, float lora_scale,
                     int R, void *y, int M, int K, int N, int G,
@@ -201,7 +214,7 @@ int q4_gemm_fwd_f16(const void *x, const int32_t *qweight, const int32_t *qzeros
  * (lora_A.weight [R, K]: lda_r = K, lda_k = 1).
  * With `drop` the adapter term of dx[m, k] is kept (and scaled) only where the dropout mask keeps x[m, k]: the
  * gradient of lora_B(lora_A(dropout(x))) with respect to x. */
-int q4_gemm_bwd_dx_f16(const void *dy, const int32_t *qweight, const int32_t *qzeros, const void *scales,
+Q4_API int q4_gemm_bwd_dx_f16(const void *dy, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                        const int32_t *g_idx, int groupsize,
                        const void *dyb, const void *lora_a, int lda_r, int lda_k, int lora_is_f32, float lora_scale,
                        int R, void *dx, int M, int K, int N, int G, const q4_dropout_t *drop,
@@ -212,7 +225,7 @@ int q4_gemm_bwd_dx_f16(const void *dy, const int32_t *qweight, const int32_t *qz
  * w_sr = K, w_sc = 1) and dyb = dy @ B (w = lora_B.weight, w_sr = 1, w_sc = R): the two products that
  * lora_A(x) and the backward of lora_B perform in the reference (models.py:66).  C % 32 == 0, 1 <= R <= 64.
  * With `drop`: out = dropout(in) @ Wm^T, i.e. lora_A(dropout(x)). */
-int q4_lora_down_f16(const void *in, const void *w, int w_sr, int w_sc, int w_is_f32, void *out,
+Q4_API int q4_lora_down_f16(const void *in, const void *w, int w_sr, int w_sc, int w_is_f32, void *out,
                      int M, int C, int R, const q4_dropout_t *drop, void *stream);
 
 /* Gradient of an adapter matrix:  out fp32 [j*o_sr + c*o_sc] = alpha * sum_m p[m, j] * in[m, c]
@@ -223,8 +236,8 @@ int q4_lora_down_f16(const void *in, const void *w, int w_sr, int w_sc, int w_is
  * aligned, contents irrelevant before and after the call: it carries fp32 partial sums of row blocks,
  * which a second kernel adds in a fixed order (bit-reproducible).  With `drop`, `in` is replaced by dropout(in)
  * (dA of lora_A(dropout(x))). */
-size_t q4_lora_grad_workspace_bytes(int M, int C, int R);
-int q4_lora_grad_f32(const void *p, const void *in, float *out, int o_sr, int o_sc, float alpha,
+Q4_API size_t q4_lora_grad_workspace_bytes(int M, int C, int R);
+Q4_API int q4_lora_grad_f32(const void *p, const void *in, float *out, int o_sr, int o_sc, float alpha,
                      int M, int C, int R, const q4_dropout_t *drop,
                      void *workspace, size_t workspace_bytes, void *stream);
 
@@ -233,7 +246,7 @@ int q4_lora_grad_f32(const void *p, const void *in, float *out, int o_sr, int o_
  * backward of models.py:66.  `workspace`: q4_lora_grad_workspace_bytes(M, C1, R) +
  * q4_lora_grad_workspace_bytes(M, C2, R) bytes, 256-byte aligned, contents irrelevant.  `drop1` applies to in1 only
  * (x in dA; xa in dB already carries the mask). */
-int q4_lora_grad_pair_f32(const void *p1, const void *in1, float *out1, int o1_sr, int o1_sc, int C1,
+Q4_API int q4_lora_grad_pair_f32(const void *p1, const void *in1, float *out1, int o1_sr, int o1_sc, int C1,
                           const void *p2, const void *in2, float *out2, int o2_sr, int o2_sc, int C2,
                           float alpha, int M, int R, const q4_dropout_t *drop1,
                           void *workspace, size_t workspace_bytes, void *stream);

@@ -31,6 +31,16 @@ def test_library_exports_every_declared_symbol():
     assert L.q4_abi_version() == _lib.ABI_VERSION
 
 
+def test_library_exports_nothing_but_the_declared_symbols():
+    """The dynamic symbol table of the library holds exactly the functions of the header: internal launchers,
+    planners and kernel stubs have hidden visibility."""
+    import subprocess
+    from alpaca_lora_4bit_amd import _lib
+    out = subprocess.run(["nm", "-D", "--defined-only", _lib.LIB_PATH], check=True, capture_output=True, text=True).stdout
+    exported = sorted(line.split()[-1] for line in out.splitlines() if len(line.split()) >= 3)
+    assert exported == _declared_functions(), sorted(set(exported) ^ set(_declared_functions()))
+
+
 def test_error_codes_and_validation_need_no_gpu():
     """Every entry point validates before launching: bad arguments return a code, never crash."""
     from alpaca_lora_4bit_amd import _lib
@@ -131,7 +141,11 @@ def test_streaming_kernel_selection_rules_need_no_gpu():
     output width; very long reductions only with the smallest row block."""
     from alpaca_lora_4bit_amd import _lib
     L = _lib.lib()
-    fwd, dx = L.q4_stream_fwd_applicable, L.q4_stream_dx_applicable
+    def fwd(*a):
+        return L.q4_gemm_route(1, *a) == 2            # Q4_ROUTE_STREAM
+
+    def dx(*a):
+        return L.q4_gemm_route(0, *a) == 2
     # (M, K, N, groupsize, has_gidx)
     assert fwd(128, 4096, 4096, 128, 0) and fwd(256, 4096, 4096, 128, 0) and fwd(65, 4096, 4096, 128, 0)
     assert not fwd(64, 4096, 4096, 128, 0)            # up to 64 rows and fewer than 128 strips: the other streaming kernel

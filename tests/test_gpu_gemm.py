@@ -265,8 +265,8 @@ def test_gemm_forward_65_to_512_rows_whole_reduction_streaming_kernel(oracle, M,
     lib = _lib.lib()
     strips = N // 64
     rb = next((rb for rb in (2, 3, 4) if strips * -(-M // (16 * rb)) <= 256), 0)
-    assert bool(lib.q4_stream_fwd_applicable(M, K, N, gs, 0)) == (rb == 2 or (rb > 2 and K <= 12288))
-    assert not lib.q4_stream_fwd_applicable(M, K, N, gs, 1) and not lib.q4_stream_fwd_applicable(64, K, N, gs, 0)
+    assert bool((lib.q4_gemm_route(1, M, K, N, gs, 0) == 2)) == (rb == 2 or (rb > 2 and K <= 12288))
+    assert not (lib.q4_gemm_route(1, M, K, N, gs, 1) == 2) and not (lib.q4_gemm_route(1, 64, K, N, gs, 0) == 2)
 
 
 @pytest.mark.parametrize("M", [17, 32, 33, 48, 49, 64])
@@ -284,7 +284,7 @@ def test_gemm_forward_17_to_64_rows_of_wide_outputs_whole_reduction_streaming_ke
     y2 = quant_hip.gemm_fwd(torch.from_numpy(x).cuda(), t["qweight"], t["qzeros"], t["scales"], None, 128)
     assert y.shape == (M, N) and torch.equal(y, y2)
     assert np.abs(y.float().cpu().numpy() - ref).max() <= 2e-3 * np.abs(ref).max()
-    assert _lib.lib().q4_stream_fwd_applicable(M, K, N, 128, 0)
+    assert _lib.lib().q4_gemm_route(1, M, K, N, 128, 0) == 2
 
 
 @pytest.mark.parametrize("M", [49, 64, 65, 96, 100, 128, 129, 192, 200, 256, 300, 512])
@@ -307,8 +307,8 @@ def test_gemm_grad_input_49_to_512_rows_whole_reduction_streaming_kernel(oracle,
     assert np.abs(dx.float().cpu().numpy() - ref).max() <= 2e-3 * np.abs(ref).max()
     lib = _lib.lib()
     rb = next((rb for rb in (2, 3) if (K // 128) * -(-M // (16 * rb)) <= 256), 0)
-    assert bool(lib.q4_stream_dx_applicable(M, K, N, gs, 0)) == (rb != 0 and N <= 2 * K)
-    assert not lib.q4_stream_dx_applicable(M, K, N, gs, 1) and not lib.q4_stream_dx_applicable(48, K, N, gs, 0)
+    assert bool((lib.q4_gemm_route(0, M, K, N, gs, 0) == 2)) == (rb != 0 and N <= 2 * K)
+    assert not (lib.q4_gemm_route(0, M, K, N, gs, 1) == 2) and not (lib.q4_gemm_route(0, 48, K, N, gs, 0) == 2)
 
 
 @pytest.mark.parametrize("act", [False, True])
