@@ -6,7 +6,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libq4gptq.so")
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 _lib = None
 
@@ -49,6 +49,15 @@ class GemvLayer(ctypes.Structure):
     _fields_ = [("x", _vp), ("qweight", _vp), ("qzeros", _vp), ("scales", _vp), ("y", _vp), ("N", _i)]
 
 
+class Layer(ctypes.Structure):
+    """q4_layer_t of include/q4_gptq.h."""
+    _fields_ = [("qweight", _vp), ("qzeros", _vp), ("scales", _vp)]
+
+
+SIGNATURES["q4_mlp_decode_workspace_bytes"] = (_sz, [_i, _i, _i])
+SIGNATURES["q4_mlp_decode_status_offset"] = (_sz, [_i, _i, _i])
+SIGNATURES["q4_mlp_decode_f16"] = (_i, [_vp, ctypes.POINTER(Layer), ctypes.POINTER(Layer), ctypes.POINTER(Layer), _i, _vp, _vp, _vp,
+                                        _i, _i, _i, _vp, _sz, _vp])
 MAX_GEMV_GROUP = 4
 SIGNATURES["q4_gemv_grouped_workspace_bytes"] = (_sz, [_i, _i])
 SIGNATURES["q4_gemv_grouped_f16"] = (_i, [ctypes.POINTER(GemvLayer), _i, _i, _i, _i, _i, _vp, _sz, _vp])

@@ -185,8 +185,13 @@ class Autograd4bitQuantLinear(nn.Module):
             rows = x.numel() // self.in_features if self.in_features else 0
             if 1 <= rows <= min(int(mm4b.auto_switch_thd), quant_hip.MAX_GEMV_ROWS) and x.shape[-1] == self.in_features:
                 scales = self.scales
-                out = quant_hip.gemv(x, self.qweight, self.qzeros, scales if scales.dtype == torch.float16 else scales.half(),
-                                     self.g_idx, self.groupsize, out_shape=x.shape[:-1] + (self.out_features,))
+                # a member of a group made by model_attn_mlp_patch (q|k|v, gate|up): the first member called runs ONE
+                # launch over every member's own tensors and the others pick their result up
+                group = self.__dict__.get('_q4_group')
+                out = group.run(self, x) if group is not None else None
+                if out is None:
+                    out = quant_hip.gemv(x, self.qweight, self.qzeros, scales if scales.dtype == torch.float16 else scales.half(),
+                                         self.g_idx, self.groupsize, out_shape=x.shape[:-1] + (self.out_features,))
                 if not self.disable_bias and not _is_all_zero(self.bias):
                     out += self.bias
                 return out

@@ -12,6 +12,7 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <tuple>
 #include <utility>
 #include <vector>
 
@@ -93,6 +94,18 @@ struct Buffers {
 };
 std::mutex g_mutex;
 std::map<std::pair<int, void*>, Buffers> g_buffers;
+// A buffer that had to grow is kept, not freed: a HIP graph captured earlier still launches with the old pointer,
+// and memory handed back to the caching allocator could by then belong to another tensor.
+std::vector<at::Tensor> g_retired;
+// Workspaces of the fused MLP step: one per (device, stream, M, H, I), because the hand-over words and the launch
+// ticket they hold are only valid for calls of one shape.
+struct MlpKey {
+    int dev; void* stream; int M, H, I;
+    bool operator<(const MlpKey& o) const {
+        return std::tie(dev, stream, M, H, I) < std::tie(o.dev, o.stream, o.M, o.H, o.I);
+    }
+};
+std::map<MlpKey, at::Tensor> g_mlp_buffers;
 const bool g_check_workspace = [] { const char* e = getenv("Q4_CHECK_WORKSPACE"); return e && e[0] == '1'; }();
 
 void* zeroed_workspace(const c10::Device& dev, void* stream, size_t nbytes, size_t* have) {
@@ -100,6 +113,7 @@ void* zeroed_workspace(const c10::Device& dev, void* stream, size_t nbytes, size
     Buffers& b = g_buffers[{dev.index(), stream}];
     if (!b.zeroed.defined() || (size_t)b.zeroed.numel() < nbytes) {
         const int64_t n = (int64_t)std::max(nbytes, (size_t)1 << 22);
+        if (b.zeroed.defined()) g_retired.push_back(b.zeroed);
         b.zeroed = at::zeros({n}, at::TensorOptions().dtype(at::kByte).device(dev));
     } else if (g_check_workspace) {
         // debugging aid: the invariant "every call leaves the accumulators zero" checked on entry (synchronises)
@@ -128,6 +142,7 @@ void* scratch_workspace(const c10::Device& dev, void* stream, size_t nbytes, siz
     Buffers& b = g_buffers[{dev.index(), stream}];
     if (!b.scratch.defined() || (size_t)b.scratch.numel() < nbytes) {
         const int64_t n = (int64_t)std::max(nbytes, (size_t)1 << 22);
+        if (b.scratch.defined()) g_retired.push_back(b.scratch);
         b.scratch = at::empty({n}, at::TensorOptions().dtype(at::kByte).device(dev));
     }
     *have = (size_t)b.scratch.numel();
@@ -237,6 +252,61 @@ std::vector<at::Tensor> gemv_grouped(const std::vector<at::Tensor>& xs,
         raise_q4(rc, "q4_gemv_grouped_f16");
     }
     return result;
+}
+
+// y = down(silu(gate(x)) * up(x)) for 1..16 rows in one launch; each layer = (qweight, qzeros, scales), sequential groups.
+// Returns y, or (y, gate_out, up_out) when `intermediates` is set.
+std::vector<at::Tensor> mlp_decode(const at::Tensor& x, const std::tuple<at::Tensor, at::Tensor, at::Tensor>& gate,
+                                   const std::tuple<at::Tensor, at::Tensor, at::Tensor>& up,
+                                   const std::tuple<at::Tensor, at::Tensor, at::Tensor>& down, int64_t groupsize,
+                                   bool intermediates, const c10::optional<std::vector<int64_t>>& out_shape) {
+    const Layer lg = check_layer(std::get<0>(gate), std::get<1>(gate), std::get<2>(gate), c10::nullopt, groupsize);
+    const Layer lu = check_layer(std::get<0>(up), std::get<1>(up), std::get<2>(up), c10::nullopt, groupsize);
+    const Layer ld = check_layer(std::get<0>(down), std::get<1>(down), std::get<2>(down), c10::nullopt, groupsize);
+    const int H = lg.K, I = lg.N;
+    TORCH_CHECK_VALUE(lu.K == H && lu.N == I && ld.K == I && ld.N == H, "gate / up must be H -> I and down I -> H");
+    TORCH_CHECK_VALUE(lu.device == lg.device && ld.device == lg.device, "the three layers must be on one device");
+    const at::Tensor x2 = flat_half(x, H, lg.device, "x");
+    const int64_t M = x2.size(0);
+    TORCH_CHECK_VALUE(M >= 1 && M <= 16, "mlp_decode handles 1..16 rows, got ", M);
+    at::Tensor y = at::empty(out_sizes(out_shape, M, H), x2.options());
+    at::Tensor go, uo;
+    if (intermediates) {
+        go = at::empty({M, (int64_t)I}, x2.options());
+        uo = at::empty({M, (int64_t)I}, x2.options());
+    }
+    Launch L(lg.device);
+    const size_t need = q4_mlp_decode_workspace_bytes((int)M, H, I);
+    at::Tensor ws;
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        at::Tensor& slot = g_mlp_buffers[MlpKey{lg.device.index(), L.stream, (int)M, H, I}];
+        if (!slot.defined()) slot = at::zeros({(int64_t)need}, at::TensorOptions().dtype(at::kByte).device(lg.device));
+        ws = slot;
+    }
+    const q4_layer_t dg{lg.qweight, lg.qzeros, lg.scales}, du{lu.qweight, lu.qzeros, lu.scales}, dd{ld.qweight, ld.qzeros, ld.scales};
+    const int rc = q4_mlp_decode_f16(x2.data_ptr(), &dg, &du, &dd, (int)groupsize, intermediates ? go.data_ptr() : nullptr,
+                                     intermediates ? uo.data_ptr() : nullptr, y.data_ptr(), (int)M, H, I, ws.data_ptr(),
+                                     (size_t)ws.numel(), L.stream);
+    if (rc != Q4_OK) {
+        if (rc == Q4_ERR_LAUNCH) ws.zero_();
+        raise_q4(rc, "q4_mlp_decode_f16");
+    }
+    if (intermediates) return {y, go, uo};
+    return {y};
+}
+
+// 1 when a wait inside some fused MLP launch on this device hit its poll limit (synchronises; for tests).
+bool mlp_decode_gave_up() {
+    std::vector<std::pair<at::Tensor, size_t>> all;
+    {
+        std::lock_guard<std::mutex> lock(g_mutex);
+        for (auto& kv : g_mlp_buffers)
+            all.emplace_back(kv.second, q4_mlp_decode_status_offset(kv.first.M, kv.first.H, kv.first.I));
+    }
+    for (auto& p : all)
+        if (p.first.narrow(0, (int64_t)p.second, 4).any().item<bool>()) return true;
+    return false;
 }
 
 struct LoraPair {
@@ -383,6 +453,7 @@ void reset_workspaces() {
     std::lock_guard<std::mutex> lock(g_mutex);
     for (auto& kv : g_buffers)
         if (kv.second.zeroed.defined()) kv.second.zeroed.zero_();
+    for (auto& kv : g_mlp_buffers) kv.second.zero_();          // all zero = the state before a workspace's first use
 }
 
 // True when the cached GEMV accumulators of every stream are all zero (synchronises; for tests and debugging).
@@ -396,6 +467,8 @@ bool workspaces_are_zero() {
 void drop_workspaces() {
     std::lock_guard<std::mutex> lock(g_mutex);
     g_buffers.clear();
+    g_mlp_buffers.clear();
+    g_retired.clear();
 }
 
 }  // namespace
@@ -403,6 +476,12 @@ void drop_workspaces() {
 PYBIND11_MODULE(_q4_host, m) {
     m.doc() = "compiled host binding of libq4gptq (checks, current stream, workspaces, launch)";
     m.def("set_error_class", [](py::object cls) { g_error_class = std::move(cls); });
+    // File-scope objects would be destroyed when the library is unloaded, after the interpreter and the HIP runtime
+    // have shut down: release what they hold while both are still alive.
+    py::module_::import("atexit").attr("register")(py::cpp_function([] {
+        g_error_class = py::object();
+        drop_workspaces();
+    }));
     m.def("abi_version", [] { return q4_abi_version(); });
     m.def("dequant", &dequant, py::arg("qweight"), py::arg("qzeros"), py::arg("scales"), py::arg("g_idx"), py::arg("groupsize"),
           py::arg("out") = py::none());
@@ -419,6 +498,9 @@ PYBIND11_MODULE(_q4_host, m) {
     m.def("lora_down", &lora_down, py::arg("inp"), py::arg("w"), py::arg("dropout") = py::none());
     m.def("lora_grad_pair", &lora_grad_pair, py::arg("p1"), py::arg("inp1"), py::arg("p2"), py::arg("inp2"), py::arg("alpha"),
           py::arg("dropout") = py::none());
+    m.def("mlp_decode", &mlp_decode, py::arg("x"), py::arg("gate"), py::arg("up"), py::arg("down"), py::arg("groupsize"),
+          py::arg("intermediates") = false, py::arg("out_shape") = py::none());
+    m.def("mlp_decode_gave_up", &mlp_decode_gave_up);
     m.def("reset_workspaces", &reset_workspaces);
     m.def("workspaces_are_zero", &workspaces_are_zero);
     m.def("drop_workspaces", &drop_workspaces);

@@ -2,6 +2,7 @@
 // No torch types, no allocation, no synchronisation.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 #include "q4_gptq.h"
 
 extern "C" {
@@ -29,6 +30,11 @@ int q4_launch_gemv_group(int, const void* const*, const int32_t* const*, const i
 size_t q4_noalloc_scratch_bytes(void);
 void* q4_noalloc_scratch_ptr(int*);
 int q4_launch_zero_words(void*, size_t, hipStream_t);
+int q4_mlp_applicable(int, int, int, int);
+size_t q4_mlp_plan_workspace(int, int, int);
+size_t q4_mlp_status_offset(int, int, int);
+int q4_launch_mlp(const void*, const int32_t* const*, const int32_t* const*, const void* const*, int, void*, void*, void*, int, int,
+                  int, void*, int, hipStream_t);
 int q4_stream_fwd_applicable(int, int, int, int, int);
 int q4_stream_dx_applicable(int, int, int, int, int);
 int q4_skinny_applicable(int, int, int, int, int);
@@ -65,7 +71,7 @@ int check_layer(const void* qweight, const void* qzeros, const void* scales, con
 }
 }  // namespace
 
-extern "C" int q4_abi_version(void) { return 11; }
+extern "C" int q4_abi_version(void) { return 12; }
 
 extern "C" const char* q4_error_string(int code) {
     switch (code) {
@@ -186,6 +192,40 @@ extern "C" int q4_gemv_grouped_f16(const q4_gemv_layer_t* layers, int n_layers, 
     if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
     return q4_launch_gemv_group(n_layers, x, qw, qz, sc, y, N, groupsize, accumulate, M, K, G, workspace,
                                 (hipStream_t)stream);
+}
+
+extern "C" size_t q4_mlp_decode_workspace_bytes(int M, int H, int I) {
+    if (M < 1 || M > 16 || H < 128 || I < 128) return 0;
+    return q4_mlp_plan_workspace(M, H, I);
+}
+
+extern "C" size_t q4_mlp_decode_status_offset(int M, int H, int I) {
+    if (M < 1 || M > 16 || H < 128 || I < 128) return 0;
+    return q4_mlp_status_offset(M, H, I);
+}
+
+extern "C" int q4_mlp_decode_f16(const void* x, const q4_layer_t* gate, const q4_layer_t* up, const q4_layer_t* down,
+                                 int groupsize, void* gate_out, void* up_out, void* y, int M, int H, int I,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
+    if (!x || !y || !gate || !up || !down) return Q4_ERR_NULL_POINTER;
+    if (M < 1 || M > 16 || H < 128 || I < 128) return Q4_ERR_BAD_SHAPE;
+    const q4_layer_t* ls[3] = {gate, up, down};
+    const int32_t* qw[3]; const int32_t* qz[3]; const void* sc[3];
+    for (int i = 0; i < 3; ++i) {
+        const int K = i < 2 ? H : I, N = i < 2 ? I : H;
+        const int rc = check_layer(ls[i]->qweight, ls[i]->qzeros, ls[i]->scales, nullptr, groupsize, K, N,
+                                   groupsize > 0 ? (K + groupsize - 1) / groupsize : 0);
+        if (rc != Q4_OK) return rc;
+        if ((unsigned long long)(K / 8) * (unsigned long long)N * 4ull >= (1ull << 32)) return Q4_ERR_BAD_SHAPE;
+        qw[i] = ls[i]->qweight; qz[i] = ls[i]->qzeros; sc[i] = ls[i]->scales;
+    }
+    if (!q4_mlp_applicable(M, H, I, groupsize)) return Q4_ERR_BAD_SHAPE;
+    if (misaligned(x) || misaligned(y) || (gate_out && misaligned(gate_out)) || (up_out && misaligned(up_out)))
+        return Q4_ERR_MISALIGNED;
+    if (!workspace || workspace_bytes < q4_mlp_plan_workspace(M, H, I)) return Q4_ERR_WORKSPACE;
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
+    static const int env_polls = getenv("Q4_MLP_POLL_LIMIT") ? atoi(getenv("Q4_MLP_POLL_LIMIT")) : 0;
+    return q4_launch_mlp(x, qw, qz, sc, groupsize, gate_out, up_out, y, M, H, I, workspace, env_polls, (hipStream_t)stream);
 }
 
 extern "C" size_t q4_gemv_noalloc_max_outputs(void) { return q4_noalloc_scratch_bytes() / 8; }

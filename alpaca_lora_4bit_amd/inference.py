@@ -8,8 +8,9 @@ Steps as in the reference: load the packed model, `model.half()` and halve `scal
 temperature 0.9, top-p 0.95, top-k 40, repetition penalty 1.1, 20 new tokens), print the text and the seconds taken.
 `--lora` applies an adapter directory written by `alpaca_lora_4bit_amd.finetune` (or by peft) first.
 
-Two additions for decode speed, both off by default: `--fuse` concatenates q/k/v and gate/up into one launch each
-(model_attn_mlp_patch.make_quant_attn / make_fused_mlp, as the reference's model server does, server/server.py:100-113),
+Two additions for decode speed, both off by default: `--fuse` gives q/k/v one grouped launch on their own tensors and
+runs the MLP decode step (gate, up, silu * up, down) as one launch, adapters included
+(model_attn_mlp_patch.make_quant_attn / make_fused_mlp, which the reference's model server calls, server/server.py:100-113),
 and `--hip_graph` captures the one-token step once as a HIP graph and replays it per token, which removes the host
 time of the ~1000 small launches a decoder step consists of; the choice of the next token (argmax with `--greedy`,
 otherwise the reference's sampling settings) runs eagerly between two replays.

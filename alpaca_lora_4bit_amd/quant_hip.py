@@ -560,6 +560,32 @@ def gemv_grouped(xs, layers, groupsize, outs=None, accumulate=False):
     return list(outs)
 
 
+def mlp_decode_applicable(M, H, I, groupsize):
+    """Shapes `mlp_decode` takes (chunks of 128 reduction rows inside one quantization group on both sides)."""
+    return (1 <= M <= MAX_GEMV_ROWS and groupsize and groupsize % 128 == 0 and H % 128 == 0 and I % 128 == 0
+            and H >= 128 and I >= 128)
+
+
+def mlp_decode(x, gate, up, down, groupsize, intermediates=False, out_shape=None):
+    """y fp16 [M, H] = down(silu(gate(x)) * up(x)) for M <= 16 rows in ONE launch: the decode step of the reference's
+    QuantLlamaMLP.forward (model_attn_mlp_patch.py:224-228).  `gate`, `up` (H -> I) and `down` (I -> H) are
+    (qweight, qzeros, scales) or (qweight, qzeros, scales, g_idx) of layers with sequential groups and no bias.
+    With `intermediates` returns (y, gate(x), up(x))."""
+    _require(_host is not None, "mlp_decode needs the compiled host binding (_q4_host)")
+    lays = []
+    for lay in (gate, up, down):
+        info = _layer_info(lay[0], lay[1], lay[2], lay[3] if len(lay) > 3 else None, groupsize)
+        _require(info.plan is None and info.gemv_gidx is None, "mlp_decode needs sequential groups (no act-order)")
+        lays.append((lay[0], lay[1], lay[2]))
+    res = _host.mlp_decode(x, lays[0], lays[1], lays[2], int(groupsize), bool(intermediates), _shape_arg(out_shape))
+    return tuple(res) if intermediates else res[0]
+
+
+def mlp_decode_gave_up():
+    """True when a device-side wait of some `mlp_decode` launch ran into its poll limit (synchronises)."""
+    return bool(_host is not None and _host.mlp_decode_gave_up())
+
+
 def _adapter_dtype_flag(w, what):
     _require(w.dtype in (torch.float16, torch.float32), f"{what} must be float16 or float32")
     return int(w.dtype == torch.float32)

@@ -118,6 +118,33 @@ Q4_API size_t q4_gemv_grouped_workspace_bytes(int M, int total_N);
 Q4_API int q4_gemv_grouped_f16(const q4_gemv_layer_t *layers, int n_layers, int groupsize, int accumulate,
                         int M, int K, void *workspace, size_t workspace_bytes, void *stream);
 
+/* Decode step of a gated MLP block in ONE launch:
+ *   y fp16 [M, H] = down( silu(gate(x)) * up(x) ),   x fp16 [M, H], 1 <= M <= 16,
+ * gate and up: 4-bit layers H -> I, down: I -> H, sequential groups (g_idx NULL), no bias.  Replaces the three
+ * products and two elementwise kernels of QuantLlamaMLP.forward (model_attn_mlp_patch.py:224-228: gate_up_proj,
+ * act_fn(gate) * up, down_proj) for the rows a decode step has; the intermediate is rounded to fp16 where those
+ * modules round it (gate, up, silu(gate), the product).  The workgroups of the down projection run in the same grid
+ * as those of gate and up, request their packed weights at once and then wait, on the device, for the part of the
+ * intermediate they need: the weight stream never pauses between the products and one launch gap disappears.
+ * gate_out / up_out (fp16 [M, I]) receive the two projections when not NULL.
+ * Shapes: groupsize % 128 == 0, H % 128 == 0, I % 128 == 0 (otherwise Q4_ERR_BAD_SHAPE: use three q4_gemv_f16 calls).
+ * `workspace`: q4_mlp_decode_workspace_bytes(M, H, I) bytes, 256-byte aligned, all zero before its first use; every
+ * call leaves it ready for the next call OF THE SAME (M, H, I) on the same stream (it holds accumulators that end at
+ * zero, the hand-over words and a ticket that numbers the launches); clear it before using it for another shape.
+ * Calls that share a workspace must not overlap.  The waits inside the kernel are bounded: a wavefront that gives up
+ * sets the 32-bit word at workspace + q4_mlp_decode_status_offset(M, H, I) to 1 (the output is then invalid); it is
+ * never set when workgroups start in index order, which is how the hardware dispatches them. */
+typedef struct {
+    const int32_t *qweight;   /* [K/8, N] */
+    const int32_t *qzeros;    /* [G, N/8] */
+    const void *scales;       /* fp16 [G, N] */
+} q4_layer_t;
+Q4_API size_t q4_mlp_decode_workspace_bytes(int M, int H, int I);
+Q4_API size_t q4_mlp_decode_status_offset(int M, int H, int I);
+Q4_API int q4_mlp_decode_f16(const void *x, const q4_layer_t *gate, const q4_layer_t *up, const q4_layer_t *down,
+                             int groupsize, void *gate_out, void *up_out, void *y, int M, int H, int I,
+                             void *workspace, size_t workspace_bytes, void *stream);
+
 /* q4_gemv_f16 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same product, same arguments
  * minus the workspace: the split-K accumulators live in a device array inside the library (4 MiB per device that

@@ -110,9 +110,9 @@ def test_hip_graph_decode_gives_the_eager_tokens(tmp_path, oracle, act_order):
     new = 24
     for fused in (False, True):
         if fused:
-            # act-order projections carry their own row permutations and cannot share one launch
-            want_fused = 0 if act_order else 2
-            assert make_quant_attn(model) == want_fused and make_fused_mlp(model) == want_fused
+            # grouped in place; act-order projections carry their own row permutations, so their groups find at the
+            # first call that they cannot share one launch and every member keeps its own
+            assert make_quant_attn(model) == 2 and make_fused_mlp(model) == 2
         with torch.no_grad():
             want = model.generate(input_ids=ids, max_new_tokens=new, min_new_tokens=new, do_sample=False)
         # eos id -1 never matches: it makes the loop read every token on the host between two replays
