@@ -238,6 +238,13 @@ extern "C" int q4_gemv_noalloc_f16(const void* x, const int32_t* qweight, const 
     if (rc != Q4_OK) return rc;
     const size_t words = (size_t)M * (size_t)N;
     if (words > q4_gemv_noalloc_max_outputs()) return Q4_ERR_TOO_LARGE;
+    // the array belongs to the CURRENT device: the output must live there too
+    hipPointerAttribute_t attr;
+    int dev = -1;
+    if (hipPointerGetAttributes(&attr, y) != hipSuccess || hipGetDevice(&dev) != hipSuccess || attr.device != dev) {
+        (void)hipGetLastError();
+        return Q4_ERR_RUNTIME;
+    }
     int herr = 0;
     void* scratch = q4_noalloc_scratch_ptr(&herr);
     if (!scratch) return Q4_ERR_RUNTIME;

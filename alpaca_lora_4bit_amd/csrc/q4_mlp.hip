@@ -131,11 +131,23 @@ __device__ __forceinline__ void mlp_down_body(const MlpArgs& a, int wg, int wg2,
     // the packed weights first: they do not depend on gate and up, so they stream while those are being finished
     SeqChunk<NSTEP, GSTEPS> ch;
     ch.load_weights_branch_free(d, k0, n0 + 4 * c, kk, live);
-    // row 0's hand-over words right behind the weights: when they were published long ago (the usual case) the look
-    // costs no round trip of its own
-    const int kw = live ? k0 : 0;
-    uint32_t g0 = load_word_agent(a.hand_gate + kw + 2 * lane), g1 = load_word_agent(a.hand_gate + kw + 2 * lane + 1);
-    uint32_t u0 = load_word_agent(a.hand_up + kw + 2 * lane), u1 = load_word_agent(a.hand_up + kw + 2 * lane + 1);
+    // the hand-over words of the first four rows right behind the weights: when they were published long ago (the
+    // usual case) the look costs no round trip of its own.  Lane l takes columns k0 + 2l, k0 + 2l + 1 of a row: 512
+    // contiguous bytes per wavefront, row and matrix.
+    constexpr int RB = 4;                                 // rows per batch of loads (one latency per batch, not per row)
+    const int kw = (live ? k0 : 0) + 2 * lane;
+    uint32_t hw[RB][4] = {};
+    auto load_batch = [&](int m0) {
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+            if (m0 + r < M) {                                                     // uniform
+                const size_t at = (size_t)(m0 + r) * d.K + kw;
+                hw[r][0] = load_word_agent(a.hand_gate + at); hw[r][1] = load_word_agent(a.hand_gate + at + 1);
+                hw[r][2] = load_word_agent(a.hand_up + at); hw[r][3] = load_word_agent(a.hand_up + at + 1);
+            }
+        }
+    };
+    load_batch(0);
     if (threadIdx.x == 0)
         *tag_lds = tag_of(__hip_atomic_load(ticket_of(a.ticket, wg), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
     __builtin_amdgcn_sched_barrier(0);
@@ -146,18 +158,16 @@ __device__ __forceinline__ void mlp_down_body(const MlpArgs& a, int wg, int wg2,
     uint32_t* tile = reinterpret_cast<uint32_t*>(red + ((wave * M) << 6));
     if (live) {
         int polls = 0;
-        for (int m = 0; m < M; ++m) {
-            // lane l takes columns k0 + 2l, k0 + 2l + 1 of row m: 512 contiguous bytes per wavefront and matrix
-            const uint32_t* pg = a.hand_gate + (size_t)m * d.K + k0 + 2 * lane;
-            const uint32_t* pu = a.hand_up + (size_t)m * d.K + k0 + 2 * lane;
-            bool have = m == 0;
+        for (int m0 = 0; m0 < M; m0 += RB) {
+            bool have = m0 == 0;
             for (;;) {
-                if (!have) {
-                    g0 = load_word_agent(pg); g1 = load_word_agent(pg + 1);
-                    u0 = load_word_agent(pu); u1 = load_word_agent(pu + 1);
-                }
+                if (!have) load_batch(m0);
                 have = false;
-                const bool stale = ((g0 >> 16) != tag) | ((g1 >> 16) != tag) | ((u0 >> 16) != tag) | ((u1 >> 16) != tag);
+                bool stale = false;
+#pragma unroll
+                for (int r = 0; r < RB; ++r)
+                    if (m0 + r < M)
+                        stale |= ((hw[r][0] >> 16) != tag) | ((hw[r][1] >> 16) != tag) | ((hw[r][2] >> 16) != tag) | ((hw[r][3] >> 16) != tag);
                 if (__builtin_amdgcn_ballot_w64(stale) == 0) break;              // wave-uniform
                 if (++polls > a.poll_limit) {
                     if (lane == 0) __hip_atomic_store(a.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -165,7 +175,10 @@ __device__ __forceinline__ void mlp_down_body(const MlpArgs& a, int wg, int wg2,
                 }
                 __builtin_amdgcn_s_sleep(16);
             }
-            tile[m * (CH / 2) + lane] = silu_mul_bits(g0, u0) | (silu_mul_bits(g1, u1) << 16);
+#pragma unroll
+            for (int r = 0; r < RB; ++r)
+                if (m0 + r < M)
+                    tile[(m0 + r) * (CH / 2) + lane] = silu_mul_bits(hw[r][0], hw[r][2]) | (silu_mul_bits(hw[r][1], hw[r][3]) << 16);
         }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

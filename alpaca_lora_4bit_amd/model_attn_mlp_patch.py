@@ -207,6 +207,11 @@ def make_quant_attn(model, is_v1_model=False, concatenate=False):
     return count
 
 
+# The one-launch MLP step re-reads the intermediate once per output strip of the down projection, which grows with the
+# number of rows: measured against grouped gate|up + two elementwise launches + down it wins up to about 4 rows.
+mlp_decode_max_rows = 4
+
+
 def _is_silu(act):
     return isinstance(act, nn.SiLU) or type(act).__name__.lower() in ("silu", "siluactivation") or act is torch.nn.functional.silu
 
@@ -228,7 +233,7 @@ def _mlp_decode_forward(mlp, x):
     if (not torch.is_grad_enabled() and x.dtype == torch.float16 and x.is_cuda and autograd_4bit.backend == 'cuda'
             and matmul_utils_4bit.use_new and matmul_utils_4bit.auto_switch and x.shape[-1] == gate.in_features):
         rows = x.numel() // gate.in_features
-        if (1 <= rows <= min(int(matmul_utils_4bit.auto_switch_thd), quant_hip.MAX_GEMV_ROWS)
+        if (1 <= rows <= min(int(matmul_utils_4bit.auto_switch_thd), quant_hip.MAX_GEMV_ROWS, mlp_decode_max_rows)
                 and quant_hip.mlp_decode_applicable(rows, gate.in_features, gate.out_features, gate.groupsize)
                 and all(_plain_no_bias(l) and l.scales.dtype == torch.float16 for l in (gate, up, down))):
             group = gate.__dict__.get('_q4_group')

@@ -165,6 +165,55 @@ def bench_single_gemv(K, N, M, act_order, reps, copies, seed=3):
     return dict(us=per * 1e6, gbs=b / per / 1e9, frac_hbm=b / per / 1e9 / HBM_PEAK_GBS, bytes=b, copies=copies)
 
 
+def bench_mlp_decode_one_launch(M, steps, n_layers=32, seed=1):
+    """The headline step through quant_hip.mlp_decode: per layer ONE launch computes gate, up, silu(gate) * up and down
+    (the same packed bytes as the grouped gate|up + down launches, plus the activation)."""
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    shapes = [("gate", 4096, 11008), ("up", 4096, 11008), ("down", 11008, 4096)]
+    layers = [[make_layer_gpu(K, N, 128, gen) for _, K, N in shapes] for _ in range(n_layers)]
+    x = torch.randn((M, 4096), device="cuda", generator=gen).half()
+    tup = lambda l: (l["qweight"], l["qzeros"], l["scales"])
+
+    def step():
+        for g, u, d in layers:
+            quant_hip.mlp_decode(x, tup(g), tup(u), tup(d), 128)
+
+    g, u, d = layers[0]
+    y = quant_hip.mlp_decode(x, tup(g), tup(u), tup(d), 128)
+    gg, uu = quant_hip.gemv_grouped(x, [tup(g), tup(u)], 128)
+    ref = quant_hip.gemv(torch.nn.functional.silu(gg) * uu, *tup(d), None, 128)
+    err = float((y.float() - ref.float()).abs().max() / ref.float().abs().max())
+    assert err < 1e-2 and not quant_hip.mlp_decode_gave_up(), f"one-launch MLP sanity check failed: {err}"
+    wall, ev = time_graph(step, steps, 2)
+    assert not quant_hip.mlp_decode_gave_up()
+    b = 3 * gemv_bytes(M, 4096, 11008, 32) - 2 * M * 4096
+    per = ev / (steps * n_layers)
+    return dict(us_per_mlp=per * 1e6, step_gbs=b * n_layers / (wall / steps) / 1e9, kernel_gbs=b / per / 1e9,
+                frac_hbm=b / per / 1e9 / HBM_PEAK_GBS, bytes_per_launch=b, launches_per_step=n_layers)
+
+
+def bench_grouped_gemv(K, Ns, M, reps, copies, seed=4):
+    """Several layers that share their input in one grouped launch (q|k|v of an attention block)."""
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    sets = [[make_layer_gpu(K, N, 128, gen) for N in Ns] for _ in range(copies)]
+    x = torch.randn((M, K), device="cuda", generator=gen).half()
+    outs = [torch.empty((M, N), dtype=torch.float16, device="cuda") for N in Ns]
+    inner = max(1, 24 // copies)
+
+    def step():
+        for _ in range(inner):
+            for lays in sets:
+                quant_hip.gemv_grouped(x, [(l["qweight"], l["qzeros"], l["scales"]) for l in lays], 128, outs=outs)
+    _, ev = time_graph(step, reps, 2)
+    per = ev / (reps * copies * inner)
+    b = sum(gemv_bytes(M, K, N, K // 128) for N in Ns) - (len(Ns) - 1) * 2 * M * K
+    return dict(us=per * 1e6, gbs=b / per / 1e9, frac_hbm=b / per / 1e9 / HBM_PEAK_GBS, bytes=b, copies=copies)
+
+
 def bench_dequant(K, N, act_order, reps, copies=6, seed=9):
     """Dense dequantization (the reference's vecquant4recons_v2): bytes = packed layer read + fp16 matrix written."""
     import torch
@@ -432,7 +481,7 @@ def bench_mid_rows(reps):
     return mid
 
 
-def cpu_baseline(seconds_budget=20.0):
+def cpu_baseline(seconds_budget=12.0):
     """Torch-CPU restatement of the reference's recons+matmul on the same workload shapes
     (one MLP: gate, up, down at M=1), repeated until ~seconds_budget of CPU time is spent."""
     import torch
@@ -469,6 +518,58 @@ def cpu_baseline(seconds_budget=20.0):
                 sample=f"{n} GEMVs (gate/up/down of one MLP, M=1) through oracle/q4_torch.py "
                        f"(dense dequant + torch.matmul), {total_t:.1f} s of CPU time",
                 ms_per_gemv=total_t / n * 1e3, ms_dequant=t_deq / n * 1e3, ms_matmul=(total_t - t_deq) / n * 1e3)
+
+
+def cpu_baseline_lora_step(seconds_budget=12.0):
+    """Config 2 on the host, the reference's algorithm with plain torch: forward = dense dequantization +
+    torch.matmul (matmul_utils_4bit.py:114-127) + the adapter terms (models.py:58-66); backward = dense dequantization
+    again + dy @ W^T (autograd_4bit.py:45-54) + the adapter's share of dx and the gradients of A and B.
+    M = 2048 tokens, K = N = 4096, r = 8, scaling 2.  One warm-up, then the median of at least 5 steps."""
+    import torch
+    from oracle import q4_torch
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    gen = torch.Generator().manual_seed(12)
+    M, K, N, r, scaling = 2048, 4096, 4096, 8, 2.0
+    G = K // 128
+    qweight = torch.randint(-2 ** 31, 2 ** 31 - 1, (K // 8, N), dtype=torch.int32, generator=gen)
+    qzeros = torch.randint(-2 ** 31, 2 ** 31 - 1, (G, N // 8), dtype=torch.int32, generator=gen)
+    scales = (torch.rand((G, N), generator=gen) * 0.015 + 0.005).half()
+    g_idx = (torch.arange(K) // 128).to(torch.int32)
+    x = torch.randn((M, K), generator=gen).half().float()
+    dy = torch.randn((M, N), generator=gen).half().float()
+    A = (torch.rand((r, K), generator=gen) * 2 - 1) * (1.0 / K) ** 0.5
+    B = torch.randn((N, r), generator=gen) * 0.02
+    times, t_deq, t_mm, t_lora = [], [], [], []
+    t_start = time.perf_counter()
+    while len(times) < 6 or (time.perf_counter() - t_start < seconds_budget and len(times) < 30):
+        t0 = time.perf_counter()
+        W = q4_torch.dequant_v2(qweight, qzeros, scales, g_idx).float()
+        t1 = time.perf_counter()
+        y = x @ W
+        t2 = time.perf_counter()
+        xa = x @ A.t()
+        y += scaling * (xa @ B.t())
+        t3 = time.perf_counter()
+        W = q4_torch.dequant_v2(qweight, qzeros, scales, g_idx).float()        # the backward dequantizes again
+        t4 = time.perf_counter()
+        dx = dy @ W.t()
+        t5 = time.perf_counter()
+        dyb = dy @ B
+        dx += scaling * (dyb @ A)
+        dB = scaling * (dy.t() @ xa)
+        dA = scaling * (dyb.t() @ x)
+        t6 = time.perf_counter()
+        times.append(t6 - t0)
+        t_deq.append((t1 - t0) + (t4 - t3)); t_mm.append((t2 - t1) + (t5 - t4)); t_lora.append((t3 - t2) + (t6 - t5))
+        del W, y, dx, dB, dA
+    med = lambda v: sorted(v[1:])[len(v[1:]) // 2]
+    step = med(times)
+    return dict(tokens_per_s=M / step, ms_per_step=step * 1e3, ms_dequant=med(t_deq) * 1e3, ms_matmul=med(t_mm) * 1e3,
+                ms_adapter=med(t_lora) * 1e3, cores=cores, steps_timed=len(times) - 1,
+                sample="config 2 (M=2048, K=N=4096, r=8) forward + backward on the host: oracle/q4_torch.py dense dequant "
+                       "(twice, as the reference's forward and backward do) + torch.matmul fp32 + adapter terms and gradients")
 
 
 def main():
@@ -571,6 +672,11 @@ def main():
         extra["mlp_decode_M1_three_launches"] = {"step_gbs": round(r["gbs_wall"], 1), "gate_or_up_us": round(r["gate_up"]["us"], 3),
                                                  "gate_or_up_frac_hbm": round(r["gate_up"]["gbs"] / HBM_PEAK_GBS, 4),
                                                  "down_us": round(r["down"]["us"], 3)}
+        for M in (1, 4):
+            one = bench_mlp_decode_one_launch(M, max(args.steps // 2, 5))
+            extra[f"mlp_decode_M{M}_one_launch_per_layer"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in one.items()}
+        qkv = bench_grouped_gemv(4096, (4096, 4096, 4096), 1, 10, 13)         # how the 4096 x 4096 layers run in a model
+        extra["qkv_grouped_3x4096x4096_M1"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in qkv.items()}
         # gate and up share x: concatenated along N they are one launch of twice the size
         gu = bench_single_gemv(4096, 22016, 1, False, 10, 16)
         extra["mlp_decode_M1_gate_up_fused_N22016"] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in gu.items()}
@@ -621,6 +727,9 @@ def main():
         out["cpu_baseline"]["value"] = round(out["cpu_baseline"]["value"], 4)
         for k in ("ms_per_gemv", "ms_dequant", "ms_matmul"):
             out["cpu_baseline"][k] = round(out["cpu_baseline"][k], 2)
+        # the second half of the metric (LoRA fwd+bwd tokens/s) on the same host cores
+        lo_cpu = cpu_baseline_lora_step()
+        out["cpu_baseline"]["lora_fwd_bwd_M2048"] = {k: (round(v, 2) if isinstance(v, float) else v) for k, v in lo_cpu.items()}
     print(json.dumps(out), flush=True)
 
 

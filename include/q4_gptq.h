@@ -152,7 +152,10 @@ Q4_API int q4_mlp_decode_f16(const void *x, const q4_layer_t *gate, const q4_lay
  * = 524 288 (e.g. 16 rows x 32 768 columns) and returns Q4_ERR_TOO_LARGE beyond that.  It calls no hipMalloc /
  * hipFree and no allocating library routine; it enqueues a small fill kernel that zeroes the accumulators and
  * then the same kernels as q4_gemv_f16, and gives bit-identical results.  All calls on one device share the
- * one array: calls that overlap on a device (two streams, two threads) race -- order them on one stream. */
+ * one array: calls that overlap on a device (two streams, two threads) race -- order them on one stream.
+ * The array is that of the CURRENT device: y must live on it (Q4_ERR_RUNTIME otherwise).  The first call on a device
+ * looks the array's address up (hipGetSymbolAddress) and must therefore come before stream capture begins; every
+ * later call may be captured into a HIP graph and replayed. */
 Q4_API size_t q4_gemv_noalloc_max_outputs(void);
 Q4_API int q4_gemv_noalloc_f16(const void *x, const int32_t *qweight, const int32_t *qzeros, const void *scales,
                         const int32_t *g_idx, int groupsize, void *y, int accumulate,

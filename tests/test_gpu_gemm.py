@@ -63,6 +63,10 @@ def test_streaming_grad_input_17_to_48_rows(oracle, K, N, gs, M):
     assert dx.shape == (M, K)
     err = float((dx.double() - ref).abs().max() / ref.abs().max())
     assert err <= TOL and err <= 2e-3, err
+    # a sample of rows against the CPU oracle itself (the line above rests on the library's own dense W)
+    rows = [0, M // 2, M - 1]
+    oref = oracle.matmul_recons_t(dy.cpu().numpy()[rows], layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
+    assert rel_err(dx.cpu().numpy()[rows], oref) <= 2e-3
     again = quant_hip.gemm_bwd_dx(dy, t["qweight"], t["qzeros"], t["scales"], None, gs)
     assert torch.equal(dx, again)                                   # ordered partial sums: bit-reproducible
     big = torch.cat([dy, torch.zeros(49 - M, N, dtype=dy.dtype, device=dy.device)])     # 49 rows: the tiled kernel
@@ -161,6 +165,15 @@ def test_wide_tiles_256x256(oracle, M, K, N, gs, act, r):
     for got, ref in ((y, yref), (dx, dxref)):
         err = float((got.float() - ref).abs().max() / ref.abs().max())
         assert err <= TOL and err <= 2e-3, err
+    # a sample of rows from different row tiles against the CPU oracle itself (float64, oracle's own dense W)
+    rows = np.array([0, 255, 256, 1000, M - 257, M - 1])
+    xs, dys = x.cpu().numpy()[rows], dy.cpu().numpy()[rows]
+    oy = oracle.matmul_recons(xs, layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"]) + bias.float().cpu().numpy()
+    odx = oracle.matmul_recons_t(dys, layer["qweight"], layer["qzeros"], layer["scales"], layer["g_idx"])
+    if r:
+        oy = oy + 2.0 * (xa.float().cpu().numpy()[rows].astype(np.float64) @ B.half().float().cpu().numpy().astype(np.float64).T)
+        odx = odx + 2.0 * (dyb.float().cpu().numpy()[rows].astype(np.float64) @ A.half().float().cpu().numpy().astype(np.float64))
+    assert rel_err(y.cpu().numpy()[rows], oy) <= 2e-3 and rel_err(dx.cpu().numpy()[rows], odx) <= 2e-3
     # the forward product of every case has at least 144 wide tiles: it runs unsplit and wants no workspace
     assert (N // 256) * -(-M // 256) >= 144 and _lib.lib().q4_gemm_workspace_bytes(1, M, K, N) == 0
     if r:

@@ -3,6 +3,7 @@ torch.matmul on the library's own bit-exact dense W.  Complements the fixed-shap
 indexing mistakes at odd combinations of rows, reduction length, column count, group size and act-order."""
 import random
 
+import numpy as np
 import pytest
 import torch
 
@@ -13,7 +14,7 @@ ROWS = [1, 2, 3, 4, 5, 7, 8, 15, 16, 17, 20, 31, 32, 33, 40, 47, 48, 49, 63, 64,
 
 
 @pytest.mark.parametrize("seed", [0, 1, 2])
-def test_random_shapes_against_dense_matmul(seed):
+def test_random_shapes_against_dense_matmul(seed, oracle):
     from alpaca_lora_4bit_amd import quant_hip
     rnd = random.Random(seed)
     g = torch.Generator().manual_seed(100 + seed)
@@ -49,6 +50,14 @@ def test_random_shapes_against_dense_matmul(seed):
             assert y.shape == ref.shape, (tag, name)
             err = float((y.float() - ref).abs().max() / ref.abs().max())
             assert err <= 3e-3, (tag, name, err)
+        # two rows of every case against the CPU oracle itself (its own unpacking and dense W, float64)
+        rows = sorted({0, M - 1})
+        lay = (qw.cpu().numpy(), qz.cpu().numpy(), sc.cpu().numpy(), gi.cpu().numpy())
+        oy = oracle.matmul_recons(x.cpu().numpy()[rows], *lay) + (bias.float().cpu().numpy() if bias is not None else 0)
+        odx = oracle.matmul_recons_t(dy.cpu().numpy()[rows], *lay)
+        for name, y, ref in (("fwd", got["fwd"][0], oy), ("bwd", got["bwd"][0], odx)):
+            err = float(np.abs(y.float().cpu().numpy()[rows] - ref).max() / np.abs(ref).max())
+            assert err <= 3e-3, (tag, name, "oracle", err)
 
 
 @pytest.mark.parametrize("K,gs", [(1408, 256), (1408, 512), (11008, 1024), (640, 512)])

@@ -186,6 +186,54 @@ def test_lora_backward_by_finite_differences():
             assert abs(fd - grad[idx]) <= 1e-5 * max(1.0, abs(fd))
 
 
+def test_lora_backward_with_a_dropout_mask_by_finite_differences_and_autograd():
+    """The `keep` branch (dropout in front of lora_A, models.py:63-66): the closed-form gradients against central
+    differences of lora_forward with the same mask, and against torch autograd through nn.Linear layers fed
+    x * keep * scale; a dropped element gets no adapter gradient."""
+    import torch
+    rng = np.random.default_rng(23)
+    K, N, r, M = 12, 10, 4, 6
+    W = rng.standard_normal((K, N))
+    A, B = rng.standard_normal((r, K)), rng.standard_normal((N, r))
+    x, dy = rng.standard_normal((M, K)), rng.standard_normal((M, N))
+    keep, scale = o.dropout_keep_counter(M, K, seed=1234567, p=0.4)
+    assert keep.shape == (M, K) and 0 < keep.sum() < keep.size and abs(scale - 32768.0 / (32768 - 13107)) < 1e-12
+    dx, dA, dB = o.lora_backward(x, dy, W, A, B, 2.0, keep=keep, drop_scale=scale)
+    loss = lambda x_, A_, B_: (o.lora_forward(x_, W, A_, B_, 2.0, keep=keep, drop_scale=scale) * dy).sum()
+    eps = 1e-6
+    for arr, grad, which in ((x, dx, 0), (A, dA, 1), (B, dB, 2)):
+        for idx in [(0, 0), (1, 2), (2, 3), (arr.shape[0] - 1, arr.shape[1] - 1)]:
+            p = arr.copy(); p[idx] += eps
+            m = arr.copy(); m[idx] -= eps
+            args_p = [x, A, B]; args_p[which] = p
+            args_m = [x, A, B]; args_m[which] = m
+            fd = (loss(*args_p) - loss(*args_m)) / (2 * eps)
+            assert abs(fd - grad[idx]) <= 1e-5 * max(1.0, abs(fd))
+    base_only = dy @ W.T
+    dropped = keep == 0
+    assert np.allclose(dx[dropped], base_only[dropped])             # no adapter share where x was dropped
+    assert not np.allclose(dx[~dropped], base_only[~dropped])
+    xt = torch.from_numpy(x.copy()).requires_grad_(True)
+    At, Bt = torch.from_numpy(A.copy()).requires_grad_(True), torch.from_numpy(B.copy()).requires_grad_(True)
+    xd = xt * torch.from_numpy(keep.astype(np.float64)) * scale
+    y = xt @ torch.from_numpy(W) + (xd @ At.t()) @ Bt.t() * 2.0
+    y.backward(torch.from_numpy(dy))
+    assert np.allclose(y.detach().numpy(), o.lora_forward(x, W, A, B, 2.0, keep=keep, drop_scale=scale))
+    assert np.allclose(xt.grad.numpy(), dx) and np.allclose(At.grad.numpy(), dA) and np.allclose(Bt.grad.numpy(), dB)
+
+
+def test_dropout_keep_counter_statistics_and_determinism():
+    """The mask is a pure function of (seed, row, column): repeatable, different for another seed, keeps about 1 - p."""
+    k1, s1 = o.dropout_keep_counter(256, 512, seed=42, p=0.05)
+    k2, _ = o.dropout_keep_counter(256, 512, seed=42, p=0.05)
+    k3, _ = o.dropout_keep_counter(256, 512, seed=43, p=0.05)
+    assert np.array_equal(k1, k2) and not np.array_equal(k1, k3)
+    assert abs(k1.mean() - 0.95) < 0.005 and abs(s1 - 32768.0 / (32768 - 1638)) < 1e-12
+    k0, s0 = o.dropout_keep_counter(8, 16, seed=1, p=0.0)
+    assert k0.all() and s0 == 1.0
+    assert np.array_equal(o.dropout_keep_counter(300, 512, seed=42, p=0.05)[0][:256], k1)     # rows do not depend on M
+
+
 def test_lora_forward_matches_torch_autograd():
     """Closed-form gradients == torch autograd through dense nn.Linear layers (models.py:58-66)."""
     import torch

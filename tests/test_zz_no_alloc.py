@@ -80,3 +80,43 @@ def test_noalloc_gemv_rejects_what_does_not_fit():
     assert L.q4_gemv_noalloc_f16(fake, fake, fake, fake, None, 128, fake, 0, 17, 256, 128, 2, None) == -2
     assert L.q4_gemv_noalloc_f16(None, fake, fake, fake, None, 128, fake, 0, 1, 256, 128, 2, None) == -1
     assert b"scratch" in L.q4_error_string(-6)
+
+
+def test_noalloc_gemv_captured_in_a_hip_graph_and_replayed(oracle):
+    """What the entry point is for: after one eager call on the device (the address look-up), a call is recorded into
+    a HIP graph and replayed several times, with eager work and synchronisations of the program's own in between;
+    every replay must give the bits of the eager call."""
+    import torch
+    from alpaca_lora_4bit_amd import _lib
+    L = _lib.lib()
+    M, K, N = 4, 4096, 4096
+    layer = oracle.make_layer(K, N, 128, seed=21)
+    t = to_cuda_layer(layer)
+    xs = [torch.from_numpy(oracle.make_activations(M, K, seed=s)).cuda() for s in (1, 2, 3)]
+    x = xs[0].clone()
+    y = torch.empty((M, N), dtype=torch.float16, device="cuda")
+
+    def call(stream):
+        return L.q4_gemv_noalloc_f16(x.data_ptr(), t["qweight"].data_ptr(), t["qzeros"].data_ptr(), t["scales"].data_ptr(),
+                                     None, 128, y.data_ptr(), 0, M, K, N, K // 128, stream)
+
+    want = []
+    for xi in xs:                                       # eager results (also the first call on the device)
+        x.copy_(xi)
+        assert call(torch.cuda.current_stream().cuda_stream) == 0
+        torch.cuda.synchronize()
+        want.append(y.clone())
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        assert call(torch.cuda.current_stream().cuda_stream) == 0
+    for rep in range(6):
+        xi = xs[rep % 3]
+        x.copy_(xi)
+        y.fill_(float("nan"))
+        (xi.float() @ xi.float().t()).sum().item()      # eager work and a host read between two replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, want[rep % 3]), rep
