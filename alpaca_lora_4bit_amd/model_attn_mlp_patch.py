@@ -81,6 +81,7 @@ class _MemberGroup:
         self.index = {id(m): i for i, m in enumerate(self.members)}
         self.groupsize = self.members[0].groupsize
         self.usable = None                                   # decided at the first call (needs the tensors on the GPU)
+        self._layer_cache = None
         self.hook = None
         self.clear()
 
@@ -96,15 +97,25 @@ class _MemberGroup:
             return False
         return all(m.scales.dtype == torch.float16 for m in self.members)
 
+    def _layers(self):
+        """(qweight, qzeros, scales) of every member, rebuilt when a member's buffers were replaced (a cast, a reload)."""
+        cached = self._layer_cache
+        if cached is not None and all(m._buffers.get('qweight') is c[0] and m._buffers.get('scales') is c[2]
+                                      for m, c in zip(self.members, cached)):
+            return cached
+        self.usable = self._check()
+        self._layer_cache = [(m.qweight, m.qzeros, m.scales) for m in self.members] if self.usable else None
+        return self._layer_cache
+
     def run(self, member, x):
-        if self.usable is None:
-            self.usable = self._check()
-        if not self.usable:
+        layers = self._layers()
+        if layers is None:
             return None
         i = self.index[id(member)]
         if self._x is not x or self._version != x._version or self._outs[i] is None:
             from . import quant_hip
-            outs = quant_hip.gemv_grouped(x, [(m.qweight, m.qzeros, m.scales) for m in self.members], self.groupsize)
+            # the compiled binding checks shapes, dtypes and devices; sequential groups were established by _check()
+            outs = quant_hip.gemv_grouped_prepared(x, layers, self.groupsize)
             lead = tuple(x.shape[:-1])
             self._outs = [o.view(lead + (o.shape[-1],)) for o in outs]
             self._x, self._version = x, x._version
@@ -126,6 +137,7 @@ class _MemberGroup:
         self.index[id(new)] = i
         new.__dict__['_q4_group'] = self
         self.usable = None
+        self._layer_cache = None
         self.clear()
 
 
@@ -184,6 +196,7 @@ def ungroup(model):
         if '_q4_mlp_forward' in m.__dict__:
             del m.__dict__['_q4_mlp_forward']
             del m.__dict__['forward']
+            m.__dict__.pop('_q4_mlp_args', None)
     return count
 
 
@@ -225,26 +238,48 @@ def _plain_no_bias(layer):
     return layer.disable_bias or _is_all_zero(layer.bias)
 
 
-def _mlp_decode_forward(mlp, x):
-    """LlamaMLP.forward with the decode step (up to 16 rows, no grad, fp16) as ONE launch: gate, up, silu(gate) * up and
-    down (quant_hip.mlp_decode); everything else goes to the block's own forward."""
-    from . import autograd_4bit, quant_hip
+def _mlp_decode_args(mlp):
+    """(gate, up, down, groupsize, H) for quant_hip's one-launch MLP step, or None when the block does not qualify right
+    now: all three layers plain 4-bit products (no active adapter, no bias to add), fp16 scales, sequential groups."""
+    from . import quant_hip
     gate, up, down = mlp.gate_proj, mlp.up_proj, mlp.down_proj
+    group = gate.__dict__.get('_q4_group')
+    if group is None or group._layers() is None:
+        return None
+    if not all(_plain_no_bias(l) and l.scales.dtype == torch.float16 for l in (gate, up, down)):
+        return None
+    info = quant_hip._layer_info(down.qweight, down.qzeros, down.scales, down.g_idx, down.groupsize)
+    if info.plan is not None or info.gemv_gidx is not None:
+        return None
+    return ((gate.qweight, gate.qzeros, gate.scales), (up.qweight, up.qzeros, up.scales),
+            (down.qweight, down.qzeros, down.scales), int(gate.groupsize), gate.in_features, gate.out_features, down.out_features)
+
+
+def _mlp_decode_forward(mlp, x):
+    """LlamaMLP.forward with the decode step (a few rows, no grad, fp16) as ONE launch: gate, up, silu(gate) * up and
+    down (quant_hip.mlp_decode); everything else goes to the block's own forward.  What the step needs of the three
+    layers is looked up once and kept while their buffers, adapters and bias switches stay the same objects / values."""
+    from . import autograd_4bit, quant_hip
+    d = mlp.__dict__
     if (not torch.is_grad_enabled() and x.dtype == torch.float16 and x.is_cuda and autograd_4bit.backend == 'cuda'
-            and matmul_utils_4bit.use_new and matmul_utils_4bit.auto_switch and x.shape[-1] == gate.in_features):
-        rows = x.numel() // gate.in_features
-        if (1 <= rows <= min(int(matmul_utils_4bit.auto_switch_thd), quant_hip.MAX_GEMV_ROWS, mlp_decode_max_rows)
-                and quant_hip.mlp_decode_applicable(rows, gate.in_features, gate.out_features, gate.groupsize)
-                and all(_plain_no_bias(l) and l.scales.dtype == torch.float16 for l in (gate, up, down))):
-            group = gate.__dict__.get('_q4_group')
-            if group is not None and group.usable is None:
-                group.usable = group._check()
-            info = quant_hip._layer_info(down.qweight, down.qzeros, down.scales, down.g_idx, down.groupsize)
-            if group is not None and group.usable and info.plan is None and info.gemv_gidx is None:
-                return quant_hip.mlp_decode(x, (gate.qweight, gate.qzeros, gate.scales), (up.qweight, up.qzeros, up.scales),
-                                            (down.qweight, down.qzeros, down.scales), gate.groupsize,
-                                            out_shape=tuple(x.shape[:-1]) + (down.out_features,))
-    return mlp.__dict__['_q4_mlp_forward'](x)
+            and matmul_utils_4bit.use_new and matmul_utils_4bit.auto_switch):
+        cached = d.get('_q4_mlp_args')
+        mods = mlp._modules
+        gate, up, down = mods['gate_proj'], mods['up_proj'], mods['down_proj']
+        bias = [l._buffers.get('bias') for l in (gate, up, down)]
+        key = (gate._buffers.get('qweight'), up._buffers.get('qweight'), down._buffers.get('qweight'),
+               gate._buffers.get('scales'), bias[0], bias[1], bias[2],
+               tuple(-1 if b is None else b._version for b in bias), gate.disable_bias, up.disable_bias, down.disable_bias,
+               getattr(gate, 'disable_adapters', None), getattr(up, 'disable_adapters', None), getattr(down, 'disable_adapters', None))
+        if cached is None or not (all(a is b for a, b in zip(cached[0][:7], key[:7])) and cached[0][7:] == key[7:]):
+            cached = d['_q4_mlp_args'] = (key, _mlp_decode_args(mlp))
+        args = cached[1]
+        if args is not None and x.shape[-1] == args[4]:
+            rows = x.numel() // args[4]
+            if (1 <= rows <= min(int(matmul_utils_4bit.auto_switch_thd), quant_hip.MAX_GEMV_ROWS, mlp_decode_max_rows)
+                    and quant_hip.mlp_decode_applicable(rows, args[4], args[5], args[3])):
+                return quant_hip.mlp_decode_prepared(x, args[0], args[1], args[2], args[3], tuple(x.shape[:-1]) + (args[6],))
+    return d['_q4_mlp_forward'](x)
 
 
 def make_fused_mlp(model, is_v1_model=False, concatenate=False, fuse_decode_step=True):

@@ -581,6 +581,18 @@ def mlp_decode(x, gate, up, down, groupsize, intermediates=False, out_shape=None
     return tuple(res) if intermediates else res[0]
 
 
+def gemv_grouped_prepared(x, layers, groupsize):
+    """gemv_grouped for callers that already know the layers qualify (sequential groups, fp16 scales: the module
+    groups of model_attn_mlp_patch establish that once): straight to the compiled binding, which still checks shapes,
+    dtypes and devices.  `layers`: list of (qweight, qzeros, scales)."""
+    return _host.gemv_grouped([x] * len(layers), layers, groupsize, None, False)
+
+
+def mlp_decode_prepared(x, gate, up, down, groupsize, out_shape):
+    """mlp_decode under the same premise as gemv_grouped_prepared."""
+    return _host.mlp_decode(x, gate, up, down, groupsize, False, out_shape)[0]
+
+
 def mlp_decode_gave_up():
     """True when a device-side wait of some `mlp_decode` launch ran into its poll limit (synchronises)."""
     return bool(_host is not None and _host.mlp_decode_gave_up())

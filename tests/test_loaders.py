@@ -154,7 +154,7 @@ def test_projections_grouped_in_place_keep_the_logits_with_and_without_adapters(
     assert make_quant_attn(model) == 0 and make_fused_mlp(model) == 0          # idempotent
     assert sorted(model.state_dict()) == keys                                 # same modules, same tensors, same keys
     calls = {"grouped": 0, "mlp": 0, "gemv": 0}
-    for name, key in (("gemv_grouped", "grouped"), ("mlp_decode", "mlp"), ("gemv", "gemv")):
+    for name, key in (("gemv_grouped_prepared", "grouped"), ("mlp_decode_prepared", "mlp"), ("gemv", "gemv")):
         real = getattr(quant_hip, name)
         monkeypatch.setattr(quant_hip, name, (lambda real, key: lambda *a, **k: (calls.__setitem__(key, calls[key] + 1), real(*a, **k))[1])(real, key))
     with torch.no_grad():
