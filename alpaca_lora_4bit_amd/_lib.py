@@ -6,7 +6,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libq4gptq.so")
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 _lib = None
 
@@ -58,6 +58,17 @@ SIGNATURES["q4_mlp_decode_workspace_bytes"] = (_sz, [_i, _i, _i])
 SIGNATURES["q4_mlp_decode_status_offset"] = (_sz, [_i, _i, _i])
 SIGNATURES["q4_mlp_decode_f16"] = (_i, [_vp, ctypes.POINTER(Layer), ctypes.POINTER(Layer), ctypes.POINTER(Layer), _i, _vp, _vp, _vp,
                                         _i, _i, _i, _vp, _sz, _vp])
+class GemmLayer(ctypes.Structure):
+    """q4_gemm_layer_t of include/q4_gptq.h."""
+    _fields_ = [("act", _vp), ("qweight", _vp), ("qzeros", _vp), ("scales", _vp), ("bias", _vp), ("la", _vp), ("lb", _vp),
+                ("lb_r", _i), ("lb_c", _i), ("lb_is_f32", _i), ("lb_scale", _f), ("R", _i), ("out", _vp), ("N", _i),
+                ("drop", ctypes.POINTER(Dropout))]
+
+
+SIGNATURES["q4_gemm_grouped_applicable"] = (_i, [_i, _i, _i, _i, ctypes.POINTER(_i)])
+SIGNATURES["q4_gemm_grouped_workspace_bytes"] = (_sz, [_i, _i, _i, _i, ctypes.POINTER(_i)])
+SIGNATURES["q4_gemm_grouped_fwd_f16"] = (_i, [ctypes.POINTER(GemmLayer), _i, _i, _i, _i, _vp])
+SIGNATURES["q4_gemm_grouped_bwd_dx_f16"] = (_i, [ctypes.POINTER(GemmLayer), _i, _i, _vp, _i, _i, _vp, _sz, _vp])
 MAX_GEMV_GROUP = 4
 SIGNATURES["q4_gemv_grouped_workspace_bytes"] = (_sz, [_i, _i])
 SIGNATURES["q4_gemv_grouped_f16"] = (_i, [ctypes.POINTER(GemvLayer), _i, _i, _i, _i, _i, _vp, _sz, _vp])

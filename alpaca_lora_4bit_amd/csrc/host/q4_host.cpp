@@ -398,6 +398,78 @@ at::Tensor gemm_bwd_dx(const at::Tensor& dy, const at::Tensor& qweight, const at
     return o;
 }
 
+// One layer of a grouped GEMM: (qweight, qzeros, scales, bias | None, rank-R operand | None, adapter matrix view | None,
+// adapter scale, dropout (seed, p) | None).  Forward: bias, xa, lora_B^T view; grad-input: no bias, dyb, lora_A.
+using GroupLayer = std::tuple<at::Tensor, at::Tensor, at::Tensor, c10::optional<at::Tensor>, c10::optional<at::Tensor>,
+                              c10::optional<at::Tensor>, double, c10::optional<std::pair<int64_t, double>>>;
+
+// y_i = x @ W_i (+ bias_i) (+ scale_i * xa_i @ lora_bt_i) for 2..4 layers in one launch; raises when the shape does not
+// qualify (the caller falls back to per-layer calls).
+std::vector<at::Tensor> gemm_grouped_fwd(const at::Tensor& x, const std::vector<GroupLayer>& layers, int64_t groupsize) {
+    const size_t n = layers.size();
+    TORCH_CHECK_VALUE(n >= 2 && n <= 4, "gemm_grouped_fwd takes 2..4 layers");
+    q4_gemm_layer_t desc[4];
+    std::vector<at::Tensor> outs;
+    at::Tensor x2;
+    int64_t M = 0, K = 0;
+    c10::optional<c10::Device> dev;
+    for (size_t i = 0; i < n; ++i) {
+        const Layer l = check_layer(std::get<0>(layers[i]), std::get<1>(layers[i]), std::get<2>(layers[i]), c10::nullopt, groupsize);
+        if (i == 0) { dev = l.device; K = l.K; x2 = flat_half(x, K, *dev, "x"); M = x2.size(0); }
+        TORCH_CHECK_VALUE(l.device == *dev && l.K == K, "grouped layers must share the device and K");
+        const auto& bias = std::get<3>(layers[i]);
+        const void* bp = nullptr;
+        if (bias.has_value()) {
+            TORCH_CHECK_VALUE(bias->scalar_type() == at::kHalf && bias->dim() == 1 && bias->size(0) == l.N && bias->is_contiguous() &&
+                              bias->device() == *dev, "bias must be a contiguous float16 [N] tensor on the same device");
+            bp = bias->data_ptr();
+        }
+        const LoraPair lp = check_lora(std::get<4>(layers[i]), std::get<5>(layers[i]), M, l.N, *dev);
+        at::Tensor o = at::empty({M, (int64_t)l.N}, x2.options());
+        desc[i] = q4_gemm_layer_t{x2.data_ptr(), l.qweight, l.qzeros, l.scales, bp, lp.la, lp.lb, lp.sr, lp.sc, lp.f32,
+                                  (float)std::get<6>(layers[i]), lp.R, o.data_ptr(), l.N, nullptr};
+        outs.push_back(o);
+    }
+    Launch L(*dev);
+    const int rc = q4_gemm_grouped_fwd_f16(desc, (int)n, (int)groupsize, (int)M, (int)K, L.stream);
+    if (rc != Q4_OK) raise_q4(rc, "q4_gemm_grouped_fwd_f16");
+    return outs;
+}
+
+// dx = sum_i ( dy_i @ W_i^T + mask_i * scale_i * dyb_i @ lora_a_i ) in one launch and one ordered reduction.
+at::Tensor gemm_grouped_bwd_dx(const std::vector<at::Tensor>& dys, const std::vector<GroupLayer>& layers, int64_t groupsize,
+                               const c10::optional<std::vector<int64_t>>& out_shape) {
+    const size_t n = layers.size();
+    TORCH_CHECK_VALUE(n >= 2 && n <= 4 && dys.size() == n, "gemm_grouped_bwd_dx takes 2..4 layers and one grad_output per layer");
+    q4_gemm_layer_t desc[4];
+    q4_dropout_t drops[4];
+    std::vector<at::Tensor> keep;
+    int n32[4];
+    int64_t M = 0, K = 0;
+    c10::optional<c10::Device> dev;
+    for (size_t i = 0; i < n; ++i) {
+        const Layer l = check_layer(std::get<0>(layers[i]), std::get<1>(layers[i]), std::get<2>(layers[i]), c10::nullopt, groupsize);
+        if (i == 0) { dev = l.device; K = l.K; }
+        TORCH_CHECK_VALUE(l.device == *dev && l.K == K, "grouped layers must share the device and K");
+        at::Tensor dy2 = flat_half(dys[i], l.N, *dev, "grad_output");
+        if (i == 0) M = dy2.size(0);
+        TORCH_CHECK_VALUE(dy2.size(0) == M, "grouped layers must share the number of rows");
+        keep.push_back(dy2);
+        const LoraPair lp = check_lora(std::get<4>(layers[i]), std::get<5>(layers[i]), M, K, *dev);
+        const bool has_drop = fill_drop(std::get<7>(layers[i]), &drops[i]);
+        desc[i] = q4_gemm_layer_t{dy2.data_ptr(), l.qweight, l.qzeros, l.scales, nullptr, lp.la, lp.lb, lp.sr, lp.sc, lp.f32,
+                                  (float)std::get<6>(layers[i]), lp.R, nullptr, l.N, has_drop ? &drops[i] : nullptr};
+        n32[i] = l.N;
+    }
+    at::Tensor dx = at::empty(out_sizes(out_shape, M, K), keep[0].options());
+    Launch L(*dev);
+    size_t have = 0;
+    void* ws = scratch_workspace(*dev, L.stream, q4_gemm_grouped_workspace_bytes(0, (int)n, (int)M, (int)K, n32), &have);
+    const int rc = q4_gemm_grouped_bwd_dx_f16(desc, (int)n, (int)groupsize, dx.data_ptr(), (int)M, (int)K, ws, have, L.stream);
+    if (rc != Q4_OK) raise_q4(rc, "q4_gemm_grouped_bwd_dx_f16");
+    return dx;
+}
+
 at::Tensor lora_down(const at::Tensor& inp, const at::Tensor& w, const c10::optional<std::pair<int64_t, double>>& dropout) {
     TORCH_CHECK_VALUE(inp.is_cuda() && inp.scalar_type() == at::kHalf && inp.dim() == 2 && inp.is_contiguous(),
                       "inp must be a contiguous float16 [M, C] CUDA tensor");
@@ -495,6 +567,9 @@ PYBIND11_MODULE(_q4_host, m) {
     m.def("gemm_bwd_dx", &gemm_bwd_dx, py::arg("dy"), py::arg("qweight"), py::arg("qzeros"), py::arg("scales"), py::arg("g_idx"),
           py::arg("groupsize"), py::arg("dyb") = py::none(), py::arg("lora_a") = py::none(), py::arg("lora_scale") = 1.0,
           py::arg("out_shape") = py::none(), py::arg("dropout") = py::none(), py::arg("out_perm") = py::none());
+    m.def("gemm_grouped_fwd", &gemm_grouped_fwd, py::arg("x"), py::arg("layers"), py::arg("groupsize"));
+    m.def("gemm_grouped_bwd_dx", &gemm_grouped_bwd_dx, py::arg("dys"), py::arg("layers"), py::arg("groupsize"),
+          py::arg("out_shape") = py::none());
     m.def("lora_down", &lora_down, py::arg("inp"), py::arg("w"), py::arg("dropout") = py::none());
     m.def("lora_grad_pair", &lora_grad_pair, py::arg("p1"), py::arg("inp1"), py::arg("p2"), py::arg("inp2"), py::arg("alpha"),
           py::arg("dropout") = py::none());

@@ -30,6 +30,12 @@ int q4_launch_gemv_group(int, const void* const*, const int32_t* const*, const i
 size_t q4_noalloc_scratch_bytes(void);
 void* q4_noalloc_scratch_ptr(int*);
 int q4_launch_zero_words(void*, size_t, hipStream_t);
+int q4_gemm_group_applicable(int, int, int, int, const int*);
+size_t q4_gemm_group_plan_workspace(int, int, int, int, const int*);
+int q4_launch_gemm_group(int, int, const void* const*, const int32_t* const*, const int32_t* const*, const void* const*, int,
+                         const void* const*, const void* const*, const void* const*, const int*, const int*, const int*,
+                         const float*, const int*, void* const*, int, int, const int*, const q4_drop_args* const*, void*, size_t,
+                         hipStream_t);
 int q4_mlp_applicable(int, int, int, int);
 size_t q4_mlp_plan_workspace(int, int, int);
 size_t q4_mlp_status_offset(int, int, int);
@@ -71,7 +77,7 @@ int check_layer(const void* qweight, const void* qzeros, const void* scales, con
 }
 }  // namespace
 
-extern "C" int q4_abi_version(void) { return 12; }
+extern "C" int q4_abi_version(void) { return 13; }
 
 extern "C" const char* q4_error_string(int code) {
     switch (code) {
@@ -339,6 +345,61 @@ extern "C" int q4_gemm_route(int fwd, int M, int K, int N, int groupsize, int ha
         if (q4_skinny_dx_applicable(M, K, N, groupsize, has_g_idx)) return Q4_ROUTE_SKINNY;
     }
     return Q4_ROUTE_TILED;
+}
+
+extern "C" int q4_gemm_grouped_applicable(int fwd, int n_layers, int M, int K, const int* N) {
+    if (!N || n_layers < 2 || n_layers > 4 || M < 1 || K < 128 || (K % 128) != 0) return 0;
+    for (int i = 0; i < n_layers; ++i)
+        if (N[i] < 128 || (N[i] % 128) != 0) return 0;
+    return q4_gemm_group_applicable(fwd, n_layers, M, K, N) ? 1 : 0;
+}
+
+extern "C" size_t q4_gemm_grouped_workspace_bytes(int fwd, int n_layers, int M, int K, const int* N) {
+    if (!N || n_layers < 2 || n_layers > 4 || M < 1 || K < 128) return 0;
+    return q4_gemm_group_plan_workspace(fwd, n_layers, M, K, N);
+}
+
+static int gemm_grouped_common(int fwd, const q4_gemm_layer_t* layers, int n, int groupsize, void* dx, int M, int K,
+                               void* workspace, size_t workspace_bytes, void* stream) {
+    if (!layers) return Q4_ERR_NULL_POINTER;
+    if (n < 2 || n > 4 || M < 1 || (K % 128) != 0 || groupsize < 64 || (groupsize % 64) != 0) return Q4_ERR_BAD_SHAPE;
+    if (!fwd && !dx) return Q4_ERR_NULL_POINTER;
+    if (!fwd && misaligned(dx)) return Q4_ERR_MISALIGNED;
+    const void* act[4]; const int32_t* qw[4]; const int32_t* qz[4]; const void* sc[4]; const void* bias[4];
+    const void* la[4]; const void* lb[4]; int sr[4], scs[4], f32[4], R[4], N[4]; float lsc[4]; void* out[4];
+    q4_drop_args da[4]; const q4_drop_args* dp[4];
+    for (int i = 0; i < n; ++i) {
+        const q4_gemm_layer_t& l = layers[i];
+        const int rc = check_layer(l.qweight, l.qzeros, l.scales, nullptr, groupsize, K, l.N, (K + groupsize - 1) / groupsize);
+        if (rc != Q4_OK) return rc;
+        if ((l.N % 128) != 0) return Q4_ERR_BAD_SHAPE;
+        if ((unsigned long long)(K / 8) * (unsigned long long)l.N * 4ull >= (1ull << 32)) return Q4_ERR_BAD_SHAPE;
+        if ((unsigned long long)(K > l.N ? K : l.N) * 512ull >= (1ull << 32)) return Q4_ERR_BAD_SHAPE;
+        if (!l.act || (fwd && !l.out)) return Q4_ERR_NULL_POINTER;
+        if (fwd && l.act != layers[0].act) return Q4_ERR_BAD_SHAPE;            // the forward shares one x
+        if ((l.la != nullptr) != (l.lb != nullptr)) return Q4_ERR_NULL_POINTER;
+        if (l.la && (l.R < 8 || l.R > 64 || (l.R % 8) != 0 || l.lb_r < 1 || l.lb_c < 1)) return Q4_ERR_BAD_SHAPE;
+        if (misaligned(l.act) || (fwd && misaligned(l.out)) || (l.la && misaligned(l.la))) return Q4_ERR_MISALIGNED;
+        if (l.lb && (reinterpret_cast<uintptr_t>(l.lb) & (l.lb_is_f32 ? 3u : 1u))) return Q4_ERR_MISALIGNED;
+        if (!make_drop(fwd ? nullptr : l.drop, &da[i], &dp[i])) return Q4_ERR_BAD_SHAPE;
+        act[i] = l.act; qw[i] = l.qweight; qz[i] = l.qzeros; sc[i] = l.scales; bias[i] = l.bias; la[i] = l.la; lb[i] = l.lb;
+        sr[i] = l.lb_r; scs[i] = l.lb_c; f32[i] = l.lb_is_f32; lsc[i] = l.lb_scale; R[i] = l.la ? l.R : 0;
+        out[i] = fwd ? l.out : dx; N[i] = l.N;
+    }
+    if (!q4_gemm_group_applicable(fwd, n, M, K, N)) return Q4_ERR_BAD_SHAPE;
+    if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
+    if (q4_gemm_group_plan_workspace(fwd, n, M, K, N) > (workspace ? workspace_bytes : 0)) return Q4_ERR_WORKSPACE;
+    return q4_launch_gemm_group(fwd, n, act, qw, qz, sc, groupsize, bias, la, lb, sr, scs, f32, lsc, R, out, M, K, N, dp,
+                                workspace, workspace ? workspace_bytes : 0, (hipStream_t)stream);
+}
+
+extern "C" int q4_gemm_grouped_fwd_f16(const q4_gemm_layer_t* layers, int n_layers, int groupsize, int M, int K, void* stream) {
+    return gemm_grouped_common(1, layers, n_layers, groupsize, nullptr, M, K, nullptr, 0, stream);
+}
+
+extern "C" int q4_gemm_grouped_bwd_dx_f16(const q4_gemm_layer_t* layers, int n_layers, int groupsize, void* dx, int M, int K,
+                                          void* workspace, size_t workspace_bytes, void* stream) {
+    return gemm_grouped_common(0, layers, n_layers, groupsize, dx, M, K, workspace, workspace_bytes, stream);
 }
 
 extern "C" int q4_lora_down_f16(const void* in, const void* w, int w_sr, int w_sc, int w_is_f32, void* out,

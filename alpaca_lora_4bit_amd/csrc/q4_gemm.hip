@@ -101,8 +101,7 @@ __device__ __forceinline__ TileMap map_tile(int phase_step, int nsteps, int col_
 struct StepRange {
     int begin, cnt;
 };
-__device__ __forceinline__ StepRange split_steps(int nsteps) {
-    const int S = gridDim.z, z = blockIdx.z;
+__device__ __forceinline__ StepRange split_steps(int nsteps, int z, int S) {
     const int base = nsteps / S, rem = nsteps - base * S;
     StepRange r;
     r.cnt = base + (z < rem ? 1 : 0);
@@ -351,7 +350,6 @@ struct BwdSlab {
     }
 };
 
-// FWD: out[M, NOUT=N], reduction length RED=K.   BWD: out[M, NOUT=K], reduction length RED=N.
 // WGM = wavefronts along M (2 or 4); the workgroup has 2*WGM wavefronts = NT threads.
 // SZ: how the sequential-group kernels get scale and zero (fewer vector-memory and vector-ALU instructions in the
 // main loop; 1.5-2.5 % of the kernel):
@@ -361,8 +359,11 @@ struct BwdSlab {
 //   2  backward: from an LDS table of the tile's group, filled once (needs the 128 output rows of a tile in one
 //      group and room for 4 bytes per column n in dynamic LDS)
 // WGN: wavefronts along N (2 or 4), each 64 columns wide: the tile is BM x 64*WGN.
-template <int BM, int WGM, bool FWD, bool GIDX, int SZ = 0, int WGN = 2>
-__global__ __launch_bounds__(64 * WGM * WGN) void gemm_kernel(GemmArgs a) {
+// The body of the kernels below.  `tm`: the output tile; `sr`: this workgroup's share of the reduction; `zsplit` of
+// `nsplit`: which share that is (share 0 carries bias and adapter term); `zpart`: index of its fp32 partial tile.
+template <int BM, int WGM, bool FWD, bool GIDX, int SZ, int WGN>
+__device__ __forceinline__ void gemm_body(const GemmArgs& a, const TileMap tm, const StepRange sr, const int zsplit,
+                                          const int nsplit, const int zpart) {
     constexpr int BNT = 64 * WGN;                     // columns of the tile
     static_assert(SZ == 0 || (!GIDX && ((FWD && SZ == 1) || (!FWD && SZ == 2))), "unsupported scale/zero mode");
     extern __shared__ __attribute__((aligned(16))) unsigned char sz_tab[];
@@ -384,8 +385,6 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_kernel(GemmArgs a) {
     const int wm = wave / WGN, wn = wave % WGN;
     const int NOUT = FWD ? a.N : a.K;
     const int RED = FWD ? a.K : a.N;
-    const StepRange sr = split_steps(RED / BK);
-    const TileMap tm = map_tile(a.phase_step, sr.cnt, a.col_tile0);
     const int m0 = tm.tile_r * BM;
     const int c0 = tm.tile_c * BNT;          // first output column of the tile
     const int rows_valid = min(BM, a.M - m0);
@@ -538,7 +537,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_kernel(GemmArgs a) {
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[0][i], bf[0][j], acc[i][j], 0, 0, 0);
         }
     };
-    const bool lora_here = a.R > 0 && blockIdx.z == 0;
+    const bool lora_here = a.R > 0 && zsplit == 0;
     const bool lora_masked = lora_here && a.drop.thr15 != 0;              // uniform
 
     const int red0 = red_of(0, sr, tm.phase), red1 = red_of(1, sr, tm.phase);
@@ -606,16 +605,16 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_kernel(GemmArgs a) {
     // Each wavefront transposes one 32 x 64 block at a time through its own 4.5 KB of LDS
     // (row stride 72 halves) and writes it as 16-byte pieces: 8 lanes cover one 128-byte row segment.
     const int lc = lane & 31, lrow = (lane >> 5) * 4;
-    if (gridDim.z > 1) {
+    if (nsplit > 1) {
         // split-K: fp32 partial sums straight from the accumulators (32 lanes cover one 128-byte row segment);
         // the bias rides with split 0, the reduction kernel adds the splits in order and rounds once
-        float* const pz = a.part + (size_t)blockIdx.z * a.M * a.part_cols - (size_t)a.col_tile0 * BNT;
+        float* const pz = a.part + (size_t)zpart * a.M * a.part_cols - (size_t)a.col_tile0 * BNT;
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
                 const int col = c0 + wn * 64 + 32 * j + lc;
-                const float bv = blockIdx.z == 0 ? bias_v[j] : 0.f;
+                const float bv = zsplit == 0 ? bias_v[j] : 0.f;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int m = m0 + wm * WROWS + 32 * i + 8 * (r >> 2) + lrow + (r & 3);
@@ -651,6 +650,47 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_kernel(GemmArgs a) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
+// FWD: out[M, NOUT=N], reduction length RED=K.   BWD: out[M, NOUT=K], reduction length RED=N.
+template <int BM, int WGM, bool FWD, bool GIDX, int SZ = 0, int WGN = 2>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_kernel(GemmArgs a) {
+    const StepRange sr = split_steps((FWD ? a.K : a.N) / BK, blockIdx.z, gridDim.z);
+    gemm_body<BM, WGM, FWD, GIDX, SZ, WGN>(a, map_tile(a.phase_step, sr.cnt, a.col_tile0), sr, blockIdx.z, gridDim.z,
+                                           blockIdx.z);
+}
+
+// Up to kGemmGroup layers that share M, K, the group size and (forward) the activations -- q|k|v, gate|up -- in ONE
+// grid, each on its own tensors.
+//   forward:    blockIdx.x walks the column tiles of layer 0, then of layer 1, ...; every workgroup computes one tile of
+//               one layer's own output, over the whole reduction (no split).
+//   grad-input: dx = sum_i dy_i @ W_i^T.  The layers are the "splits" of one launch: blockIdx.z = layer * zs + share,
+//               every workgroup leaves an fp32 partial tile (adapter term and dropout mask of ITS layer included) and
+//               the ordered reduction adds them all into dx: one launch and one reduction instead of one of each per
+//               layer plus the additions of the per-layer results.
+constexpr int kGemmGroup = 4;
+struct GemmGroupArgs {
+    GemmArgs layer[kGemmGroup];
+    int tile_end[kGemmGroup];          // forward: running total of column tiles (tile width of the launch)
+    int zs;                            // grad-input: reduction shares per layer
+};
+
+template <int BM, int WGM, bool FWD, bool GIDX, int SZ = 0, int WGN = 2>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_group_kernel(GemmGroupArgs g) {
+    if constexpr (FWD) {
+        const GemmArgs& a0 = g.layer[0];
+        const StepRange sr = split_steps(a0.K / BK, 0, 1);
+        TileMap tm = map_tile(a0.phase_step, sr.cnt, 0);
+        const int li = (tm.tile_c >= g.tile_end[0]) + (tm.tile_c >= g.tile_end[1]) + (tm.tile_c >= g.tile_end[2]);   // uniform
+        tm.tile_c -= li == 0 ? 0 : g.tile_end[li - 1];
+        const GemmArgs a = g.layer[li];
+        gemm_body<BM, WGM, FWD, GIDX, SZ, WGN>(a, tm, sr, 0, 1, 0);
+    } else {
+        const int li = blockIdx.z / g.zs, zz = blockIdx.z - li * g.zs;
+        const GemmArgs a = g.layer[li];
+        const StepRange sr = split_steps(a.N / BK, zz, g.zs);
+        gemm_body<BM, WGM, FWD, GIDX, SZ, WGN>(a, map_tile(a.phase_step, sr.cnt, 0), sr, zz, gridDim.z, blockIdx.z);
     }
 }
 
@@ -923,6 +963,132 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     if (fwd) e = gidx ? launch_gemm_cfg<true, true>(p, a, nout, stream) : launch_gemm_cfg<true, false>(p, a, nout, stream);
     else e = gidx ? launch_gemm_cfg<false, true>(p, a, nout, stream) : launch_gemm_cfg<false, false>(p, a, nout, stream);
     return e == hipSuccess ? 0 : -4;
+}
+
+// ---- several layers in one launch (sequential groups only) ---------------------------------------------------------
+namespace q4 {
+struct GroupPlan { int cfg; int zs; };      // cfg as in launch_gemm_cfg (0: 128 x 128, 2: 256 x 128, 3: 256 x 256); -1: not applicable
+
+// Forward: one tile of one layer per workgroup, no split, so the launch needs enough tiles by itself.
+// Grad-input: every layer is a share of the reduction (times zs shares per layer when the tiles are few).
+static GroupPlan plan_gemm_group(int fwd, int n, int M, int K, const int* N) {
+    GroupPlan p{-1, 1};
+    if (n < 2 || n > kGemmGroup || M <= 128) return p;
+    const int nr = (M + 255) / 256;
+    if (fwd) {
+        long tot = 0;
+        bool all256 = true;
+        for (int i = 0; i < n; ++i) { tot += N[i]; all256 = all256 && N[i] % 256 == 0; }
+        const long twide = all256 ? (tot / 256) * nr : 0, t256 = (tot / BN) * nr;
+        if (twide >= 144 && (twide <= 256 || 5 * twide >= 4 * 256 * ((twide + 255) / 256))) p.cfg = 3;
+        else if (t256 >= 192) p.cfg = 2;
+        return p;
+    }
+    const long twide = K % 256 == 0 ? (long)(K / 256) * nr * n : 0, t256 = (long)(K / BN) * nr * n;
+    if (twide >= 144 && twide <= 256) { p.cfg = 3; return p; }
+    p.cfg = 2;
+    if (t256 < 192) {
+        int mn = N[0];
+        for (int i = 1; i < n; ++i) mn = N[i] < mn ? N[i] : mn;
+        if (mn / BK >= 16) p.zs = 2;                     // at least eight steps per workgroup
+    }
+    return p;
+}
+
+template <int BM, int WGM, bool FWD, int WGN>
+static void launch_group_tiles(const GemmGroupArgs& g, int n, dim3 grid, hipStream_t stream) {
+    const GemmArgs& a = g.layer[0];
+    const dim3 block(64 * WGM * WGN);
+    if (a.groupsize % 128 == 0) {
+        if constexpr (FWD) {
+            if ((a.K / BK) % 2 == 0 && ((a.phase_step & 0xff) % 2) == 0) {
+                hipLaunchKernelGGL((gemm_group_kernel<BM, WGM, FWD, false, 1, WGN>), grid, block, 0, stream, g);
+                return;
+            }
+        } else if constexpr (WGN == 2) {
+            int mx = 0;
+            for (int i = 0; i < n; ++i) mx = g.layer[i].N > mx ? g.layer[i].N : mx;
+            const size_t tab = (size_t)mx * 4;
+            static const bool attr_ok = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_group_kernel<BM, WGM, FWD, false, 2, WGN>),
+                                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kSzTableMax) == hipSuccess;
+            if (attr_ok && tab <= kSzTableMax) {
+                hipLaunchKernelGGL((gemm_group_kernel<BM, WGM, FWD, false, 2, WGN>), grid, block, tab, stream, g);
+                return;
+            }
+        }
+    }
+    hipLaunchKernelGGL((gemm_group_kernel<BM, WGM, FWD, false, 0, WGN>), grid, block, 0, stream, g);
+}
+}  // namespace q4
+
+extern "C" int q4_gemm_group_applicable(int fwd, int n, int M, int K, const int* N) {
+    return q4::plan_gemm_group(fwd, n, M, K, N).cfg >= 0;
+}
+
+extern "C" size_t q4_gemm_group_plan_workspace(int fwd, int n, int M, int K, const int* N) {
+    const q4::GroupPlan p = q4::plan_gemm_group(fwd, n, M, K, N);
+    if (fwd || p.cfg < 0) return 0;
+    return (size_t)n * p.zs * (size_t)M * (size_t)K * sizeof(float);
+}
+
+// act: forward the shared x (act[i] may all be the same pointer), grad-input dy_i.  out: forward y_i, grad-input out[0] = dx.
+extern "C" int q4_launch_gemm_group(int fwd, int n, const void* const* act, const int32_t* const* qweight,
+                                    const int32_t* const* qzeros, const void* const* scales, int groupsize,
+                                    const void* const* bias, const void* const* la, const void* const* lb, const int* lb_sr,
+                                    const int* lb_sc, const int* lb_is_f32, const float* lb_scale, const int* R,
+                                    void* const* out, int M, int K, const int* N, const q4::DropArgs* const* drop,
+                                    void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    using namespace q4;
+    const GroupPlan p = plan_gemm_group(fwd, n, M, K, N);
+    if (p.cfg < 0) return -2;
+    const size_t need = fwd ? 0 : (size_t)n * p.zs * (size_t)M * (size_t)K * sizeof(float);
+    if (need > 0 && (!workspace || workspace_bytes < need)) return -3;
+    static const int env_phase = getenv("Q4_GEMM_PHASE") ? atoi(getenv("Q4_GEMM_PHASE")) : 2;
+    static const int env_order = getenv("Q4_GEMM_ORDER") ? atoi(getenv("Q4_GEMM_ORDER")) : 2;
+    GemmGroupArgs g;
+    const int tile_w = p.cfg == 3 ? 256 : BN;
+    int tiles = 0;
+    for (int i = 0; i < kGemmGroup; ++i) {
+        const int j = i < n ? i : n - 1;                // unused slots repeat the last layer (never selected)
+        GemmArgs& a = g.layer[i];
+        a.drop = (drop && drop[j]) ? *drop[j] : DropArgs{0u, 0u, 0u, 1.0f};
+        a.a = reinterpret_cast<const half_t*>(act[j]);
+        a.qweight = reinterpret_cast<const uint32_t*>(qweight[j]);
+        a.qzeros = reinterpret_cast<const uint32_t*>(qzeros[j]);
+        a.scales = reinterpret_cast<const half_t*>(scales[j]);
+        a.g_idx = nullptr;
+        a.groupsize = groupsize;
+        a.gs_inv31 = (uint32_t)(((1ull << 31) + (uint64_t)(groupsize / 64) - 1) / (uint64_t)(groupsize / 64));
+        a.bias = fwd && bias ? reinterpret_cast<const half_t*>(bias[j]) : nullptr;
+        a.la = la ? reinterpret_cast<const half_t*>(la[j]) : nullptr;
+        a.lb = lb ? lb[j] : nullptr;
+        a.R = (a.la && a.lb) ? R[j] : 0;
+        a.lb_sr = a.R ? lb_sr[j] : 0; a.lb_sc = a.R ? lb_sc[j] : 0; a.lb_is_f32 = a.R ? lb_is_f32[j] : 0;
+        a.lb_scale = (a.R ? lb_scale[j] : 0.f) * a.drop.scale;
+        a.out = reinterpret_cast<half_t*>(fwd ? out[j] : out[0]);
+        a.M = M; a.K = K; a.N = N[j]; a.G = (K + groupsize - 1) / groupsize;
+        a.phase_step = (env_phase < 0 ? 0 : env_phase) | (env_order > 0 ? (env_order > 64 ? 64 : env_order) << 8 : 0);
+        a.part = reinterpret_cast<float*>(workspace);
+        a.col_tile0 = 0;
+        a.part_cols = fwd ? N[j] : K;
+        if (i < n) tiles += N[i] / tile_w;
+        g.tile_end[i] = i < n ? tiles : 0x7fffffff;
+    }
+    g.zs = p.zs;
+    const int bm = p.cfg == 0 ? 128 : 256;
+    const int nr = (M + bm - 1) / bm;
+    const dim3 grid(fwd ? tiles : K / tile_w, nr, fwd ? 1 : n * p.zs);
+    if (fwd) {
+        if (p.cfg == 3) launch_group_tiles<256, 2, true, 4>(g, n, grid, stream);
+        else launch_group_tiles<256, 4, true, 2>(g, n, grid, stream);
+    } else {
+        if (p.cfg == 3) launch_group_tiles<256, 2, false, 4>(g, n, grid, stream);
+        else launch_group_tiles<256, 4, false, 2>(g, n, grid, stream);
+        const long total = (long)M * K;
+        hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, stream,
+                           g.layer[0].part, g.layer[0].out, total, n * p.zs);
+    }
+    return hipGetLastError() == hipSuccess ? 0 : -4;
 }
 
 // Workspace that lets q4_launch_gemm use its preferred split for this shape (0: no split wanted).

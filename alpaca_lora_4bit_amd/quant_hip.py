@@ -661,6 +661,43 @@ def gemm_fwd(x, qweight, qzeros, scales, g_idx=None, groupsize=None, bias=None, 
     return out
 
 
+def gemm_grouped_applicable(fwd, M, K, Ns):
+    """True when gemm_grouped_fwd / gemm_grouped_bwd_dx take this shape (2..4 layers, more than 128 rows, enough tiles
+    for one launch); the layers must also have sequential groups and scales below 64 (checked by those calls)."""
+    n = len(Ns)
+    if not 2 <= n <= 4:
+        return False
+    arr = (ctypes.c_int * n)(*[int(v) for v in Ns])
+    return bool(_lib.lib().q4_gemm_grouped_applicable(int(bool(fwd)), n, int(M), int(K), arr))
+
+
+def _group_layer_ok(lay, groupsize):
+    info = _layer_info(lay[0], lay[1], lay[2], None, groupsize)
+    return info.plan is None and info.gemm_args()[0] is None
+
+
+def gemm_grouped_fwd(x, layers, groupsize):
+    """[x @ W_i (+ bias_i) (+ scale_i * xa_i @ lora_bt_i)] for 2..4 layers that share x, K and the group size, in ONE
+    launch over the layers' own tensors (q|k|v or gate|up of a decoder block above 128 rows).  `layers`: list of
+    (qweight, qzeros, scales, bias | None, xa | None, lora_bt | None, lora_scale).  Returns the [M, N_i] outputs."""
+    _require(_host is not None, "gemm_grouped_fwd needs the compiled host binding (_q4_host)")
+    for lay in layers:
+        _require(_group_layer_ok(lay, groupsize), "gemm_grouped_fwd needs sequential groups and scales below 64")
+    return _host.gemm_grouped_fwd(x, [(l[0], l[1], l[2], l[3], l[4], l[5], float(l[6]), None) for l in layers], int(groupsize))
+
+
+def gemm_grouped_bwd_dx(dys, layers, groupsize, out_shape=None):
+    """dx = sum_i (dy_i @ W_i^T + mask_i * scale_i * dyb_i @ lora_a_i): the grad-inputs of 2..4 layers that share their
+    input, summed, in one launch and one ordered reduction.  `layers`: list of (qweight, qzeros, scales, dyb | None,
+    lora_a | None, lora_scale, dropout (seed, p) | None)."""
+    _require(_host is not None, "gemm_grouped_bwd_dx needs the compiled host binding (_q4_host)")
+    for lay in layers:
+        _require(_group_layer_ok(lay, groupsize), "gemm_grouped_bwd_dx needs sequential groups and scales below 64")
+    return _host.gemm_grouped_bwd_dx(list(dys), [(l[0], l[1], l[2], None, l[3], l[4], float(l[5]),
+                                                  None if l[6] is None else (int(l[6][0]), float(l[6][1]))) for l in layers],
+                                     int(groupsize), _shape_arg(out_shape))
+
+
 def _drop_arg(dropout):
     """(seed, p) -> ctypes descriptor (kept alive by the caller for the duration of the call), or None."""
     if dropout is None:

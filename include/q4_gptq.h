@@ -250,6 +250,38 @@ Q4_API int q4_gemm_bwd_dx_f16(const void *dy, const int32_t *qweight, const int3
                        int R, void *dx, int M, int K, int N, int G, const q4_dropout_t *drop,
                        void *workspace, size_t workspace_bytes, void *stream);
 
+/* The two GEMMs for 2..4 layers that share M, K and the group size (q|k|v, gate|up of a decoder block), each on its
+ * own tensors, in ONE launch.  Sequential groups only (no g_idx), every |scale| < 64, M > 128; otherwise, and for
+ * shapes with too few tiles to fill the GPU, Q4_ERR_BAD_SHAPE: use the per-layer entry points.
+ *   q4_gemm_grouped_fwd_f16:     y_i [M, N_i] = x @ W_i (+ bias_i) (+ lb_scale_i * la_i @ Lb_i), la_i = xa_i [M, R_i];
+ *                                act of every layer = x.  No workspace.
+ *   q4_gemm_grouped_bwd_dx_f16:  dx [M, K] = sum_i ( dy_i @ W_i^T + mask_i * lb_scale_i * la_i @ Lb_i ), act = dy_i
+ *                                [M, N_i], la_i = dyb_i [M, R_i], Lb_i = lora_A_i [R_i, K], mask_i the dropout mask of
+ *                                drop_i (NULL: none).  The layers are the shares of one split reduction: fp32 partial
+ *                                tiles in `workspace` (q4_gemm_grouped_workspace_bytes), added in a fixed order.
+ * They replace the per-projection recons + torch.matmul calls (matmul_utils_4bit.py:114-127) that the reference fuses
+ * by concatenating the packed tensors (model_attn_mlp_patch.py:88-100, 180-190), and for the grad-input also the
+ * additions with which autograd sums the per-projection results.  Lb_i[r, c] = lb[r*lb_r + c*lb_c], fp16 or fp32. */
+typedef struct {
+    const void *act;
+    const int32_t *qweight, *qzeros;
+    const void *scales;
+    const void *bias;             /* forward only; fp16 [N] or NULL */
+    const void *la, *lb;          /* both NULL: no adapter term */
+    int lb_r, lb_c, lb_is_f32;
+    float lb_scale;
+    int R;                        /* 0 or a multiple of 8, at most 64 */
+    void *out;                    /* forward: y_i; grad-input: unused */
+    int N;
+    const q4_dropout_t *drop;     /* grad-input only */
+} q4_gemm_layer_t;
+/* 1 when the two entry points below take this shape (enough tiles for one launch), 0 otherwise. */
+Q4_API int q4_gemm_grouped_applicable(int fwd, int n_layers, int M, int K, const int *N);
+Q4_API size_t q4_gemm_grouped_workspace_bytes(int fwd, int n_layers, int M, int K, const int *N);
+Q4_API int q4_gemm_grouped_fwd_f16(const q4_gemm_layer_t *layers, int n_layers, int groupsize, int M, int K, void *stream);
+Q4_API int q4_gemm_grouped_bwd_dx_f16(const q4_gemm_layer_t *layers, int n_layers, int groupsize, void *dx, int M, int K,
+                                      void *workspace, size_t workspace_bytes, void *stream);
+
 /* Rank-R down projection of the adapter:  out fp16 [M, R] = in fp16 [M, C] @ Wm^T,
  * Wm[j, c] = w[j*w_sr + c*w_sc] (fp16, or fp32 when w_is_f32 != 0).  xa = x @ A^T (w = lora_A.weight,
  * w_sr = K, w_sc = 1) and dyb = dy @ B (w = lora_B.weight, w_sr = 1, w_sc = R): the two products that
