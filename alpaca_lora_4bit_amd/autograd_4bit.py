@@ -195,6 +195,13 @@ class Autograd4bitQuantLinear(nn.Module):
                 if not self.disable_bias and not _is_all_zero(self.bias):
                     out += self.bias
                 return out
+        group = self.__dict__.get('_q4_group')
+        if group is not None and self.bits == 4 and not self.is_v1_model and backend == 'cuda':
+            # a member of a group made by model_attn_mlp_patch, above the decode sizes: one grouped GEMM launch for
+            # all members (forward and, under autograd, grad-input), each member picks its output up
+            out = group.run_gemm(self, x)
+            if out is not None:
+                return out
         zeros = self.zeros if self.is_v1_model else self.qzeros
         if self.bits == 4:
             if torch.is_grad_enabled():
@@ -323,6 +330,33 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
         return out.addmm_(act, w)
 
     @staticmethod
+    def _adapter_grads(dyb, x2, xa, dy, scaling, dropout, need_a, need_b, ab_dtypes):
+        """(dA, dB) = scaling * (dyb^T @ dropout(x), dy^T @ xa) in the parameters' dtypes (None where not needed)."""
+        da = db = None
+        r = dyb.shape[1]
+        if need_a and need_b and r in quant_hip.LORA_GRAD_RANKS:
+            da, db = quant_hip.lora_grad_pair(dyb, x2, xa, dy, scaling, dropout=dropout)   # one launch for both gradients
+        else:
+            if need_a:
+                if r in quant_hip.LORA_GRAD_RANKS:
+                    da = quant_hip.lora_grad(dyb, x2, scaling, dropout=dropout)
+                elif dropout is not None:
+                    xd = x2 * quant_hip.dropout_keep_mask(x2.shape[0], x2.shape[1], dropout[0], dropout[1], x2.device)
+                    da = torch.mm(dyb.t(), xd).float().mul_(scaling * quant_hip.dropout_scale(dropout[1]))
+                else:
+                    da = torch.mm(dyb.t(), x2).float().mul_(scaling)
+            if need_b:
+                if r in quant_hip.LORA_GRAD_RANKS:
+                    db = quant_hip.lora_grad(xa, dy, scaling, transposed=True)
+                else:
+                    db = torch.mm(dy.t(), xa).float().mul_(scaling)
+        if da is not None:
+            da = da.to(ab_dtypes[0])
+        if db is not None:
+            db = db.to(ab_dtypes[1])
+        return da, db
+
+    @staticmethod
     @custom_fwd(device_type='cuda', cast_inputs=None)
     def forward(ctx, x, qweight, scales, zeros, g_idx, bias, lora_a, lora_b, scaling, groupsize, drop_p=0.0,
                 drop_seed=0):
@@ -375,27 +409,99 @@ class AutogradMatmul4bitLora(torch.autograd.Function):
             else:
                 dx = quant_hip.gemm_bwd_dx(dy, qweight, zeros, scales, g_idx, ctx.groupsize, dyb=dyb, lora_a=a,
                                            lora_scale=ctx.scaling, out_shape=dx_shape, dropout=dropout)
-        if need_a and need_b and r in quant_hip.LORA_GRAD_RANKS:
-            da, db = quant_hip.lora_grad_pair(dyb, x2, xa, dy, ctx.scaling, dropout=dropout)   # one launch for both gradients
-        else:
-            if need_a:
-                if r in quant_hip.LORA_GRAD_RANKS:
-                    da = quant_hip.lora_grad(dyb, x2, ctx.scaling, dropout=dropout)
-                elif dropout is not None:
-                    xd = x2 * quant_hip.dropout_keep_mask(x2.shape[0], x2.shape[1], dropout[0], dropout[1], x2.device)
-                    da = torch.mm(dyb.t(), xd).float().mul_(ctx.scaling * quant_hip.dropout_scale(dropout[1]))
-                else:
-                    da = torch.mm(dyb.t(), x2).float().mul_(ctx.scaling)
-            if need_b:
-                if r in quant_hip.LORA_GRAD_RANKS:
-                    db = quant_hip.lora_grad(xa, dy, ctx.scaling, transposed=True)
-                else:
-                    db = torch.mm(dy.t(), xa).float().mul_(ctx.scaling)
-        if da is not None:
-            da = da.to(ctx.ab_dtypes[0])
-        if db is not None:
-            db = db.to(ctx.ab_dtypes[1])
+        da, db = AutogradMatmul4bitLora._adapter_grads(dyb, x2, xa, dy, ctx.scaling, dropout, need_a, need_b, ctx.ab_dtypes)
         return dx, None, None, None, None, None, da, db, None, None, None, None
+
+
+class AutogradMatmul4bitGroup(torch.autograd.Function):
+    """The products of 2..4 layers that share their input (q|k|v, gate|up of a decoder block), LoRA adapters included,
+    as ONE node: forward = one grouped launch on the layers' own tensors, backward = one grouped grad-input launch
+    whose ordered reduction also does the sum over the layers that autograd would otherwise add up.
+
+    No counterpart in the reference as a single op; per layer it computes what AutogradMatmul4bitCuda
+    (autograd_4bit.py:32-54) and, for a layer with an adapter, the adapter lines of Linear4bitLt.forward
+    (models.py:58-66) compute, and the reference reaches the single launch by concatenating the packed tensors
+    (model_attn_mlp_patch.py:88-100, 180-190).
+
+    apply(x, groupsize, specs, *tensors): specs[i] = (scaling | None, drop_p, drop_seed) of layer i; tensors holds six
+    entries per layer: qweight, scales, qzeros, bias | None, lora_A.weight | None, lora_B.weight | None.
+    Returns one output per layer."""
+
+    @staticmethod
+    @custom_fwd(device_type='cuda', cast_inputs=None)
+    def forward(ctx, x, groupsize, specs, *tensors):
+        n = len(specs)
+        lay = [tensors[6 * i:6 * i + 6] for i in range(n)]
+        K = lay[0][0].shape[0] * 8
+        x2 = x.reshape(-1, K)
+        if x2.dtype != torch.float16:
+            x2 = x2.half()
+        x2 = x2.contiguous()
+        fwd, xas, adapters, dropouts = [], [], [], []
+        for (qweight, scales, zeros, bias, lora_a, lora_b), (scaling, drop_p, drop_seed) in zip(lay, specs):
+            if bias is not None and bias.dtype != torch.float16:
+                bias = bias.half()
+            dropout = (int(drop_seed), float(drop_p)) if drop_p and drop_p > 0.0 else None
+            if lora_a is not None:
+                a = AutogradMatmul4bitLora._kernel_dtype(lora_a.detach())
+                b = AutogradMatmul4bitLora._kernel_dtype(lora_b.detach())
+                xa = quant_hip.lora_down(x2, a, dropout=dropout)
+                fwd.append((qweight, zeros, scales, bias, xa, b.t(), scaling))
+            else:
+                a = b = xa = None
+                fwd.append((qweight, zeros, scales, bias, None, None, 1.0))
+            xas.append(xa); adapters.append((a, b)); dropouts.append(dropout)
+        ys = quant_hip.gemm_grouped_fwd(x2, fwd, groupsize)
+        lead = tuple(x.shape[:-1])
+        saved = [x2]
+        for (qweight, scales, zeros, _, _, _), xa, (a, b) in zip(lay, xas, adapters):
+            saved += [qweight, scales, zeros] + ([xa, a, b] if a is not None else [])
+        ctx.save_for_backward(*saved)
+        ctx.specs = specs
+        ctx.groupsize = groupsize
+        ctx.has_adapter = [a is not None for a, _ in adapters]
+        ctx.dropouts = dropouts
+        ctx.ab_dtypes = [(l[4].dtype, l[5].dtype) if l[4] is not None else None for l in lay]
+        return tuple(y.view(lead + (y.shape[-1],)) for y in ys)
+
+    @staticmethod
+    @custom_bwd(device_type='cuda')
+    def backward(ctx, *grad_outputs):
+        saved = list(ctx.saved_tensors)
+        x2 = saved.pop(0)
+        n = len(ctx.specs)
+        grads = [None] * (6 * n)
+        layers, dys, per_layer = [], [], []
+        for i in range(n):
+            qweight, scales, zeros = saved.pop(0), saved.pop(0), saved.pop(0)
+            xa = a = b = None
+            if ctx.has_adapter[i]:
+                xa, a, b = saved.pop(0), saved.pop(0), saved.pop(0)
+            N = qweight.shape[1]
+            g = grad_outputs[i]
+            if g is None:
+                dy = torch.zeros((x2.shape[0], N), dtype=torch.float16, device=x2.device)
+            else:
+                dy = g.reshape(-1, N)
+                if dy.dtype != torch.float16:
+                    dy = dy.half()
+                dy = dy.contiguous()
+            dyb = quant_hip.lora_down(dy, b.t()) if a is not None else None
+            dys.append(dy)
+            layers.append((qweight, zeros, scales, dyb, a, ctx.specs[i][0] if a is not None else 1.0, ctx.dropouts[i]))
+            per_layer.append((xa, dyb, dy))
+        dx = None
+        if ctx.needs_input_grad[0]:
+            lead = next((tuple(g.shape[:-1]) for g in grad_outputs if g is not None), (x2.shape[0],))
+            dx = quant_hip.gemm_grouped_bwd_dx(dys, layers, ctx.groupsize, out_shape=lead + (x2.shape[1],))
+        for i in range(n):
+            if ctx.has_adapter[i]:
+                xa, dyb, dy = per_layer[i]
+                need_a, need_b = ctx.needs_input_grad[3 + 6 * i + 4], ctx.needs_input_grad[3 + 6 * i + 5]
+                if need_a or need_b:
+                    grads[6 * i + 4], grads[6 * i + 5] = AutogradMatmul4bitLora._adapter_grads(
+                        dyb, x2, xa, dy, ctx.specs[i][0], ctx.dropouts[i], need_a, need_b, ctx.ab_dtypes[i])
+        return (dx, None, None) + tuple(grads)
 
 
 _LOADER_NAMES = ('load_llama_model_4bit_low_ram', 'load_llama_model_4bit_low_ram_and_offload',

@@ -82,6 +82,7 @@ class _MemberGroup:
         self.groupsize = self.members[0].groupsize
         self.usable = None                                   # decided at the first call (needs the tensors on the GPU)
         self._layer_cache = None
+        self._gemm_ok = None                                 # sequential groups AND scales below 64 (the tiled kernels' fused form)
         self.hook = None
         self.clear()
 
@@ -104,6 +105,7 @@ class _MemberGroup:
                                       for m, c in zip(self.members, cached)):
             return cached
         self.usable = self._check()
+        self._gemm_ok = None
         self._layer_cache = [(m.qweight, m.qzeros, m.scales) for m in self.members] if self.usable else None
         return self._layer_cache
 
@@ -124,10 +126,67 @@ class _MemberGroup:
             self._x = None
         return y
 
+    def _gemm_spec(self, m, x):
+        """How member `m` enters a grouped GEMM for input x: (bias | None, lora_A | None, lora_B | None, scaling, drop_p)."""
+        from .autograd_4bit import _is_all_zero
+        bias = None
+        if not m.disable_bias and not _is_all_zero(m.bias):
+            bias = m.bias
+        name = None
+        if type(m) is not Autograd4bitQuantLinear and not getattr(m, 'disable_adapters', False):
+            name = m._fusable_adapter(x)                     # the adapter rides in the launch; otherwise the layer adds it
+        if name is None:
+            return (bias, None, None, None, 0.0)
+        return (bias, m.lora_A[name].weight, m.lora_B[name].weight, float(m.scaling[name]), m._dropout_p(name))
+
+    def run_gemm(self, member, x):
+        """Above the decode sizes: ONE grouped GEMM launch for all members (under autograd one node, whose backward is
+        one grouped grad-input launch).  Returns the member's output, bias and fused adapter included, or None when
+        the group does not take this call (the member then runs by itself)."""
+        i = self.index[id(member)]
+        key = (x._version, torch.is_grad_enabled())
+        if self._gx is x and self._gkey == key and self._gouts[i] is not None:
+            y, self._gouts[i] = self._gouts[i], None
+            if all(o is None for o in self._gouts):
+                self._gx = None
+            return y
+        from . import autograd_4bit, quant_hip
+        layers = self._layers()
+        if layers is None or not x.is_cuda or x.shape[-1] != member.in_features:
+            return None
+        rows = x.numel() // member.in_features
+        if rows <= quant_hip.MAX_GEMV_ROWS or not (x.dtype == torch.float16 or torch.is_autocast_enabled('cuda')):
+            return None
+        if matmul_utils_4bit.use_dense_route(rows) or member.in_features % 128 or any(m.out_features % 128 for m in self.members):
+            return None
+        Ns = [m.out_features for m in self.members]
+        grad = torch.is_grad_enabled()
+        if not quant_hip.gemm_grouped_applicable(True, rows, member.in_features, Ns) or \
+                (grad and not quant_hip.gemm_grouped_applicable(False, rows, member.in_features, Ns)):
+            return None
+        if self._gemm_ok is None:
+            self._gemm_ok = all(quant_hip._group_layer_ok(l, self.groupsize) for l in layers)
+        if not self._gemm_ok:
+            return None
+        specs, tensors = [], []
+        for m, (qweight, qzeros, scales) in zip(self.members, layers):
+            bias, la, lb, scaling, drop_p = self._gemm_spec(m, x)
+            seed = int(torch.randint(0, 2 ** 62, (1,)).item()) if drop_p > 0.0 else 0
+            specs.append((scaling, drop_p, seed))
+            tensors += [qweight, scales, qzeros, bias, la, lb]
+        outs = autograd_4bit.AutogradMatmul4bitGroup.apply(x, self.groupsize, tuple(specs), *tensors)
+        self._gouts = list(outs)
+        self._gx, self._gkey = x, key
+        y, self._gouts[i] = self._gouts[i], None
+        return y
+
     def clear(self, *unused):
         self._x = None
         self._version = -1
         self._outs = [None] * len(self.members)
+        self._gx = None
+        self._gkey = None
+        self._gouts = [None] * len(self.members)
 
     def replace(self, old, new):
         """`new` (for instance a LoRA layer sharing `old`'s packed tensors) takes `old`'s place in the group."""

@@ -182,6 +182,11 @@ class Linear4bitLt(Autograd4bitQuantLinear, LoraLayer):
                 return result
             name = self._fusable_adapter(x)
             if name is not None:
+                group = self.__dict__.get('_q4_group')
+                if group is not None:
+                    out = group.run_gemm(self, x)            # one grouped launch for all members, adapters included
+                    if out is not None:
+                        return out
                 bias = None
                 if not self.disable_bias and not autograd_4bit._is_all_zero(self.bias):
                     bias = self.bias if self.bias.dtype == torch.float16 else self.bias.half()

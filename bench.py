@@ -387,17 +387,23 @@ def bench_llama7b_decode(new_tokens=64, prompt=16, seed=13):
     return res
 
 
-def bench_llama7b_lora_train_step(reps=4, seed=11, n_layers=32, batch=4, seq=256):
+def bench_llama7b_lora_train_step(reps=4, seed=11, n_layers=32, batch=4, seq=256, grouped=True):
     """configs[4] of the benchmark definition: random-init 32-layer LLaMA-7B decoder, every q/k/v/o/gate/up/down projection a 4-bit
     GPTQ layer (groupsize 128), LoRA r=8 alpha=16 on q_proj / v_proj, one forward + backward + AdamW step on
     batch 4 x seq 256 random token ids under fp16 autocast, gradient checkpointing off.  Eager PyTorch around
-    the HIP kernels (attention = torch SDPA, lm_head = library GEMM)."""
+    the HIP kernels (attention = torch SDPA, lm_head = library GEMM).  grouped: q|k|v and gate|up of every block
+    grouped in place (model_attn_mlp_patch.make_quant_attn / make_fused_mlp): one forward and one grad-input launch
+    per group, on the layers' own tensors."""
     import torch
     from alpaca_lora_4bit_amd import autograd_4bit as ag
     from alpaca_lora_4bit_amd.models import inject_lora_layers
     gen = torch.Generator(device="cuda").manual_seed(seed)
     model = _random_llama7b(gen, n_layers)
     lora = inject_lora_layers(model, target_modules=("q_proj", "v_proj"), r=8, lora_alpha=16)
+    if grouped:
+        from alpaca_lora_4bit_amd.model_attn_mlp_patch import make_fused_mlp, make_quant_attn
+        make_quant_attn(model)
+        make_fused_mlp(model)
     with torch.no_grad():
         for l in lora.values():
             l.lora_B["default"].weight.normal_(0, 0.02, generator=gen)
@@ -584,6 +590,8 @@ def main():
                          "FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--llama7b-step-only", action="store_true",
                     help="run only the config-4 full-model LoRA training step (32-layer LLaMA-7B shapes, random init)")
+    ap.add_argument("--ungrouped", action="store_true",
+                    help="with --llama7b-step-only: every projection its own launch (no in-place grouping of q|k|v, gate|up)")
     ap.add_argument("--llama7b-decode-only", action="store_true",
                     help="run only the greedy decode of the random-init 4-bit LLaMA-7B through transformers' generate")
     ap.add_argument("--dequant-only", action="store_true",
@@ -609,8 +617,9 @@ def main():
         print(json.dumps({"workload": "llama7b_greedy_decode_b1", **{k: (round(v, 2) if isinstance(v, float) else v) for k, v in r.items()}}))
         return
     if args.llama7b_step_only:
-        r = bench_llama7b_lora_train_step(max(args.steps, 2))
-        print(json.dumps({"workload": "config4_llama7b_lora_train_step_b4_s256", **{k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()}}))
+        r = bench_llama7b_lora_train_step(max(args.steps, 2), grouped=not args.ungrouped)
+        print(json.dumps({"workload": "config4_llama7b_lora_train_step_b4_s256", "grouped": not args.ungrouped,
+                          **{k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()}}))
         return
     if args.dequant_only:
         r = bench_dequant(4096, 11008, False, max(args.steps, 5))
@@ -711,8 +720,11 @@ def main():
         try:
             with contextlib.redirect_stdout(sys.stderr):
                 c4 = bench_llama7b_lora_train_step(4)
+                c4u = bench_llama7b_lora_train_step(4, grouped=False)
             extra["config4_llama7b_lora_train_step_b4_s256"] = {k: (round(v, 4) if isinstance(v, float) else v)
                                                                   for k, v in c4.items()}
+            extra["config4_llama7b_lora_train_step_b4_s256"]["projections"] = "q|k|v and gate|up grouped in place"
+            extra["config4_llama7b_lora_train_step_b4_s256"]["ms_per_step_every_projection_its_own_launch"] = round(c4u["ms_per_step"], 4)
         except Exception as e:                       # the headline line must not depend on the installed transformers
             extra["config4_llama7b_lora_train_step_b4_s256"] = {"error": f"{type(e).__name__}: {e}"[:300]}
         try:

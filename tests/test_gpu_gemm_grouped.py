@@ -95,3 +95,84 @@ def test_grouped_gemm_refuses_what_it_does_not_take(oracle):
     assert L.q4_gemm_grouped_fwd_f16(desc, 2, 128, 256, 256, None) == -2                   # not enough tiles
     assert L.q4_gemm_grouped_fwd_f16(None, 2, 128, 256, 256, None) == -1
     assert L.q4_gemm_grouped_bwd_dx_f16(desc, 2, 128, None, 256, 256, None, 0, None) == -1
+
+
+class _Block:
+    """Stands for an attention block: three projections of one input, two of them with LoRA adapters."""
+
+    def __new__(cls, oracle, K, N, gs, dropout, seed):
+        import torch
+        import torch.nn as nn
+        from alpaca_lora_4bit_amd import autograd_4bit as ag, models
+
+        class Block(nn.Module):
+            def __init__(self):
+                super().__init__()
+                for i, name in enumerate(("q_proj", "k_proj", "v_proj")):
+                    lay = oracle.make_layer(K, N, gs, seed=seed + i)
+                    if name == "k_proj":
+                        m = ag.Autograd4bitQuantLinear(K, N, groupsize=gs)
+                    else:
+                        m = models.Linear4bitLt("default", K, N, gs, False, r=8, lora_alpha=16, lora_dropout=dropout)
+                        A, B = oracle.make_lora(K, N, 8, seed=seed + 10 + i)
+                        m.lora_A["default"].weight.data = torch.from_numpy(A)
+                        m.lora_B["default"].weight.data = torch.from_numpy(B)
+                    m.qweight.data = torch.from_numpy(lay["qweight"])
+                    m.qzeros.data = torch.from_numpy(lay["qzeros"])
+                    m.scales = torch.from_numpy(lay["scales"])
+                    m.g_idx.data = torch.from_numpy(lay["g_idx"])
+                    m.bias = torch.zeros(N, dtype=torch.float16) if name != "v_proj" else (torch.arange(N) % 7 - 3).half() * 0.25
+                    setattr(self, name, m)
+
+            def forward(self, x):
+                return self.q_proj(x), self.k_proj(x), self.v_proj(x)
+        return Block().cuda()
+
+
+@pytest.mark.parametrize("dropout", [0.0, 0.1])
+def test_grouped_block_matches_the_ungrouped_block_forward_and_gradients(oracle, dropout, monkeypatch):
+    """make_quant_attn on a block above the decode sizes: q|k|v (LoRA on q and v, a bias on v) run as ONE grouped
+    forward launch and, in backward, ONE grouped grad-input launch.  Outputs, grad_input and adapter gradients
+    against the same block ungrouped (whose layers are held to the oracle in test_gpu_autograd.py); with adapter
+    dropout both draw their mask seeds in the same order, so the masks are the same."""
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    from alpaca_lora_4bit_amd.model_attn_mlp_patch import make_quant_attn, ungroup
+    K, N, gs, M = 1024, 4096, 128, 512
+    grouped, plain = _Block(oracle, K, N, gs, dropout, 40), _Block(oracle, K, N, gs, dropout, 40)
+    assert make_quant_attn(grouped) == 1
+    grouped.train(); plain.train()
+    calls = {"fwd": 0, "bwd": 0}
+    for name, key in (("gemm_grouped_fwd", "fwd"), ("gemm_grouped_bwd_dx", "bwd")):
+        real = getattr(quant_hip, name)
+        monkeypatch.setattr(quant_hip, name, (lambda real, key: lambda *a, **k: (calls.__setitem__(key, calls[key] + 1), real(*a, **k))[1])(real, key))
+    xh = oracle.make_activations(M, K, seed=3)
+    gys = [_t(oracle.make_activations(M, N, seed=4 + i)).view(2, M // 2, N) for i in range(3)]
+    results = []
+    for block in (grouped, plain):
+        torch.manual_seed(1234)
+        x = _t(xh).view(2, M // 2, K).requires_grad_(True)
+        with torch.amp.autocast(device_type="cuda", dtype=torch.float16):
+            ys = block(x)
+        torch.autograd.backward(ys, gys)
+        grads = [p.grad.clone() for p in block.parameters() if p.requires_grad]
+        results.append(([y.detach() for y in ys], x.grad.clone(), grads))
+        block.zero_grad()
+    assert calls == {"fwd": 1, "bwd": 1}
+    (ys_g, dx_g, gr_g), (ys_p, dx_p, gr_p) = results
+    for a, b in zip(ys_g, ys_p):
+        assert a.shape == (2, M // 2, N)
+        assert float((a.float() - b.float()).abs().max() / b.float().abs().max()) <= 2e-3
+    assert float((dx_g.float() - dx_p.float()).abs().max() / dx_p.float().abs().max()) <= 3e-3
+    assert len(gr_g) == 4
+    for a, b in zip(gr_g, gr_p):
+        assert float((a.float() - b.float()).abs().max() / b.float().abs().max()) <= 3e-3
+    # no grad, eval: the same grouped launch for a prefill-sized input; 8 rows go to the grouped GEMV
+    grouped.eval(); plain.eval()
+    with torch.no_grad():
+        for rows in (M, 8):
+            x = _t(xh)[:rows]
+            for a, b in zip(grouped(x), plain(x)):
+                assert float((a.float() - b.float()).abs().max() / b.float().abs().max()) <= 2e-3
+    assert calls["fwd"] == 2
+    assert ungroup(grouped) == 1 and "_q4_group" not in grouped.k_proj.__dict__
