@@ -230,8 +230,7 @@ extern "C" int q4_mlp_decode_f16(const void* x, const q4_layer_t* gate, const q4
         return Q4_ERR_MISALIGNED;
     if (!workspace || workspace_bytes < q4_mlp_plan_workspace(M, H, I)) return Q4_ERR_WORKSPACE;
     if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0) return Q4_ERR_MISALIGNED;
-    static const int env_polls = getenv("Q4_MLP_POLL_LIMIT") ? atoi(getenv("Q4_MLP_POLL_LIMIT")) : 0;
-    return q4_launch_mlp(x, qw, qz, sc, groupsize, gate_out, up_out, y, M, H, I, workspace, env_polls, (hipStream_t)stream);
+    return q4_launch_mlp(x, qw, qz, sc, groupsize, gate_out, up_out, y, M, H, I, workspace, 0, (hipStream_t)stream);
 }
 
 extern "C" size_t q4_gemv_noalloc_max_outputs(void) { return q4_noalloc_scratch_bytes() / 8; }

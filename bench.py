@@ -594,6 +594,8 @@ def main():
                     help="with --llama7b-step-only: every projection its own launch (no in-place grouping of q|k|v, gate|up)")
     ap.add_argument("--llama7b-decode-only", action="store_true",
                     help="run only the greedy decode of the random-init 4-bit LLaMA-7B through transformers' generate")
+    ap.add_argument("--mlp-one-launch-only", action="store_true",
+                    help="run only the headline step through the one-launch MLP kernel (short run for profiling)")
     ap.add_argument("--dequant-only", action="store_true",
                     help="run only the dense dequantization of a 4096x11008 layer (short run for profiling)")
     ap.add_argument("--mid-rows-only", action="store_true",
@@ -620,6 +622,10 @@ def main():
         r = bench_llama7b_lora_train_step(max(args.steps, 2), grouped=not args.ungrouped)
         print(json.dumps({"workload": "config4_llama7b_lora_train_step_b4_s256", "grouped": not args.ungrouped,
                           **{k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()}}))
+        return
+    if args.mlp_one_launch_only:
+        r = bench_mlp_decode_one_launch(1, max(args.steps, 5))
+        print(json.dumps({"workload": "mlp_decode_M1_one_launch_per_layer", **{k: (round(v, 4) if isinstance(v, float) else v) for k, v in r.items()}}))
         return
     if args.dequant_only:
         r = bench_dequant(4096, 11008, False, max(args.steps, 5))
