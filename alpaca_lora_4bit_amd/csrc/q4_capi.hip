@@ -77,7 +77,7 @@ int check_layer(const void* qweight, const void* qzeros, const void* scales, con
 }
 }  // namespace
 
-extern "C" int q4_abi_version(void) { return 13; }
+extern "C" int q4_abi_version(void) { return 14; }
 
 extern "C" const char* q4_error_string(int code) {
     switch (code) {
@@ -101,6 +101,18 @@ extern "C" int q4_dequant_f16(const int32_t* qweight, const int32_t* qzeros, con
     if (misaligned(out)) return Q4_ERR_MISALIGNED;
     if (!g_idx && groupsize % 8 != 0) return Q4_ERR_BAD_SHAPE;
     return q4_launch_dequant(qweight, qzeros, scales, g_idx, groupsize, out, K, N, (hipStream_t)stream);
+}
+
+extern "C" int q4_launch_dequant_f32(const int32_t*, const int32_t*, const float*, const int32_t*, int, float*, int, int, hipStream_t);
+
+extern "C" int q4_dequant_f32(const int32_t* qweight, const int32_t* qzeros, const float* scales,
+                              const int32_t* g_idx, int groupsize, float* out, int K, int N, int G, void* stream) {
+    int rc = check_layer(qweight, qzeros, scales, g_idx, groupsize, K, N, G);
+    if (rc != Q4_OK) return rc;
+    if (!out) return Q4_ERR_NULL_POINTER;
+    if (misaligned(out)) return Q4_ERR_MISALIGNED;
+    if (!g_idx && groupsize % 8 != 0) return Q4_ERR_BAD_SHAPE;
+    return q4_launch_dequant_f32(qweight, qzeros, scales, g_idx, groupsize, out, K, N, (hipStream_t)stream);
 }
 
 extern "C" {

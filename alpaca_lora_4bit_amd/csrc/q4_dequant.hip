@@ -54,6 +54,53 @@ __global__ __launch_bounds__(256) void dequant_kernel(
     }
 }
 
+// fp32 flavour: scales fp32 [G, N], out fp32 [K, N]  (the float instantiation of the reference's template,
+// src/alpaca_lora_4bit/quant_cuda/quant_cuda_kernel.cu:1126-1152, which _matmul4bit_v2_recons reaches when a model's
+// scales were converted to float, matmul_utils_4bit.py:121-122).  zero = rn32(s * (z + 1)) and
+// W = fma(s, q, -zero): one rounding for the product and the difference together, which is what the reference's build
+// (nvcc defaults, setup.py passes no flags, so a * b - c contracts) computes; the separately rounded form differs from
+// it by at most one unit in the last place.  Same thread mapping as dequant_kernel; HBM-bound on the 4*K*N B it writes.
+__global__ __launch_bounds__(256) void dequant_f32_kernel(
+    const uint32_t* __restrict__ qweight, const uint32_t* __restrict__ qzeros,
+    const float* __restrict__ scales, const int32_t* __restrict__ g_idx, int groupsize,
+    float* __restrict__ out, int K, int N) {
+    const int ncol8 = N >> 3;
+    const long tid = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long total = (long)(K >> 3) * ncol8;
+    if (tid >= total) return;
+    const int kw = (int)(tid / ncol8);
+    const int nb = (int)(tid - (long)kw * ncol8);
+    const int n0 = nb << 3;
+
+    const uint4_t* wp = reinterpret_cast<const uint4_t*>(qweight + (size_t)kw * N + n0);
+    const uint4_t wa = wp[0], wb = wp[1];
+    const uint32_t w[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+
+    int gprev = -1;
+    float s[8], zero[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int k = (kw << 3) + e;
+        const int g = g_idx ? g_idx[k] : k / groupsize;
+        if (g != gprev) {
+            gprev = g;
+            const float4_t sa = *reinterpret_cast<const float4_t*>(scales + (size_t)g * N + n0);
+            const float4_t sb = *reinterpret_cast<const float4_t*>(scales + (size_t)g * N + n0 + 4);
+            const uint32_t zw = qzeros[(size_t)g * ncol8 + nb];
+            s[0] = sa.x; s[1] = sa.y; s[2] = sa.z; s[3] = sa.w;
+            s[4] = sb.x; s[5] = sb.y; s[6] = sb.z; s[7] = sb.w;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) zero[c] = s[c] * (float)(((zw >> (4 * c)) & 0xFu) + 1u);
+        }
+        float o[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) o[c] = __builtin_fmaf(s[c], (float)((w[c] >> (4 * e)) & 0xFu), -zero[c]);
+        float* dst = out + (size_t)k * N + n0;
+        __builtin_nontemporal_store(float4_t{o[0], o[1], o[2], o[3]}, reinterpret_cast<float4_t*>(dst));
+        __builtin_nontemporal_store(float4_t{o[4], o[5], o[6], o[7]}, reinterpret_cast<float4_t*>(dst + 4));
+    }
+}
+
 // Row permutation of the packed weights: out row p holds the codes of input row perm[p].
 // Used once per act-order layer to sort the rows by quantization group, after which the layer
 // runs through the sequential-group kernels with x gathered through the same permutation.
@@ -180,6 +227,16 @@ __global__ __launch_bounds__(256) void dequant2_kernel(const uint32_t* __restric
 }
 
 }  // namespace q4
+
+extern "C" int q4_launch_dequant_f32(const int32_t* qweight, const int32_t* qzeros, const float* scales,
+                                     const int32_t* g_idx, int groupsize, float* out, int K, int N,
+                                     hipStream_t stream) {
+    const long total = (long)(K / 8) * (N / 8);
+    hipLaunchKernelGGL(q4::dequant_f32_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
+                       reinterpret_cast<const uint32_t*>(qweight), reinterpret_cast<const uint32_t*>(qzeros),
+                       scales, g_idx, groupsize, out, K, N);
+    return hipGetLastError() == hipSuccess ? 0 : -4;
+}
 
 extern "C" int q4_launch_dequant_v1(const int32_t* qweight, const void* scales, const void* zeros, void* out,
                                     int K, int N, hipStream_t stream) {

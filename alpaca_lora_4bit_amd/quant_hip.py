@@ -368,6 +368,34 @@ def dequant(qweight, qzeros, scales, g_idx=None, groupsize=None, out=None):
     return out
 
 
+def dequant_f32(qweight, qzeros, scales, g_idx=None, groupsize=None, out=None):
+    """W fp32 [K, N] from fp32 scales: the float instantiation of vecquant4recons_v2
+    (quant_cuda_kernel.cu:1126-1152 through the dispatch at :1173-1181).  zero = rn32(s * (z + 1)),
+    W = fma(s, q, -zero), the contraction the reference's default build applies."""
+    _require(scales.dtype == torch.float32, "scales must be float32 [G, N]")
+    _require(qweight.is_cuda and qweight.dtype == torch.int32 and qweight.dim() == 2, "qweight must be int32 [K/8, N] on the GPU")
+    dev = qweight.device
+    K, N = qweight.shape[0] * 8, qweight.shape[1]
+    _require(scales.dim() == 2 and scales.shape[1] == N, "scales must be float32 [G, N]")
+    G = scales.shape[0]
+    _require(qzeros.dtype == torch.int32 and tuple(qzeros.shape) == (G, N // 8), "qzeros must be int32 [G, N/8]")
+    for t in (qweight, qzeros, scales):
+        _require(t.is_contiguous() and t.device == dev, "quantized tensors must be contiguous and on one device")
+    if g_idx is not None:
+        _require(g_idx.dtype == torch.int32 and g_idx.shape == (K,) and g_idx.is_contiguous() and g_idx.device == dev,
+                 "g_idx must be a contiguous int32 [K] tensor on the same device")
+    gp, gs = _gidx_arg(g_idx, groupsize, G, need_multiple=8)
+    if out is None:
+        out = torch.empty((K, N), dtype=torch.float32, device=dev)
+    _require(out.dtype == torch.float32 and tuple(out.shape) == (K, N) and out.is_contiguous() and out.device == dev,
+             "out must be a contiguous float32 [K, N] tensor on the same device")
+    with _device_ctx(dev):
+        rc = _lib.lib().q4_dequant_f32(qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), gp, gs,
+                                       out.data_ptr(), K, N, G, _stream(dev))
+    _lib.check(rc, "q4_dequant_f32")
+    return out
+
+
 def dequant_v1(qweight, scales, zeros, out=None):
     """W fp16 [K, N] of a v1 layer (per-column fp16 scale and zero), bit-exact with vecquant4recons_v1
     (quant_cuda_kernel.cu:1076-1097)."""
@@ -918,10 +946,18 @@ def vecquant2recons_v2(mat, res, scales, zeros, g_idx):
 
 def vecquant4recons_v2(mat, res, scales, zeros, g_idx):
     """quant_cuda.vecquant4recons_v2(mat, res, scales, zeros, g_idx) -> None; res[K,N] = W.
-    (quant_cuda.cpp:143-148).  fp16 `res` is written in place; other dtypes via one cast."""
+    (quant_cuda.cpp:143-148).  fp16 scales: fp16 `res` is written in place, other dtypes via one cast.
+    fp32 scales: the float kernel, `res` float32."""
     K = mat.shape[0] * 8
     gs = _infer_groupsize(K, scales.shape[0])
-    if res.dtype == torch.float16 and res.is_contiguous():
+    if scales.dtype == torch.float32:
+        # the reference dispatches on scales.type() (quant_cuda_kernel.cu:1173) and reads `res` as that type
+        _require(res.dtype == torch.float32, "res must be float32 when scales are float32")
+        if res.is_contiguous():
+            dequant_f32(mat, zeros, scales, g_idx, gs, out=res)
+        else:
+            res.copy_(dequant_f32(mat, zeros, scales, g_idx, gs))
+    elif res.dtype == torch.float16 and res.is_contiguous():
         dequant(mat, zeros, _scales_half(scales), g_idx, gs, out=res)
     else:
         res.copy_(dequant(mat, zeros, _scales_half(scales), g_idx, gs))

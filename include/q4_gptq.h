@@ -54,6 +54,17 @@ Q4_API int q4_dequant_f16(const int32_t *qweight, const int32_t *qzeros, const v
                    const int32_t *g_idx, int groupsize, void *out,
                    int K, int N, int G, void *stream);
 
+/* Dense dequantization in float: scales fp32 [G, N], out fp32 [K, N].
+ * Replaces the float instantiation of the same operator (AT_DISPATCH on scales.type(),
+ * quant_cuda/quant_cuda_kernel.cu:1173-1181; reached from matmul_utils_4bit.py:121-122 when a
+ * model's scales were converted to float).  zero = rn32(s * (z + 1)), W = fma(s, q, -zero): the
+ * product and the difference round once together, as in the reference's build (nvcc contracts
+ * a * b - c by default and setup.py sets no flag); rounding them separately moves a value by at
+ * most one unit in the last place.  Same shape rules as q4_dequant_f16. */
+Q4_API int q4_dequant_f32(const int32_t *qweight, const int32_t *qzeros, const float *scales,
+                   const int32_t *g_idx, int groupsize, float *out,
+                   int K, int N, int G, void *stream);
+
 /* Dense dequantization of the older "v1" layout: one fp16 scale and one fp16 zero per column
  * (scales, zeros: [N]),  W[k,n] = rn16( rn16(s[n]*q) - zero[n] ).
  * Replaces quant_cuda.vecquant4recons_v1 (quant_cuda/quant_cuda.cpp:131-135, kernel quant_cuda_kernel.cu:1076-1097). */

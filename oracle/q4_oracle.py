@@ -23,6 +23,9 @@ Parity status of each function (what pins it is in tests/test_oracle_*.py):
   dequant_v1 / dequant2_v2                  pinned  (exact Fraction arithmetic with the independent
                                                      round-to-nearest-even of tests/golden/make_fixtures.py,
                                                      pure-Python index loops for the 2-bit packing)
+  dequant_v2_f32                            pinned  (exact Fraction arithmetic with a round-to-binary32 of its own,
+                                                     tests/golden/q4_golden_f32.npz: scalar table over all (q, z),
+                                                     an act-order layer, and cases where fused != separate)
   peft 0.6 LoraLayer internals              parity unpinned (peft is not importable here; only the
                                                      arithmetic in models.py:58-66 is restated)
 """
@@ -167,6 +170,27 @@ def dequant2_v2(qweight, qzeros, scales, g_idx) -> np.ndarray:
     s_rows = scales[g]
     zero = s_rows * (z + 1).astype(np.float16)[g]
     return s_rows * q - zero
+
+
+def dequant_v2_f32(qweight, qzeros, scales, g_idx, fused=True) -> np.ndarray:
+    """Dense fp32 W [K, N] as VecQuant4ReconsV2Kernel<float> produces it (fp32 scales; the dispatch on
+    scales.type() at quant_cuda_kernel.cu:1173-1181 instantiates the template of :1126-1152 for float).
+
+    zero = rn32(s * (z + 1)); result = s * q - zero.  nvcc contracts a * b - c into one fma by default and the
+    reference's setup.py passes no flag, so the built kernel rounds once: rn32(s*q - zero) (fused=True).  float64
+    holds s*q (24 + 4 bits) and its difference with a float32 of nearby exponent exactly, so one cast to float32
+    is that single rounding.  fused=False rounds the product first (what the source says without contraction).
+    """
+    scales = np.asarray(scales)
+    assert scales.dtype == np.float32
+    q = unpack_qweight(qweight)
+    z = unpack_qzeros(qzeros)
+    g = np.asarray(g_idx).astype(np.int64)
+    s_rows = scales[g]
+    zero = s_rows * (z.astype(np.int32) + 1).astype(np.float32)[g]            # rn32(s*(z+1))
+    if fused:
+        return (s_rows.astype(np.float64) * q.astype(np.float64) - zero.astype(np.float64)).astype(np.float32)
+    return s_rows * q.astype(np.float32) - zero
 
 
 def dequant_v2_single_rounding(qweight, qzeros, scales, g_idx) -> np.ndarray:

@@ -9,7 +9,10 @@ pure-Python loops that follow the reference kernel's thread-index arithmetic
 rational arithmetic (fractions.Fraction) and a hand-written round-to-nearest-even to binary16.
 Matmul expectations are exact rational sums of the dequantized values, stored as float64.
 
-Run:  python tests/golden/make_fixtures.py     (about half a minute)
+tests/golden/q4_golden_f32.npz holds the same for the kernel's float instantiation (fp32 scales, fp32 result), from
+exact rational arithmetic and a round-to-nearest-even to binary32 written for it.
+
+Run:  python tests/golden/make_fixtures.py     (about a minute; --f32-only writes the float file alone)
 """
 import os
 import struct
@@ -126,6 +129,99 @@ def make_case(seed, K, N, groupsize, act_order, M):
                 codes=codes.astype(np.uint8), zcodes=zc.astype(np.uint8))
 
 
+# ------------------------------------------------------------------------------------------------ float flavour
+def float_bits_to_fraction(u: int) -> Fraction:
+    sign = -1 if (u >> 31) & 1 else 1
+    exp = (u >> 23) & 0xFF
+    man = u & 0x7FFFFF
+    assert exp != 255, "fixtures use finite values only"
+    if exp == 0:
+        return sign * Fraction(man, 1 << 149)
+    return sign * Fraction((1 << 23) + man, 1 << 23) * (Fraction(2) ** (exp - 127))
+
+
+def rn32(v: Fraction) -> int:
+    """Exact rational -> nearest binary32 bit pattern, ties to even (written on its own, not derived from rn16:
+    it scales to an integer significand first and rounds the integer)."""
+    if v == 0:
+        return 0
+    sign = 0x80000000 if v < 0 else 0
+    a = abs(v)
+    e = max(a.numerator.bit_length() - a.denominator.bit_length() - 2, -126)      # a lower bound of floor(log2 a)
+    while Fraction(2) ** (e + 1) <= a:
+        e += 1                                        # subnormals keep the exponent -126
+    ulp = Fraction(2) ** (e - 23)
+    n, twice_rem = divmod(2 * (a / ulp), 2)
+    n = int(n)
+    if twice_rem > 1 or (twice_rem == 1 and n % 2 == 1):
+        n += 1
+    if n == (1 << 24):
+        n, e = 1 << 23, e + 1
+    assert e <= 127, "fixtures stay finite"
+    if n < (1 << 23):
+        return sign | n
+    return sign | ((e + 127) << 23) | (n - (1 << 23))
+
+
+def recons_v2_float(s: Fraction, q: int, z: int):
+    """(fused, separate) bit patterns of VecQuant4ReconsV2Kernel<float> for one element
+    (quant_cuda_kernel.cu:1146-1151): zero = rn32(s * (z + 1)); result = s * q - zero, which nvcc's default
+    contraction evaluates as one fma (one rounding); the separately rounded form is kept beside it."""
+    zero = float_bits_to_fraction(rn32(s * (z + 1)))
+    fused = rn32(s * q - zero)
+    separate = rn32(float_bits_to_fraction(rn32(s * q)) - zero)
+    return fused, separate
+
+
+def main_f32():
+    out = {}
+    rng = np.random.default_rng(11)
+    # scale bit patterns: typical GPTQ magnitudes with all 23 fraction bits in play, plus edge patterns
+    typical = rng.uniform(0.003, 0.03, size=160).astype(np.float32).view(np.uint32)
+    wide = (rng.integers(100, 140, size=60).astype(np.uint32) << 23) | rng.integers(0, 1 << 23, size=60).astype(np.uint32)
+    edge = np.array([0x00000001, 0x007FFFFF, 0x00800000, 0x3F800000, 0x3FFFFFFF, 0x80000001, 0xBF800000, 0x7B7FFFFF],
+                    dtype=np.uint32)
+    sb = np.concatenate([typical, wide, edge]).astype(np.uint32)
+    fused = np.zeros((sb.size, 16, 16), dtype=np.uint32)
+    separate = np.zeros_like(fused)
+    for i, u in enumerate(sb):
+        S = float_bits_to_fraction(int(u))
+        for q in range(16):
+            for z in range(16):
+                fused[i, q, z], separate[i, q, z] = recons_v2_float(S, q, z)
+    out["scalar_scale_bits"] = sb
+    out["scalar_fused"] = fused
+    out["scalar_separate"] = separate
+    # one small act-order layer, thread-index arithmetic as in recons_v2_reference_loops
+    K, N, groupsize = 128, 64, 32
+    G = K // groupsize
+    codes = rng.integers(0, 16, size=(K, N))
+    zc = rng.integers(0, 16, size=(G, N))
+    qweight = np.zeros((K // 8, N), dtype=np.int64)
+    for k in range(K):
+        qweight[k // 8] |= codes[k] << (4 * (k % 8))
+    qzeros = np.zeros((G, N // 8), dtype=np.int64)
+    for n in range(N):
+        qzeros[:, n // 8] |= zc[:, n] << (4 * (n % 8))
+    qweight = qweight.astype(np.uint32).view(np.int32)
+    qzeros = qzeros.astype(np.uint32).view(np.int32)
+    scales = rng.uniform(0.003, 0.03, size=(G, N)).astype(np.float32)
+    perm = rng.permutation(K)
+    g_idx = np.empty(K, dtype=np.int32)
+    g_idx[perm] = (np.arange(K) // groupsize).astype(np.int32)
+    W = np.zeros((K, N), dtype=np.uint32)
+    sbits = scales.view(np.uint32)
+    for n_rows in range(K):
+        for n_cols in range(N):
+            z_rows = int(g_idx[n_rows])
+            z = (as_unsigned(int(qzeros[z_rows, n_cols // 8])) >> ((n_cols % 8) * 4)) & 0xF
+            q = (as_unsigned(int(qweight[n_rows // 8, n_cols])) >> (n_rows % 8 * 4)) & 0xF
+            W[n_rows, n_cols] = recons_v2_float(float_bits_to_fraction(int(sbits[z_rows, n_cols])), q, z)[0]
+    out.update(layer_qweight=qweight, layer_qzeros=qzeros, layer_scales=scales, layer_g_idx=g_idx, layer_W_bits=W)
+    np.savez_compressed(os.path.join(HERE, "q4_golden_f32.npz"), **out)
+    print("wrote", os.path.join(HERE, "q4_golden_f32.npz"))
+
+
 def main():
     out = {}
     for name, kw in (("seq", dict(seed=101, K=256, N=128, groupsize=128, act_order=False, M=2)),
@@ -151,4 +247,7 @@ def main():
 
 
 if __name__ == "__main__":
-    main()
+    import sys
+    if "--f32-only" not in sys.argv:
+        main()
+    main_f32()

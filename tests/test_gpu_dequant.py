@@ -115,3 +115,45 @@ def test_dequant_rejects_bad_arguments(oracle):
     bad[3] = 99
     with pytest.raises(ValueError):
         quant_hip.dequant(t["qweight"], t["qzeros"], t["scales"], bad, 128)
+
+
+# --------------------------------------------------------------------------- float flavour (fp32 scales, fp32 W)
+def test_dequant_f32_matches_committed_golden_fixture():
+    """Bit-exact with tests/golden/q4_golden_f32.npz (exact rational arithmetic, made without oracle/): the table of
+    every (q, z) for 228 scale patterns through the kernel, and an act-order layer."""
+    import os
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    from test_oracle import _scalar_layer_f32, _scalar_table_of
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "q4_golden_f32.npz"))
+    qw, qz, scales, g_idx, n = _scalar_layer_f32()
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    for gi in (dev(g_idx), None):                                # gathered and sequential group lookup
+        W = quant_hip.dequant_f32(dev(qw), dev(qz), dev(scales), gi, 32)
+        got = _scalar_table_of(W.cpu().numpy().view(np.uint32), n)
+        exp = gold["scalar_fused"]
+        assert ((got == exp) | (((got | exp) & 0x7FFFFFFF) == 0)).all()
+    W = quant_hip.dequant_f32(dev(gold["layer_qweight"]), dev(gold["layer_qzeros"]), dev(gold["layer_scales"]),
+                              dev(gold["layer_g_idx"]), 32)
+    assert np.array_equal(W.cpu().numpy().view(np.uint32), gold["layer_W_bits"])
+
+
+@pytest.mark.parametrize("K,N,gs,act", [(256, 128, 128, True), (4096, 4096, 128, False), (5120, 13824, 128, True),
+                                        (11008, 4096, 128, False)])
+def test_dequant_f32_bit_exact_with_oracle_and_through_the_quant_cuda_name(oracle, K, N, gs, act):
+    import torch
+    from alpaca_lora_4bit_amd import quant_hip
+    layer = oracle.make_layer(K, N, gs, act_order=act, seed=K + N + 1)
+    rng = np.random.default_rng(K)
+    scales = (layer["scales"].astype(np.float32) * rng.uniform(0.9, 1.1, size=layer["scales"].shape)).astype(np.float32)
+    ref = oracle.dequant_v2_f32(layer["qweight"], layer["qzeros"], scales, layer["g_idx"])
+    t = to_cuda_layer(layer)
+    res = torch.zeros((K, N), dtype=torch.float32, device="cuda")
+    assert quant_hip.vecquant4recons_v2(t["qweight"], res, torch.from_numpy(scales).cuda(), t["qzeros"], t["g_idx"]) is None
+    assert np.array_equal(res.cpu().numpy().view(np.uint32), ref.view(np.uint32))
+    with pytest.raises(ValueError):                              # the reference reads `res` as the scales' type
+        quant_hip.vecquant4recons_v2(t["qweight"], res.half(), torch.from_numpy(scales).cuda(), t["qzeros"], t["g_idx"])
+    # fp32 copies of fp16 scales still give the fp16 kernel's values when `res` is fp16-typed storage of the module path
+    W16 = quant_hip.dequant(t["qweight"], t["qzeros"], t["scales"], t["g_idx"], gs)
+    W32 = quant_hip.dequant_f32(t["qweight"], t["qzeros"], t["scales"].float(), t["g_idx"], gs)
+    assert (W32 - W16.float()).abs().max().item() <= 2.0 ** -9 * W16.abs().max().item()     # fp16 roundings only

@@ -349,3 +349,76 @@ def test_dequant2_against_loops_and_exact_arithmetic(oracle):
             prod = gen.half_bits_to_fraction(gen.rn16(s * q))
             expect = gen.rn16(prod - zero)
             assert int(wb[k, n]) == expect or (expect & 0x7FFF) == 0 and (int(wb[k, n]) & 0x7FFF) == 0
+
+
+# --------------------------------------------------------------------------- float flavour of the dense dequant
+GOLD32 = np.load(os.path.join(os.path.dirname(__file__), "golden", "q4_golden_f32.npz"))
+
+
+def _scalar_layer_f32():
+    """A layer holding every (scale, q, z) of the golden table: column n = scale index, row k has q = k % 16,
+    groups of 32 rows (the smallest the library takes), one group per zero code."""
+    sb = GOLD32["scalar_scale_bits"]
+    n_pad = (sb.size + 63) // 64 * 64
+    s = np.zeros(n_pad, dtype=np.uint32)
+    s[:sb.size] = sb
+    codes = np.tile(np.arange(16, dtype=np.uint8)[:, None], (32, n_pad))              # [512, N]: row k -> q = k % 16
+    zc = np.tile(np.arange(16, dtype=np.uint8)[:, None], (1, n_pad))                  # group g -> z = g
+    scales = np.tile(s.view(np.float32)[None, :], (16, 1))
+    g_idx = (np.arange(512) // 32).astype(np.int32)
+    return o.pack_qweight(codes), o.pack_qzeros(zc), scales, g_idx, sb.size
+
+
+def _scalar_table_of(W_bits, n):
+    """[512, N] patterns of that layer -> [scale, q, z]."""
+    return W_bits.reshape(16, 2, 16, -1)[:, 0, :, :n].transpose(2, 1, 0)
+
+
+def test_generator_round_to_binary32_on_known_values():
+    """The fixture generator's own rounding against values whose binary32 pattern is known by hand."""
+    from fractions import Fraction
+    gen = _load_generator()
+    assert gen.rn32(Fraction(1)) == 0x3F800000 and gen.rn32(Fraction(-2)) == 0xC0000000
+    assert gen.rn32(Fraction(1, 10)) == 0x3DCCCCCD and gen.rn32(Fraction(1, 3)) == 0x3EAAAAAB
+    assert gen.rn32(1 + Fraction(1, 1 << 24)) == 0x3F800000            # tie -> even (down)
+    assert gen.rn32(1 + Fraction(3, 1 << 24)) == 0x3F800002            # tie -> even (up)
+    assert gen.rn32(2 - Fraction(1, 1 << 25)) == 0x40000000            # carries into the next binade
+    assert gen.rn32(Fraction(1, 1 << 149)) == 0x00000001 and gen.rn32(Fraction(1, 1 << 150)) == 0   # subnormal, tie to 0
+    assert gen.rn32(Fraction(3, 1 << 150)) == 0x00000002
+    for u in (0x00000001, 0x007FFFFF, 0x00800000, 0x3FFFFFFF, 0xBF800001, 0x7B7FFFFF):
+        assert gen.rn32(gen.float_bits_to_fraction(u)) == u
+
+
+def test_dequant_f32_matches_golden_scalar_table_both_forms():
+    qw, qz, scales, g_idx, n = _scalar_layer_f32()
+    for fused, key in ((True, "scalar_fused"), (False, "scalar_separate")):
+        got = _scalar_table_of(o.dequant_v2_f32(qw, qz, scales, g_idx, fused=fused).view(np.uint32), n)
+        exp = GOLD32[key]
+        same = (got == exp) | (((got | exp) & 0x7FFFFFFF) == 0)                            # +0 == -0
+        assert same.all(), key
+
+
+def test_dequant_f32_fused_and_separate_forms_are_distinguishable_and_within_one_ulp():
+    f, s = GOLD32["scalar_fused"].astype(np.int64), GOLD32["scalar_separate"].astype(np.int64)
+    typical = slice(0, 160)                                     # the GPTQ-magnitude scales
+    differ = f[typical] != s[typical]
+    assert 0.01 < differ.mean() < 0.6                           # a merged or split rounding in the oracle would show
+    both_nonzero = ((f & 0x7FFFFFFF) != 0) & ((s & 0x7FFFFFFF) != 0) & ((f >> 31) == (s >> 31))
+    # rounding the product first moves it by half a unit of ITS last place, which the difference can magnify
+    # when it cancels; for same-sign neighbours the patterns are adjacent or a few steps apart
+    gap = np.abs(f - s)[both_nonzero]
+    assert np.median(gap[gap > 0]) == 1
+
+
+def test_dequant_f32_matches_golden_act_order_layer():
+    W = o.dequant_v2_f32(GOLD32["layer_qweight"], GOLD32["layer_qzeros"], GOLD32["layer_scales"], GOLD32["layer_g_idx"])
+    assert np.array_equal(W.view(np.uint32), GOLD32["layer_W_bits"])
+    # with fp16-representable scales and the fp16 flavour's operands the float result rounds to ... the exact value:
+    # s*q - s*(z+1) needs at most 11 + 5 bits, so both float forms are exact there and equal (q - z - 1) * s
+    lay = o.make_layer(128, 64, 32, act_order=True, seed=3)
+    s32 = lay["scales"].astype(np.float32)
+    for fused in (True, False):
+        W32 = o.dequant_v2_f32(lay["qweight"], lay["qzeros"], s32, lay["g_idx"], fused=fused)
+        q = o.unpack_qweight(lay["qweight"]).astype(np.float64)
+        z = o.unpack_qzeros(lay["qzeros"]).astype(np.float64)[lay["g_idx"]]
+        assert np.array_equal(W32.astype(np.float64), (q - z - 1.0) * s32[lay["g_idx"]].astype(np.float64))
