@@ -950,6 +950,8 @@ def vecquant4recons_v2(mat, res, scales, zeros, g_idx):
     fp32 scales: the float kernel, `res` float32."""
     K = mat.shape[0] * 8
     gs = _infer_groupsize(K, scales.shape[0])
+    _require(scales.dtype in (torch.float16, torch.float32),
+             "scales must be float16 or float32 (the reference's float64 instantiation has no counterpart here)")
     if scales.dtype == torch.float32:
         # the reference dispatches on scales.type() (quant_cuda_kernel.cu:1173) and reads `res` as that type
         _require(res.dtype == torch.float32, "res must be float32 when scales are float32")
