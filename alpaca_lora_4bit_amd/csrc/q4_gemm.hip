@@ -728,10 +728,9 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce_cols_kernel(const floa
 constexpr size_t kSzTableMax = 48 * 1024;     // dynamic LDS left beside the 108 KB of tile buffers
 template <int BM, int WGM, bool FWD, bool GIDX>
 static void launch_tiles(const GemmArgs& a, dim3 grid, hipStream_t stream) {
-    static const int env_sz = getenv("Q4_GEMM_SZ") ? atoi(getenv("Q4_GEMM_SZ")) : 1;
     const dim3 block(128 * WGM);
     if constexpr (!GIDX) {
-        if (env_sz && a.groupsize % 128 == 0) {
+        if (a.groupsize % 128 == 0) {
             if constexpr (FWD) {
                 const int nsteps = a.K / BK, S = (int)grid.z;
                 if (nsteps % (2 * S) == 0 && ((a.phase_step & 0xff) % 2) == 0) {
@@ -809,13 +808,14 @@ static hipError_t launch_gemm_cfg(const GemmPlan& p, const GemmArgs& a, int nout
     }
 }
 
+// What TileMap is told: row tile r starts its reduction loop kPhaseStep * r steps later; tiles are ordered in groups
+// of kRowTilesPerGroup row tiles (measured optimum over the benchmark shapes).
+constexpr int kPhaseStep = 2, kRowTilesPerGroup = 2;
+
 // Launch plan shared by q4_launch_gemm and q4_gemm_plan_workspace.  Few output tiles (small M) leave most CUs
 // idle while each tile walks the whole reduction: the reduction is then split over gridDim.z workgroups that
 // write fp32 partial tiles, about 1.5 workgroups per CU in total.
 static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
-    static const int env_cfg = getenv("Q4_GEMM_CFG") ? atoi(getenv("Q4_GEMM_CFG")) : -1;
-    static const int env_splits = getenv("Q4_GEMM_SPLITS") ? atoi(getenv("Q4_GEMM_SPLITS")) : 0;
-    static const int env_tail = getenv("Q4_GEMM_TAIL") ? atoi(getenv("Q4_GEMM_TAIL")) : 1;
     GemmPlan p;
     p.tail_cols = 0; p.tail_splits = 1;
     const int nsteps = red / BK;
@@ -831,8 +831,7 @@ static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
     // fill theirs better: 3072 x (4096 -> 11008) has 516 wide tiles = 3 rounds for 2.02 rounds of work and stays
     // with the narrow ones (270 against 294 us), 4096 rows have 688 (313 against 356 us).
     const long twide = (nout % 256 == 0) ? (long)(nout / 256) * ((M + 255) / 256) : 0;
-    static const int env_wide = getenv("Q4_GEMM_WIDE") ? atoi(getenv("Q4_GEMM_WIDE")) : 1;
-    if (env_wide && env_cfg < 0 && env_splits == 0 && twide >= 144 &&
+    if (twide >= 144 &&
         (twide <= 256 || 5 * twide >= 4 * 256 * ((twide + 255) / 256))) {
         p.cfg = 3; p.splits = 1;
         return p;
@@ -843,7 +842,7 @@ static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
         // remainder run as a second launch with the reduction split so that it takes a fraction of a round.
         const int nr = (M + 255) / 256;
         const long rem = t256 % 256;
-        if (env_tail && t256 > 256 && rem > 0) {
+        if (t256 > 256 && rem > 0) {
             const int tcols = (int)((rem + nr - 1) / nr);
             const long tt = (long)tcols * nr;
             int ts = tt <= 128 ? (int)(256 / tt) : 1;
@@ -868,23 +867,6 @@ static GemmPlan plan_gemm(int M, int red, int nout, size_t workspace_bytes) {
             if (splits > nsteps / 4) splits = nsteps / 4;      // at least four steps per workgroup
         }
     }
-    if (env_cfg == 3 && nout % 256 == 0 && M > 256) {          // experiments: wide tiles wherever they apply
-        p.cfg = 3; p.splits = 1; p.tail_cols = 0; p.tail_splits = 1;
-        return p;
-    }
-    if (env_cfg >= 0 && env_cfg != 3 && env_cfg != p.cfg) {    // experiments: forced tile shape, splits as before
-        p.cfg = env_cfg;
-        p.tail_cols = 0;
-        const int bm = p.cfg == 0 ? 128 : 256;
-        const long tiles = (long)(nout / BN) * ((M + bm - 1) / bm);
-        splits = 1;
-        if (tiles < 192) {
-            splits = (int)((384 + tiles - 1) / tiles);
-            if (splits > 8) splits = 8;
-            if (splits > nsteps / 4) splits = nsteps / 4;
-        }
-    }
-    if (env_splits > 0) { splits = env_splits > nsteps ? nsteps : env_splits; p.tail_cols = 0; }
     while (splits > 1 && (size_t)splits * (size_t)M * (size_t)nout * sizeof(float) > workspace_bytes) --splits;
     p.splits = splits < 1 ? 1 : splits;
     return p;
@@ -937,10 +919,7 @@ extern "C" int q4_launch_gemm(int fwd, const void* act, const int32_t* qweight, 
     a.R = (la && lb) ? R : 0;
     a.out = reinterpret_cast<half_t*>(out);
     a.M = M; a.K = K; a.N = N; a.G = G;
-    static const int env_phase = getenv("Q4_GEMM_PHASE") ? atoi(getenv("Q4_GEMM_PHASE")) : 2;
-    a.phase_step = env_phase < 0 ? 0 : env_phase;
-    static const int env_order = getenv("Q4_GEMM_ORDER") ? atoi(getenv("Q4_GEMM_ORDER")) : 2;   // row tiles per group
-    if (env_order > 0) a.phase_step |= (env_order > 64 ? 64 : env_order) << 8;
+    a.phase_step = kPhaseStep | (kRowTilesPerGroup << 8);
     const int nout = fwd ? N : K;
     const bool gidx = g_idx != nullptr;
     // some hundred rows of an output that one round of workgroups covers, no adapter: whole-reduction streaming kernels
@@ -1043,8 +1022,6 @@ extern "C" int q4_launch_gemm_group(int fwd, int n, const void* const* act, cons
     if (p.cfg < 0) return -2;
     const size_t need = fwd ? 0 : (size_t)n * p.zs * (size_t)M * (size_t)K * sizeof(float);
     if (need > 0 && (!workspace || workspace_bytes < need)) return -3;
-    static const int env_phase = getenv("Q4_GEMM_PHASE") ? atoi(getenv("Q4_GEMM_PHASE")) : 2;
-    static const int env_order = getenv("Q4_GEMM_ORDER") ? atoi(getenv("Q4_GEMM_ORDER")) : 2;
     GemmGroupArgs g;
     const int tile_w = p.cfg == 3 ? 256 : BN;
     int tiles = 0;
@@ -1067,7 +1044,7 @@ extern "C" int q4_launch_gemm_group(int fwd, int n, const void* const* act, cons
         a.lb_scale = (a.R ? lb_scale[j] : 0.f) * a.drop.scale;
         a.out = reinterpret_cast<half_t*>(fwd ? out[j] : out[0]);
         a.M = M; a.K = K; a.N = N[j]; a.G = (K + groupsize - 1) / groupsize;
-        a.phase_step = (env_phase < 0 ? 0 : env_phase) | (env_order > 0 ? (env_order > 64 ? 64 : env_order) << 8 : 0);
+        a.phase_step = kPhaseStep | (kRowTilesPerGroup << 8);
         a.part = reinterpret_cast<float*>(workspace);
         a.col_tile0 = 0;
         a.part_cols = fwd ? N[j] : K;

@@ -1165,8 +1165,7 @@ extern "C" int q4_launch_splitk_reduce(const float* part, void* out, long total,
 
 // Shapes the skinny kernel takes: 17..64 rows, sequential groups that are multiples of 128 rows.
 extern "C" int q4_skinny_applicable(int M, int K, int N, int groupsize, int has_gidx) {
-    static const int max_rows = getenv("Q4_SKINNY_MAX_ROWS") ? atoi(getenv("Q4_SKINNY_MAX_ROWS")) : 64;
-    return M > 16 && M <= max_rows && M <= 64 && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 64 == 0;
+    return M > 16 && M <= 64 && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 64 == 0;
 }
 
 static int skinny_splits(int K) {
@@ -1197,9 +1196,8 @@ extern "C" int q4_launch_skinny(const void* x, const int32_t* qweight, const int
     const int strips = N / kColsPerWave;
     // neighbouring strips per workgroup: enough for the whole grid to be resident at once (two workgroups
     // per compute unit fit with two row blocks, one with more), at most 4
-    static const int force_l = getenv("Q4_SKINNY_STRIPS") ? atoi(getenv("Q4_SKINNY_STRIPS")) : 0;
     const int slots = M <= 32 ? 512 : 256;
-    int L = force_l > 0 ? force_l : (strips * S + slots - 1) / slots;
+    int L = (strips * S + slots - 1) / slots;
     L = L < 1 ? 1 : (L > 4 ? 4 : L);
     a.strips_per_wg = L;
     const dim3 grid((strips + L - 1) / L, S), block(512);    // wavefronts past the end of K read zeros
@@ -1219,16 +1217,13 @@ extern "C" int q4_launch_skinny(const void* x, const int32_t* qweight, const int
 // against 22-34 us; 4096 -> 11008 never fits one round).
 // Row blocks of 32, 48 or 64 rows: the smallest that fits (more workgroups, fewer idle CUs).
 static int stream_fwd_row_blocks(int M, int N) {
-    static const int force_rb = getenv("Q4_STREAM_FWD_RB") ? atoi(getenv("Q4_STREAM_FWD_RB")) : 0;
-    if (force_rb >= 2 && force_rb <= 4) return force_rb;
     const int strips = N / q4::kColsPerWave;
     for (int rb = 2; rb <= 4; ++rb)
         if (strips * ((M + 16 * rb - 1) / (16 * rb)) <= 256) return rb;
     return 0;
 }
 extern "C" int q4_stream_fwd_applicable(int M, int K, int N, int groupsize, int has_gidx) {
-    static const int max_rows = getenv("Q4_STREAM_FWD_MAX_ROWS") ? atoi(getenv("Q4_STREAM_FWD_MAX_ROWS")) : 512;
-    if (!(M > 16 && M <= max_rows && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 64 == 0))
+    if (!(M > 16 && M <= 512 && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 64 == 0))
         return 0;
     // up to 64 rows there is one row block, i.e. one workgroup per strip: worth it from 128 strips on, where it beats
     // the kernel with the split reduction and the second launch (4096 -> 11008 at 17..64 rows: 9.7-14.7 against
@@ -1271,16 +1266,13 @@ extern "C" int q4_launch_stream_fwd(const void* x, const int32_t* qweight, const
 // 15.5-17.3 against 15.5-24.8 us, 2048 x 2048 10 against 12-18.5 us, 4096 outputs over 1024 columns 7.6 against 11-18 us,
 // 11008 outputs over 4096 columns (up to 96 rows) 18-21 against 28-32 us.
 static int stream_dx_row_blocks(int M, int K) {
-    static const int force_rb = getenv("Q4_STREAM_DX_RB") ? atoi(getenv("Q4_STREAM_DX_RB")) : 0;
-    if (force_rb >= 2 && force_rb <= 3) return force_rb;
     const int blocks = K / 128;
     for (int rb = 2; rb <= 3; ++rb)
         if (blocks * ((M + 16 * rb - 1) / (16 * rb)) <= 256) return rb;
     return 0;
 }
 extern "C" int q4_stream_dx_applicable(int M, int K, int N, int groupsize, int has_gidx) {
-    static const int max_rows = getenv("Q4_STREAM_DX_MAX_ROWS") ? atoi(getenv("Q4_STREAM_DX_MAX_ROWS")) : 512;
-    if (!(M > 48 && M <= max_rows && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 128 == 0))
+    if (!(M > 48 && M <= 512 && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 && N % 128 == 0))
         return 0;
     if (K > 65536 || N > 65536 || (long)K * N > (1L << 28)) return 0;      // 32-bit byte offsets, far offset included
     // a workgroup walks the whole reduction alone: with a long reduction and few output blocks (4096 outputs over 11008
@@ -1311,8 +1303,7 @@ extern "C" int q4_launch_stream_dx(const void* dy, const int32_t* qweight, const
 
 // Shapes the streaming grad-input kernel takes: 17..48 rows, sequential groups that are multiples of 128 rows.
 extern "C" int q4_skinny_dx_applicable(int M, int K, int N, int groupsize, int has_gidx) {
-    static const int max_rows = getenv("Q4_SKINNY_DX_MAX_ROWS") ? atoi(getenv("Q4_SKINNY_DX_MAX_ROWS")) : 48;
-    return M > 16 && M <= max_rows && M <= 48 && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 &&
+    return M > 16 && M <= 48 && !has_gidx && groupsize > 0 && groupsize % 128 == 0 && K % 128 == 0 &&
            N % 128 == 0;
 }
 
@@ -1340,9 +1331,8 @@ extern "C" int q4_launch_skinny_dx(const void* dy, const int32_t* qweight, const
     a.M = M; a.K = K; a.N = N; a.G = G;
     const int S = skinny_dx_splits(N);
     const int blocks = K / 128;
-    static const int force_l = getenv("Q4_SKINNY_DX_STRIPS") ? atoi(getenv("Q4_SKINNY_DX_STRIPS")) : 0;
     const int slots = 256;                        // one workgroup per compute unit (register budget)
-    int L = force_l > 0 ? force_l : (blocks * S + slots - 1) / slots;
+    int L = (blocks * S + slots - 1) / slots;
     L = L < 1 ? 1 : (L > 4 ? 4 : L);
     a.strips_per_wg = L;
     const dim3 grid((blocks + L - 1) / L, S), block(512);     // wavefronts past the end of N read zeros

@@ -309,14 +309,11 @@ inline bool group_compatible(int gs32, int nstep, int* gsteps) {
 // per workgroup reduce through LDS, the rest of K goes to gridDim.y (measured best on MI355X:
 // ~700 workgroups of 512 threads for the LLaMA-7B MLP shapes).
 inline GemvPlan plan_gemv(int K, int N, int groupsize, bool seq, int max_nstep) {
-    static const int env_nstep = getenv("Q4_GEMV_NSTEP") ? atoi(getenv("Q4_GEMV_NSTEP")) : 0;
-    static const int env_waves = getenv("Q4_GEMV_WAVES") ? atoi(getenv("Q4_GEMV_WAVES")) : 0;
     const int steps = K / 32;
     const int gs32 = seq ? groupsize / 32 : 1;
     GemvPlan p{1, 0, 1, 1};
     for (int ns : {16, 8, 4, 2, 1}) {
         if (ns > max_nstep || steps % ns) continue;
-        if (env_nstep && ns > env_nstep) continue;
         int gst = 0;
         if (seq && !group_compatible(gs32, ns, &gst)) continue;
         p.nstep = ns; p.gsteps = gst;
@@ -327,7 +324,6 @@ inline GemvPlan plan_gemv(int K, int N, int groupsize, bool seq, int max_nstep) 
     (void)strips;
     int waves = 8;
     const int max_waves = (!seq || p.nstep >= 16) ? 8 : 16;      // register budget of the kernels' launch bounds
-    if (env_waves) waves = env_waves;
     if (waves > chunks) waves = chunks;
     if (waves > max_waves) waves = max_waves;
     if (waves < 1) waves = 1;

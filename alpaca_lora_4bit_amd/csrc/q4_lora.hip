@@ -434,10 +434,9 @@ __global__ __launch_bounds__(256) void dropout_keep_kernel(uint8_t* __restrict__
 // tiles cost 2 * splits * R * C * 4 bytes of traffic); rows per workgroup a multiple of 128 (4 wavefronts x 32 rows).
 struct GradPlan { int col_blocks, splits, rows_per_wg; };
 inline GradPlan plan_grad(int M, int C) {
-    static const int env_wgs = getenv("Q4_LORA_GRAD_WGS") ? atoi(getenv("Q4_LORA_GRAD_WGS")) : 384;
     GradPlan g;
     g.col_blocks = (C + kG2Cols - 1) / kG2Cols;
-    int splits = (env_wgs + g.col_blocks - 1) / g.col_blocks;
+    int splits = (384 + g.col_blocks - 1) / g.col_blocks;
     if (splits > 64) splits = 64;
     if (splits < 1) splits = 1;
     const int unit = 32 * kG2Waves;
@@ -453,10 +452,8 @@ static void launch_down_kernel(const q4::half_t* ip, const void* w, int w_sr, in
                                int M, int C, int R, const q4::DropArgs& drop, hipStream_t stream) {
     // rows of `in` per workgroup: 16 fill the MFMA operand, but with few rows that leaves compute units idle and
     // the kernel is bound by the latency of its single burst of loads, so smaller blocks spread it out
-    static const int force_rows = getenv("Q4_LORA_DOWN_ROWS") ? atoi(getenv("Q4_LORA_DOWN_ROWS")) : 0;
     int rows = 16;
     while (rows > 4 && (M + rows - 1) / rows < 256) rows >>= 1;
-    if (force_rows == 4 || force_rows == 8 || force_rows == 16) rows = force_rows;
     hipLaunchKernelGGL((q4::lora_down_kernel<RB, WL, F32, RQ>), dim3((M + rows - 1) / rows), dim3(64 * q4::kDownWaves), 0,
                        stream, ip, w, w_sr, w_sc, op, M, C, R, rows, drop);
 }
